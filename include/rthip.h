@@ -1,0 +1,193 @@
+/*
+ * rthip.h -- kernel-level C ABI of the MI355X (gfx950) backend for the packed
+ * NF4 QLoRA linear path of riftco-transformer.
+ *
+ * This is the whole boundary between host code and the GPU: plain pointers and
+ * sizes, int status codes, no C++ types, no exceptions, no framework types.
+ * The C++ `hip` backend adapter (the counterpart of the reference's CPU, Metal,
+ * CUDA and TPU adapters) is the intended caller; Python reaches the same
+ * symbols through ctypes for tests and measurement.
+ *
+ * Conventions
+ *   - Every function returns an rthip_status; on failure a thread-local,
+ *     NUL-terminated message is available from rthip_last_error().
+ *   - All tensor pointers are DEVICE pointers unless named host_*.
+ *   - Tensors are contiguous row-major fp32; packed codes are bytes with the
+ *     even flat index in the low nibble (src/core/quantization/nf4.cpp:70-75).
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *     Compute entry points only enqueue work; the caller synchronises.  The
+ *     reference contract "an adapter finishes writing its output before
+ *     returning" (docs/BACKENDS_AND_PYTHON.md:168) is met by the adapter, which
+ *     calls rthip_stream_synchronize() after each launch.
+ *   - A packed weight is described by the same six values the reference's CUDA
+ *     launch passes to its kernels
+ *     (src/core/backend/nn/quantized_linear/cuda/operations.cu:76-81,196-211):
+ *       codes              uint8  [ceil(O*I/2)]
+ *       primary_scales     float  [blocks]   when encoding == RTHIP_NF4_SCALE_FLOAT32
+ *                          uint8  [blocks]   when encoding == RTHIP_NF4_SCALE_DOUBLE_QUANTIZED_UINT8
+ *       secondary_scales   float  [ceil(blocks / second_level_block)] (DQ only, else NULL)
+ *       encoding, second_level_block, offset
+ *     with blocks = ceil(O*I / block_size) counted over the FLATTENED weight
+ *     (src/core/backend/nn/quantized_linear/reference/operations.cpp:44).
+ */
+#ifndef RTHIP_H
+#define RTHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RTHIP_ABI_VERSION_MAJOR 1u
+#define RTHIP_ABI_VERSION_MINOR 0u
+
+typedef int32_t rthip_status;
+
+enum {
+    RTHIP_OK = 0,
+    /* bad pointer/size/enum: the adapter maps it to std::invalid_argument */
+    RTHIP_INVALID_ARGUMENT = 1,
+    /* no usable gfx950 device: maps to "hip execution backend is unavailable" */
+    RTHIP_UNAVAILABLE = 2,
+    /* device allocation failed: maps to std::bad_alloc, as
+     * src/core/backend/adapters/cuda/adapter.cu:25-32 does for CUDA */
+    RTHIP_OUT_OF_MEMORY = 3,
+    /* any other HIP runtime failure: maps to std::runtime_error */
+    RTHIP_RUNTIME_ERROR = 4,
+    /* a forced algorithm cannot handle the given shape */
+    RTHIP_UNSUPPORTED = 5
+};
+
+/* Nf4ScaleEncoding, src/core/backend/nn/quantized_linear/storage.hpp:13-16 */
+enum {
+    RTHIP_NF4_SCALE_FLOAT32 = 0,
+    RTHIP_NF4_SCALE_DOUBLE_QUANTIZED_UINT8 = 1
+};
+
+/* Kernel families.  AUTO picks by shape; the others exist so that tests can
+ * pin one family and compare it with another on the same inputs. */
+enum {
+    RTHIP_NF4_ALGORITHM_AUTO = 0,
+    /* one thread per output, per-element decode, any shape or block size */
+    RTHIP_NF4_ALGORITHM_GENERIC = 1,
+    /* wavefront-reduced streaming GEMV for small row counts (HBM-bound) */
+    RTHIP_NF4_ALGORITHM_GEMV = 2,
+    /* LDS-tiled fp32 MFMA GEMM with dequantisation fused into the tile load */
+    RTHIP_NF4_ALGORITHM_MFMA = 3
+};
+
+/* ---- library / device ------------------------------------------------- */
+
+/* (major << 16) | minor of this ABI. */
+uint32_t rthip_abi_version(void);
+
+/* Thread-local message of the last failing call on this thread ("" if none). */
+const char* rthip_last_error(void);
+
+/* Number of usable gfx950 devices.  Returns RTHIP_UNAVAILABLE (and *count = 0)
+ * when there is no driver or no device -- the adapter's is_available().
+ * Replaces the role of cudaGetDeviceCount in
+ * src/core/backend/adapters/cuda/adapter.cu:40-51. */
+rthip_status rthip_device_count(int32_t* count);
+
+/* Human-readable device description, e.g. "AMD Instinct MI355X (gfx950), 256 CUs". */
+rthip_status rthip_device_description(char* buffer, size_t capacity);
+
+/* ---- memory ----------------------------------------------------------- */
+
+/* Device (HBM) allocation; *pointer is 256-byte aligned.  bytes == 0 yields
+ * NULL.  Counterpart of the allocations in
+ * src/core/backend/nn/quantized_linear/cuda/storage.cu:26-43. */
+rthip_status rthip_malloc(void** pointer, size_t bytes);
+rthip_status rthip_free(void* pointer);
+
+/* Synchronous copies between host and device memory. */
+rthip_status rthip_copy_to_device(void* device, const void* host, size_t bytes);
+rthip_status rthip_copy_to_host(void* host, const void* device, size_t bytes);
+
+/* Fills count floats (make_storage(element_count, fill_value),
+ * src/core/backend/adapter.hpp:37-40).  Enqueued on `stream`. */
+rthip_status rthip_fill_f32(float* device, float value, uint64_t count,
+                            void* stream);
+
+rthip_status rthip_stream_synchronize(void* stream);
+
+/* ---- the hot path ----------------------------------------------------- */
+
+/*
+ * y[r,o] = sum_i x[r,i] * deq(W)[o,i]  (+ bias[o] when bias_or_null != NULL)
+ *
+ * Replaces BackendAdapter::quantized_linear_forward
+ * (src/core/backend/nn/quantized_linear/capability.hpp:36-42), whose CPU form
+ * is reference_quantized_linear_forward
+ * (src/core/backend/nn/quantized_linear/reference/operations.cpp:49-81).
+ * x is [rows, input_width], y is [rows, output_width] and is overwritten.
+ * The optional bias fuses the broadcast add the reference performs afterwards
+ * (src/nn/linear.cpp:165-168).  x/y must not overlap each other or the weight.
+ */
+rthip_status rthip_nf4_linear_forward(
+    const float* x, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, const float* bias_or_null,
+    float* y, uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream);
+
+/*
+ * dx[r,i] = sum_o dy[r,o] * deq(W)[o,i]
+ *
+ * Replaces BackendAdapter::quantized_linear_input_backward
+ * (src/core/backend/nn/quantized_linear/capability.hpp:44-50; CPU form
+ * src/core/backend/nn/quantized_linear/reference/operations.cpp:83-115).
+ * dy is [rows, output_width], dx is [rows, input_width] and is overwritten.
+ */
+rthip_status rthip_nf4_linear_input_backward(
+    const float* dy, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, float* dx, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream);
+
+/* The same two operations with the kernel family pinned (tests, measurement).
+ * RTHIP_UNSUPPORTED when `algorithm` cannot handle the shape. */
+rthip_status rthip_nf4_linear_forward_with(
+    int32_t algorithm, const float* x, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset,
+    const float* bias_or_null, float* y, uint64_t rows, uint64_t input_width,
+    uint64_t output_width, uint64_t block_size, void* stream);
+
+rthip_status rthip_nf4_linear_input_backward_with(
+    int32_t algorithm, const float* dy, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset, float* dx,
+    uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream);
+
+/* Which family AUTO selects for a shape: direction 0 = forward, 1 = input
+ * backward.  Pure host computation; needs no device. */
+rthip_status rthip_nf4_select_algorithm(
+    int32_t direction, uint64_t rows, uint64_t input_width,
+    uint64_t output_width, uint64_t block_size, int32_t* algorithm);
+
+/*
+ * out[j] = scale(j / block_size) * codebook[code(j)] for j < element_count.
+ *
+ * Device form of QuantizedWeight::dequantize
+ * (src/core/quantization/quantized_weight.cpp:453-467).  The linear kernels
+ * never call it (they never materialise an fp32 weight); it exists so that the
+ * bit-exactness of nibble unpack, codebook lookup and scale decode on the GPU
+ * can be checked directly, and for the explicit dequantize() API.
+ */
+rthip_status rthip_nf4_dequantize(
+    const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, float* out,
+    uint64_t element_count, uint64_t block_size, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* RTHIP_H */

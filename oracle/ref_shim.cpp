@@ -1,0 +1,222 @@
+// TEST INFRASTRUCTURE ONLY.  A C-callable wrapper around the *compiled
+// reference itself*: this file is linked against objects built from the
+// reference's own sources where they lie under /root/reference (recipe:
+// oracle/Makefile, target _ref) and exposes its CPU backend through plain C
+// signatures, so that the restatement in nf4_oracle.c can be diffed against
+// it and so that it can serve as the timed CPU baseline.  Nothing of the
+// reference is copied here; only its public and internal headers are included.
+//
+// Entry points used (reference file:line):
+//   QuantizedWeight::quantize_nf4 / quantize_nf4_double_quantized /
+//   from_packed_nf4 / copy_payload_to_host / dequantize
+//       include/riftco_transformer/core/quantized_weight.hpp:69-111
+//   dispatch_quantized_linear_forward / _input_backward
+//       src/core/backend/nn/quantized_linear/dispatch.hpp:19-27
+
+#include "core/backend/nn/quantized_linear/dispatch.hpp"
+#include "riftco_transformer/core/backend.hpp"
+#include "riftco_transformer/core/quantized_weight.hpp"
+#include "riftco_transformer/core/tensor.hpp"
+
+#include <algorithm>
+#include <cstddef>
+#include <cstdint>
+#include <cstring>
+#include <exception>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+namespace {
+
+using riftco_transformer::ExecutionBackend;
+using riftco_transformer::Nf4DoubleQuantizedScales;
+using riftco_transformer::Nf4Payload;
+using riftco_transformer::QuantizedWeight;
+using riftco_transformer::Tensor;
+namespace backend = riftco_transformer::backend_detail;
+
+thread_local std::string g_last_error;
+
+// 0 ok, 1 invalid_argument, 2 logic_error, 3 overflow_error, 4 runtime_error,
+// 255 anything else -- the first three match nf4_oracle.h's status codes.
+template <typename Function> int guarded(Function&& function) noexcept {
+    try {
+        function();
+        g_last_error.clear();
+        return 0;
+    } catch (const std::invalid_argument& error) {
+        g_last_error = error.what();
+        return 1;
+    } catch (const std::overflow_error& error) {
+        g_last_error = error.what();
+        return 3;
+    } catch (const std::logic_error& error) {
+        g_last_error = error.what();
+        return 2;
+    } catch (const std::runtime_error& error) {
+        g_last_error = error.what();
+        return 4;
+    } catch (const std::exception& error) {
+        g_last_error = error.what();
+        return 255;
+    }
+}
+
+Nf4Payload make_payload(
+    const std::uint8_t* codes, std::size_t code_bytes, int encoding,
+    const float* fp32_scales, std::size_t fp32_count,
+    const std::uint8_t* scale_codes, std::size_t scale_code_count,
+    const float* second_level, std::size_t second_level_count,
+    std::size_t second_level_block, float offset
+) {
+    Nf4Payload payload;
+    payload.packed_codes.assign(codes, codes + code_bytes);
+    if (fp32_count != 0) {
+        payload.block_scales.assign(fp32_scales, fp32_scales + fp32_count);
+    }
+    if (encoding == 1) {
+        Nf4DoubleQuantizedScales nested;
+        nested.scale_codes.assign(scale_codes, scale_codes + scale_code_count);
+        nested.second_level_scales.assign(
+            second_level, second_level + second_level_count);
+        nested.scale_block_size = second_level_block;
+        nested.offset = offset;
+        payload.double_quantized_scales = std::move(nested);
+    }
+    return payload;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* nf4ref_last_error(void) { return g_last_error.c_str(); }
+
+// Quantizes values[output_width*input_width] with the reference quantizer.
+// encoding 0: fills fp32_scales.  encoding 1: fills scale_codes, second_level
+// and *offset.  Buffers are sized by the caller from the block counts.
+int nf4ref_quantize(
+    const float* values, std::size_t output_width, std::size_t input_width,
+    std::size_t block_size, int encoding, std::size_t second_level_block,
+    std::uint8_t* codes, float* fp32_scales, std::uint8_t* scale_codes,
+    float* second_level, float* offset
+) {
+    return guarded([&] {
+        const std::size_t count = output_width * input_width;
+        Tensor source(
+            {output_width, input_width},
+            std::vector<float>(values, values + count),
+            ExecutionBackend::Cpu
+        );
+        const QuantizedWeight weight = encoding == 1
+            ? QuantizedWeight::quantize_nf4_double_quantized(
+                  source, block_size, second_level_block)
+            : QuantizedWeight::quantize_nf4(source, block_size);
+        const Nf4Payload payload = weight.copy_payload_to_host();
+        std::copy(payload.packed_codes.begin(), payload.packed_codes.end(),
+                  codes);
+        if (encoding == 1) {
+            const auto& nested = *payload.double_quantized_scales;
+            std::copy(nested.scale_codes.begin(), nested.scale_codes.end(),
+                      scale_codes);
+            std::copy(nested.second_level_scales.begin(),
+                      nested.second_level_scales.end(), second_level);
+            *offset = nested.offset;
+        } else {
+            std::copy(payload.block_scales.begin(), payload.block_scales.end(),
+                      fp32_scales);
+        }
+    });
+}
+
+// Validates and imports a packed payload exactly as a checkpoint load would
+// (QuantizedWeight::from_packed_nf4), then runs mode 0 = dequantize,
+// 1 = forward, 2 = input backward on the reference CPU backend.
+int nf4ref_run(
+    int mode, const float* activations, float* result, std::size_t rows,
+    std::size_t input_width, std::size_t output_width, std::size_t block_size,
+    const std::uint8_t* codes, std::size_t code_bytes, int encoding,
+    const float* fp32_scales, std::size_t fp32_count,
+    const std::uint8_t* scale_codes, std::size_t scale_code_count,
+    const float* second_level, std::size_t second_level_count,
+    std::size_t second_level_block, float offset
+) {
+    return guarded([&] {
+        const QuantizedWeight weight = QuantizedWeight::from_packed_nf4(
+            {output_width, input_width}, block_size,
+            make_payload(codes, code_bytes, encoding, fp32_scales, fp32_count,
+                         scale_codes, scale_code_count, second_level,
+                         second_level_count, second_level_block, offset),
+            ExecutionBackend::Cpu
+        );
+        if (mode == 0) {
+            const Tensor dense = weight.dequantize();
+            const auto data = dense.data();
+            std::copy(data.begin(), data.end(), result);
+            return;
+        }
+        const std::size_t in_width = mode == 1 ? input_width : output_width;
+        const std::size_t out_width = mode == 1 ? output_width : input_width;
+        const Tensor source(
+            {rows, in_width},
+            std::vector<float>(activations, activations + rows * in_width),
+            ExecutionBackend::Cpu
+        );
+        Tensor target({rows, out_width}, ExecutionBackend::Cpu);
+        const backend::QuantizedLinearDimensions dimensions{
+            rows, input_width, output_width, block_size};
+        if (mode == 1) {
+            backend::dispatch_quantized_linear_forward(
+                ExecutionBackend::Cpu,
+                {backend::tensor_storage(source),
+                 backend::quantized_weight_storage(weight),
+                 backend::tensor_storage(target), dimensions});
+        } else {
+            backend::dispatch_quantized_linear_input_backward(
+                ExecutionBackend::Cpu,
+                {backend::tensor_storage(source),
+                 backend::quantized_weight_storage(weight),
+                 backend::tensor_storage(target), dimensions});
+        }
+        const auto data = target.data();
+        std::copy(data.begin(), data.end(), result);
+    });
+}
+
+// Byte accounting of QuantizedWeight::memory_usage() for a quantized tensor of
+// element_count zeros-free synthetic values is not needed; this reports the
+// nine counters for an imported payload instead (out[9], order of the struct
+// in include/riftco_transformer/core/quantized_weight.hpp:52-65).
+int nf4ref_memory_usage(
+    std::size_t input_width, std::size_t output_width, std::size_t block_size,
+    const std::uint8_t* codes, std::size_t code_bytes, int encoding,
+    const float* fp32_scales, std::size_t fp32_count,
+    const std::uint8_t* scale_codes, std::size_t scale_code_count,
+    const float* second_level, std::size_t second_level_count,
+    std::size_t second_level_block, float offset, std::size_t* out
+) {
+    return guarded([&] {
+        const QuantizedWeight weight = QuantizedWeight::from_packed_nf4(
+            {output_width, input_width}, block_size,
+            make_payload(codes, code_bytes, encoding, fp32_scales, fp32_count,
+                         scale_codes, scale_code_count, second_level,
+                         second_level_count, second_level_block, offset),
+            ExecutionBackend::Cpu
+        );
+        const auto usage = weight.memory_usage();
+        out[0] = usage.packed_code_bytes;
+        out[1] = usage.scale_bytes;
+        out[2] = usage.logical_payload_bytes;
+        out[3] = usage.resident_payload_bytes;
+        out[4] = usage.fp32_equivalent_bytes;
+        out[5] = usage.fp32_scale_bytes;
+        out[6] = usage.scale_code_bytes;
+        out[7] = usage.second_level_scale_bytes;
+        out[8] = usage.scale_offset_bytes;
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,255 @@
+"""ctypes binding of the kernel C ABI (include/rthip.h -> lib/librthip.so).
+
+This is plumbing for tests and measurement: PyTorch supplies device memory and
+the current HIP stream, every computation goes through the C ABI.  There is no
+fallback of any kind -- a missing library, a missing symbol or a failing call
+raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import dataclasses
+import os
+from typing import Optional
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIBRARY_PATH = os.path.join(_HERE, "lib", "librthip.so")
+
+OK = 0
+INVALID_ARGUMENT = 1
+UNAVAILABLE = 2
+OUT_OF_MEMORY = 3
+RUNTIME_ERROR = 4
+UNSUPPORTED = 5
+
+SCALE_FLOAT32 = 0
+SCALE_DOUBLE_QUANTIZED_UINT8 = 1
+
+ALGORITHM_AUTO = 0
+ALGORITHM_GENERIC = 1
+ALGORITHM_GEMV = 2
+ALGORITHM_MFMA = 3
+ALGORITHM_NAMES = {0: "auto", 1: "generic", 2: "gemv", 3: "mfma"}
+
+FORWARD = 0
+INPUT_BACKWARD = 1
+
+
+class RthipError(RuntimeError):
+    """A C-ABI call returned a non-zero status."""
+
+    def __init__(self, status: int, message: str):
+        super().__init__(f"rthip status {status}: {message}")
+        self.status = status
+        self.message = message
+
+
+class InvalidArgument(RthipError, ValueError):
+    pass
+
+
+class Unavailable(RthipError):
+    pass
+
+
+class Unsupported(RthipError):
+    pass
+
+
+_ERRORS = {
+    INVALID_ARGUMENT: InvalidArgument,
+    UNAVAILABLE: Unavailable,
+    OUT_OF_MEMORY: RthipError,
+    RUNTIME_ERROR: RthipError,
+    UNSUPPORTED: Unsupported,
+}
+
+_u64 = ctypes.c_uint64
+_i32 = ctypes.c_int32
+_f32 = ctypes.c_float
+_ptr = ctypes.c_void_p
+_size = ctypes.c_size_t
+
+# The six values that describe a packed weight, in ABI order.
+_WEIGHT = [_ptr, _ptr, _ptr, _i32, _u64, _f32]
+
+_PROTOTYPES = {
+    "rthip_abi_version": (ctypes.c_uint32, []),
+    "rthip_last_error": (ctypes.c_char_p, []),
+    "rthip_device_count": (_i32, [ctypes.POINTER(_i32)]),
+    "rthip_device_description": (_i32, [ctypes.c_char_p, _size]),
+    "rthip_malloc": (_i32, [ctypes.POINTER(_ptr), _size]),
+    "rthip_free": (_i32, [_ptr]),
+    "rthip_copy_to_device": (_i32, [_ptr, _ptr, _size]),
+    "rthip_copy_to_host": (_i32, [_ptr, _ptr, _size]),
+    "rthip_fill_f32": (_i32, [_ptr, _f32, _u64, _ptr]),
+    "rthip_stream_synchronize": (_i32, [_ptr]),
+    "rthip_nf4_linear_forward": (
+        _i32, [_ptr] + _WEIGHT + [_ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
+    "rthip_nf4_linear_input_backward": (
+        _i32, [_ptr] + _WEIGHT + [_ptr, _u64, _u64, _u64, _u64, _ptr]),
+    "rthip_nf4_linear_forward_with": (
+        _i32,
+        [_i32, _ptr] + _WEIGHT + [_ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
+    "rthip_nf4_linear_input_backward_with": (
+        _i32, [_i32, _ptr] + _WEIGHT + [_ptr, _u64, _u64, _u64, _u64, _ptr]),
+    "rthip_nf4_select_algorithm": (
+        _i32, [_i32, _u64, _u64, _u64, _u64, ctypes.POINTER(_i32)]),
+    "rthip_nf4_dequantize": (_i32, _WEIGHT + [_ptr, _u64, _u64, _ptr]),
+}
+
+EXPORTED_SYMBOLS = tuple(_PROTOTYPES)
+
+
+@dataclasses.dataclass
+class DeviceWeight:
+    """A packed NF4 weight whose payload lives in device memory.
+
+    The tensors are kept alive here; the ABI only ever sees their addresses.
+    """
+
+    output_width: int
+    input_width: int
+    block_size: int
+    encoding: int
+    codes: object                      # torch.uint8 [ceil(O*I/2)]
+    primary_scales: object             # torch.float32 or torch.uint8 [blocks]
+    secondary_scales: Optional[object]  # torch.float32 [groups] or None
+    second_level_block: int = 0
+    offset: float = 0.0
+
+    def abi_arguments(self):
+        secondary = (None if self.secondary_scales is None
+                     else self.secondary_scales.data_ptr())
+        return [self.codes.data_ptr(), self.primary_scales.data_ptr(),
+                secondary, self.encoding, self.second_level_block,
+                self.offset]
+
+    @property
+    def payload_bytes(self) -> int:
+        total = self.codes.numel() + (
+            self.primary_scales.numel() * self.primary_scales.element_size())
+        if self.secondary_scales is not None:
+            total += self.secondary_scales.numel() * 4 + 4
+        return total
+
+
+class Library:
+    """librthip.so with typed entry points."""
+
+    def __init__(self, path: str = LIBRARY_PATH):
+        if not os.path.exists(path):
+            raise FileNotFoundError(
+                f"{path} is missing: build it with "
+                "`make -C riftco-transformer_amd` (or __graft_entry__.build())")
+        self.path = path
+        self._lib = ctypes.CDLL(path)
+        for name, (restype, argtypes) in _PROTOTYPES.items():
+            function = getattr(self._lib, name)  # AttributeError if absent
+            function.restype = restype
+            function.argtypes = argtypes
+
+    # -- helpers ---------------------------------------------------------
+    def last_error(self) -> str:
+        return (self._lib.rthip_last_error() or b"").decode()
+
+    def _check(self, status: int) -> None:
+        if status != OK:
+            raise _ERRORS.get(status, RthipError)(status, self.last_error())
+
+    # -- library / device -------------------------------------------------
+    def abi_version(self):
+        value = self._lib.rthip_abi_version()
+        return value >> 16, value & 0xFFFF
+
+    def device_count(self) -> int:
+        count = _i32(0)
+        self._check(self._lib.rthip_device_count(ctypes.byref(count)))
+        return count.value
+
+    def is_available(self) -> bool:
+        count = _i32(0)
+        return self._lib.rthip_device_count(ctypes.byref(count)) == OK
+
+    def device_description(self) -> str:
+        buffer = ctypes.create_string_buffer(256)
+        self._check(self._lib.rthip_device_description(buffer, 256))
+        return buffer.value.decode()
+
+    # -- memory ------------------------------------------------------------
+    def malloc(self, size: int) -> int:
+        pointer = _ptr()
+        self._check(self._lib.rthip_malloc(ctypes.byref(pointer), size))
+        return pointer.value or 0
+
+    def free(self, pointer: int) -> None:
+        self._check(self._lib.rthip_free(pointer))
+
+    def copy_to_device(self, device: int, host: int, size: int) -> None:
+        self._check(self._lib.rthip_copy_to_device(device, host, size))
+
+    def copy_to_host(self, host: int, device: int, size: int) -> None:
+        self._check(self._lib.rthip_copy_to_host(host, device, size))
+
+    def fill_f32(self, device: int, value: float, count: int,
+                 stream: int = 0) -> None:
+        self._check(self._lib.rthip_fill_f32(device, value, count, stream))
+
+    def synchronize(self, stream: int = 0) -> None:
+        self._check(self._lib.rthip_stream_synchronize(stream))
+
+    # -- the hot path --------------------------------------------------------
+    def select_algorithm(self, direction: int, rows: int, input_width: int,
+                         output_width: int, block_size: int) -> int:
+        algorithm = _i32(0)
+        self._check(self._lib.rthip_nf4_select_algorithm(
+            direction, rows, input_width, output_width, block_size,
+            ctypes.byref(algorithm)))
+        return algorithm.value
+
+    def linear_forward(self, x_ptr: int, weight: DeviceWeight,
+                       bias_ptr: Optional[int], y_ptr: int, rows: int,
+                       stream: int = 0,
+                       algorithm: Optional[int] = None) -> None:
+        tail = [bias_ptr, y_ptr, rows, weight.input_width,
+                weight.output_width, weight.block_size, stream]
+        if algorithm is None:
+            status = self._lib.rthip_nf4_linear_forward(
+                x_ptr, *weight.abi_arguments(), *tail)
+        else:
+            status = self._lib.rthip_nf4_linear_forward_with(
+                algorithm, x_ptr, *weight.abi_arguments(), *tail)
+        self._check(status)
+
+    def linear_input_backward(self, dy_ptr: int, weight: DeviceWeight,
+                              dx_ptr: int, rows: int, stream: int = 0,
+                              algorithm: Optional[int] = None) -> None:
+        tail = [dx_ptr, rows, weight.input_width, weight.output_width,
+                weight.block_size, stream]
+        if algorithm is None:
+            status = self._lib.rthip_nf4_linear_input_backward(
+                dy_ptr, *weight.abi_arguments(), *tail)
+        else:
+            status = self._lib.rthip_nf4_linear_input_backward_with(
+                algorithm, dy_ptr, *weight.abi_arguments(), *tail)
+        self._check(status)
+
+    def dequantize(self, weight: DeviceWeight, out_ptr: int,
+                   element_count: Optional[int] = None,
+                   stream: int = 0) -> None:
+        if element_count is None:
+            element_count = weight.output_width * weight.input_width
+        self._check(self._lib.rthip_nf4_dequantize(
+            *weight.abi_arguments(), out_ptr, element_count,
+            weight.block_size, stream))
+
+
+_library: Optional[Library] = None
+
+
+def load_library() -> Library:
+    """The process-wide Library; raises if librthip.so is not built."""
+    global _library
+    if _library is None:
+        _library = Library()
+    return _library

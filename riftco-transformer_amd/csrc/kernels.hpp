@@ -1,0 +1,51 @@
+// Host-callable launchers of the packed NF4 linear kernels.  Each launcher
+// only enqueues work on `stream`; shape preconditions are checked by the
+// matching *_supports() predicate, which the C ABI consults before launching.
+#pragma once
+
+#include "nf4_decode.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace rthip {
+
+// One forward (activations = x, result = y) or input-backward
+// (activations = dy, result = dx) problem.  The weight is row-major
+// [output_width, input_width] in both directions.
+struct LinearProblem {
+    const float* activations;
+    Nf4WeightView weight;
+    const float* bias;  // forward only, may be null
+    float* result;
+    std::size_t rows;
+    std::size_t input_width;
+    std::size_t output_width;
+    unsigned block_shift;  // log2(block_size)
+};
+
+// nf4_generic.hip
+void launch_generic_forward(const LinearProblem& problem, hipStream_t stream);
+void launch_generic_input_backward(const LinearProblem& problem,
+                                   hipStream_t stream);
+void launch_dequantize(const Nf4WeightView& weight, float* out,
+                       std::size_t element_count, unsigned block_shift,
+                       hipStream_t stream);
+void launch_fill(float* out, float value, std::size_t count,
+                 hipStream_t stream);
+
+// nf4_gemv.hip -- forward only, small row counts.
+constexpr std::size_t kGemvMaxRows = 4;
+bool gemv_forward_supports(const LinearProblem& problem);
+void launch_gemv_forward(const LinearProblem& problem, hipStream_t stream);
+
+// nf4_mfma.hip
+bool mfma_forward_supports(const LinearProblem& problem);
+void launch_mfma_forward(const LinearProblem& problem, hipStream_t stream);
+bool mfma_input_backward_supports(const LinearProblem& problem);
+void launch_mfma_input_backward(const LinearProblem& problem,
+                                hipStream_t stream);
+
+}  // namespace rthip

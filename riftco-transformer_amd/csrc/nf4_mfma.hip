@@ -1,0 +1,359 @@
+// LDS-tiled fp32 MFMA GEMM with NF4 dequantisation fused into the tile load,
+// for prefill / training row counts.  Two products over the same packed
+// weight W [output_width, input_width]:
+//
+//   forward         y [M, O] = x  [M, I] * deq(W)^T     (contract over I)
+//   input backward  dx[M, I] = dy [M, O] * deq(W)       (contract over O)
+//
+// restating reference_quantized_linear_forward / _input_backward
+// (src/core/backend/nn/quantized_linear/reference/operations.cpp:49-115).
+// The fp32 weight never exists in HBM: packed nibbles and block scales are
+// read straight from global memory, decoded in registers
+// (codebook[code] * scale, one rounded multiply) and written to the LDS tile
+// the matrix cores read.
+//
+// Tiling.  A workgroup of four wavefronts computes a 128 x 128 output tile in
+// steps of 32 along the contraction; each wavefront owns a 64 x 64 quadrant as
+// 2 x 2 blocks of v_mfma_f32_32x32x2_f32.  Both LDS tiles are laid out
+// [row-or-column][contraction] with a padded stride of 36 floats, so that one
+// ds_read_b128 per lane fetches four consecutive contraction values; lanes
+// 0-31 take offsets 0..3 and lanes 32-63 offsets 4..7 of each group of eight,
+// which the four MFMAs of the group consume as (k, k+4) pairs -- any pairing is
+// valid because both operands use the same one.  Global loads for step t+1 are
+// issued before the MFMAs of step t.
+//
+// The two directions share everything except the weight-tile loader: forward
+// reads 128 weight rows x 32 contiguous columns, backward reads 32 weight rows
+// (the contraction) x 128 contiguous columns and transposes while writing LDS.
+
+#include "kernels.hpp"
+#include "nf4_decode.hpp"
+
+namespace rthip {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int kTileM = 128;       // output rows per workgroup
+constexpr int kTileN = 128;       // output columns per workgroup
+constexpr int kTileK = 32;        // contraction per step
+constexpr int kStride = 36;       // padded LDS row stride in floats
+constexpr int kChunk = 16;        // weights decoded per thread per step
+
+struct GemmShape {
+    unsigned rows;         // M
+    unsigned contraction;  // I (forward) or O (backward)
+    unsigned columns;      // O (forward) or I (backward)
+    unsigned input_width;  // I: the weight's row length
+};
+
+// Registers holding one step's global loads of a thread.
+struct Staged {
+    float4 a[4];
+    uint2 codes;
+    float scale;
+};
+
+__device__ __forceinline__ void load_activation_tile(
+    Staged& staged, const float* __restrict__ activations,
+    const GemmShape& shape, unsigned row0, unsigned k0
+) {
+    const unsigned thread = threadIdx.x;
+    const unsigned column = (thread % 8) * 4;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const unsigned row = row0 + thread / 8 + 32 * pass;
+        staged.a[pass] = row < shape.rows
+            ? *reinterpret_cast<const float4*>(
+                  activations +
+                  static_cast<std::size_t>(row) * shape.contraction + k0 +
+                  column)
+            : make_float4(0.0F, 0.0F, 0.0F, 0.0F);
+    }
+}
+
+__device__ __forceinline__ void store_activation_tile(
+    const Staged& staged, float* __restrict__ tile
+) {
+    const unsigned thread = threadIdx.x;
+    const unsigned column = (thread % 8) * 4;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const unsigned row = thread / 8 + 32 * pass;
+        *reinterpret_cast<float4*>(tile + row * kStride + column) =
+            staged.a[pass];
+    }
+}
+
+// Forward weight tile: output columns n0..n0+127 are weight rows; the step's
+// 32 contraction values are 16 contiguous code bytes of each row.  Thread t
+// decodes 16 weights of row t / 2.
+template <bool kDoubleQuantized>
+__device__ __forceinline__ void load_weight_tile_forward(
+    Staged& staged, const Nf4WeightView& weight, const GemmShape& shape,
+    unsigned n0, unsigned k0, unsigned block_shift
+) {
+    const unsigned thread = threadIdx.x;
+    const unsigned n = n0 + thread / 2;
+    if (n < shape.columns) {
+        const std::size_t flat =
+            static_cast<std::size_t>(n) * shape.input_width + k0 +
+            (thread % 2) * kChunk;
+        staged.codes =
+            *reinterpret_cast<const uint2*>(weight.codes + (flat >> 1));
+        staged.scale =
+            load_block_scale<kDoubleQuantized>(weight, flat >> block_shift);
+    } else {
+        staged.codes = make_uint2(0x77777777U, 0x77777777U);
+        staged.scale = 0.0F;
+    }
+}
+
+// Backward weight tile: the step's 32 contraction values are weight rows
+// c0..c0+31; output columns k0..k0+127 are contiguous within each row.
+// Thread t decodes 16 weights of row c0 + t % 32.
+template <bool kDoubleQuantized>
+__device__ __forceinline__ void load_weight_tile_backward(
+    Staged& staged, const Nf4WeightView& weight, const GemmShape& shape,
+    unsigned k0, unsigned c0, unsigned block_shift
+) {
+    const unsigned thread = threadIdx.x;
+    const unsigned column = k0 + (thread / 32) * kChunk;
+    if (column < shape.columns) {
+        const std::size_t flat =
+            static_cast<std::size_t>(c0 + thread % 32) * shape.input_width +
+            column;
+        staged.codes =
+            *reinterpret_cast<const uint2*>(weight.codes + (flat >> 1));
+        staged.scale =
+            load_block_scale<kDoubleQuantized>(weight, flat >> block_shift);
+    } else {
+        staged.codes = make_uint2(0x77777777U, 0x77777777U);
+        staged.scale = 0.0F;
+    }
+}
+
+__device__ __forceinline__ void decode_chunk(
+    const Staged& staged, const float* __restrict__ table, float (&out)[16]
+) {
+#pragma clang fp contract(off)
+    const unsigned words[2] = {staged.codes.x, staged.codes.y};
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+            out[8 * w + n] =
+                table[(words[w] >> (4 * n)) & 0xFU] * staged.scale;
+        }
+    }
+}
+
+template <bool kBackward>
+__device__ __forceinline__ void store_weight_tile(
+    const Staged& staged, const float* __restrict__ table,
+    float* __restrict__ tile
+) {
+    const unsigned thread = threadIdx.x;
+    float decoded[16];
+    decode_chunk(staged, table, decoded);
+    if constexpr (!kBackward) {
+        float* destination =
+            tile + (thread / 2) * kStride + (thread % 2) * kChunk;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            *reinterpret_cast<float4*>(destination + 4 * q) = make_float4(
+                decoded[4 * q], decoded[4 * q + 1], decoded[4 * q + 2],
+                decoded[4 * q + 3]);
+        }
+    } else {
+        // tile[column][contraction]: transpose while writing.
+        float* destination =
+            tile + ((thread / 32) * kChunk) * kStride + thread % 32;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            destination[i * kStride] = decoded[i];
+        }
+    }
+}
+
+template <bool kDoubleQuantized, bool kBackward>
+__global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
+    const float* __restrict__ activations, Nf4WeightView weight,
+    const float* __restrict__ bias, float* __restrict__ result,
+    GemmShape shape, unsigned block_shift
+) {
+    __shared__ __attribute__((aligned(16))) float a_tile[kTileM * kStride];
+    __shared__ __attribute__((aligned(16))) float b_tile[kTileN * kStride];
+    __shared__ float table[16];
+    load_codebook_to_lds(table);
+
+    const unsigned thread = threadIdx.x;
+    const unsigned lane = thread % 64;
+    const unsigned wave = thread / 64;
+    const unsigned wave_m = wave / 2;
+    const unsigned wave_n = wave % 2;
+    const unsigned row0 = blockIdx.y * kTileM;
+    const unsigned col0 = blockIdx.x * kTileN;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                acc[i][j][e] = 0.0F;
+            }
+        }
+    }
+
+    Staged staged;
+    load_activation_tile(staged, activations, shape, row0, 0);
+    if constexpr (!kBackward) {
+        load_weight_tile_forward<kDoubleQuantized>(staged, weight, shape,
+                                                   col0, 0, block_shift);
+    } else {
+        load_weight_tile_backward<kDoubleQuantized>(staged, weight, shape,
+                                                    col0, 0, block_shift);
+    }
+
+    const float* a_fragment =
+        a_tile + (wave_m * 64 + lane % 32) * kStride + 4 * (lane / 32);
+    const float* b_fragment =
+        b_tile + (wave_n * 64 + lane % 32) * kStride + 4 * (lane / 32);
+
+    for (unsigned k0 = 0; k0 < shape.contraction; k0 += kTileK) {
+        __syncthreads();  // previous step's fragment reads are done
+        store_activation_tile(staged, a_tile);
+        store_weight_tile<kBackward>(staged, table, b_tile);
+        __syncthreads();
+
+        const unsigned next = k0 + kTileK;
+        if (next < shape.contraction) {
+            load_activation_tile(staged, activations, shape, row0, next);
+            if constexpr (!kBackward) {
+                load_weight_tile_forward<kDoubleQuantized>(
+                    staged, weight, shape, col0, next, block_shift);
+            } else {
+                load_weight_tile_backward<kDoubleQuantized>(
+                    staged, weight, shape, col0, next, block_shift);
+            }
+        }
+
+#pragma unroll
+        for (int kk = 0; kk < kTileK; kk += 8) {
+            float4 a[2];
+            float4 b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                a[i] = *reinterpret_cast<const float4*>(
+                    a_fragment + i * 32 * kStride + kk);
+                b[i] = *reinterpret_cast<const float4*>(
+                    b_fragment + i * 32 * kStride + kk);
+            }
+            const float a_values[2][4] = {{a[0].x, a[0].y, a[0].z, a[0].w},
+                                          {a[1].x, a[1].y, a[1].z, a[1].w}};
+            const float b_values[2][4] = {{b[0].x, b[0].y, b[0].z, b[0].w},
+                                          {b[1].x, b[1].y, b[1].z, b[1].w}};
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                            a_values[i][s], b_values[j][s], acc[i][j], 0, 0,
+                            0);
+                    }
+                }
+            }
+        }
+    }
+
+    // Accumulator element e of lane l is output row 8*(e/4) + 4*(l/32) + e%4,
+    // column l%32 of its 32 x 32 block.
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const unsigned column = col0 + wave_n * 64 + j * 32 + lane % 32;
+            if (column >= shape.columns) {
+                continue;
+            }
+            float addend = 0.0F;
+            if constexpr (!kBackward) {
+                if (bias != nullptr) {
+                    addend = bias[column];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const unsigned row = row0 + wave_m * 64 + i * 32 +
+                                     8 * (e / 4) + 4 * (lane / 32) + e % 4;
+                if (row < shape.rows) {
+                    result[static_cast<std::size_t>(row) * shape.columns +
+                           column] = acc[i][j][e] + addend;
+                }
+            }
+        }
+    }
+}
+
+template <bool kBackward>
+void launch(const LinearProblem& p, hipStream_t stream) {
+    GemmShape shape;
+    shape.rows = static_cast<unsigned>(p.rows);
+    shape.input_width = static_cast<unsigned>(p.input_width);
+    if constexpr (!kBackward) {
+        shape.contraction = static_cast<unsigned>(p.input_width);
+        shape.columns = static_cast<unsigned>(p.output_width);
+    } else {
+        shape.contraction = static_cast<unsigned>(p.output_width);
+        shape.columns = static_cast<unsigned>(p.input_width);
+    }
+    const dim3 grid((shape.columns + kTileN - 1) / kTileN,
+                    (shape.rows + kTileM - 1) / kTileM);
+    if (p.weight.encoding == 0) {
+        mfma_gemm_kernel<false, kBackward><<<grid, kThreads, 0, stream>>>(
+            p.activations, p.weight, p.bias, p.result, shape, p.block_shift);
+    } else {
+        mfma_gemm_kernel<true, kBackward><<<grid, kThreads, 0, stream>>>(
+            p.activations, p.weight, p.bias, p.result, shape, p.block_shift);
+    }
+}
+
+bool common_supports(const LinearProblem& p) {
+    constexpr std::size_t kLimit = 1ULL << 31;
+    return p.rows >= 1 && p.rows < kLimit && p.input_width < kLimit &&
+           p.output_width < kLimit &&
+           (p.rows + kTileM - 1) / kTileM <= 65535 &&
+           reinterpret_cast<std::uintptr_t>(p.weight.codes) % 8 == 0 &&
+           reinterpret_cast<std::uintptr_t>(p.activations) % 16 == 0;
+}
+
+}  // namespace
+
+bool mfma_forward_supports(const LinearProblem& p) {
+    // Contraction over the row width in steps of 32; a 16-weight chunk must
+    // sit inside one quantisation block (true for every supported block size
+    // once the row width is a multiple of 16).
+    return common_supports(p) && p.input_width % kTileK == 0;
+}
+
+void launch_mfma_forward(const LinearProblem& p, hipStream_t stream) {
+    launch<false>(p, stream);
+}
+
+bool mfma_input_backward_supports(const LinearProblem& p) {
+    // Contraction over weight rows in steps of 32; output columns in chunks
+    // of 16 within a row.
+    return common_supports(p) && p.output_width % kTileK == 0 &&
+           p.input_width % kChunk == 0;
+}
+
+void launch_mfma_input_backward(const LinearProblem& p, hipStream_t stream) {
+    launch<true>(p, stream);
+}
+
+}  // namespace rthip

@@ -1,0 +1,520 @@
+// The C ABI of include/rthip.h: argument validation, kernel-family selection
+// and launch.  No C++ type crosses this boundary and no exception leaves it.
+
+#include "../../include/rthip.h"
+
+#include "kernels.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <limits>
+#include <mutex>
+
+namespace {
+
+thread_local char g_last_error[512] = "";
+
+rthip_status fail(rthip_status status, const char* format, ...) {
+    va_list arguments;
+    va_start(arguments, format);
+    std::vsnprintf(g_last_error, sizeof(g_last_error), format, arguments);
+    va_end(arguments);
+    return status;
+}
+
+rthip_status ok() {
+    g_last_error[0] = '\0';
+    return RTHIP_OK;
+}
+
+rthip_status from_hip(hipError_t error, const char* what) {
+    if (error == hipSuccess) {
+        return ok();
+    }
+    const rthip_status status = error == hipErrorOutOfMemory
+        ? RTHIP_OUT_OF_MEMORY
+        : RTHIP_RUNTIME_ERROR;
+    return fail(status, "%s: %s", what, hipGetErrorString(error));
+}
+
+// Device discovery runs once per process; the result (including the reason
+// for unavailability) is immutable afterwards.
+struct DeviceState {
+    rthip_status status = RTHIP_UNAVAILABLE;
+    int count = 0;
+    char description[256] = "";
+    char reason[256] = "";
+};
+
+const DeviceState& device_state() {
+    static DeviceState state;
+    static std::once_flag once;
+    std::call_once(once, [] {
+        int count = 0;
+        const hipError_t error = hipGetDeviceCount(&count);
+        if (error != hipSuccess || count <= 0) {
+            // Clear the sticky error so later calls report their own.
+            static_cast<void>(hipGetLastError());
+            std::snprintf(state.reason, sizeof(state.reason),
+                          "no HIP device is visible (%s)",
+                          error == hipSuccess ? "device count is zero"
+                                              : hipGetErrorString(error));
+            return;
+        }
+        hipDeviceProp_t properties;
+        if (hipGetDeviceProperties(&properties, 0) != hipSuccess) {
+            static_cast<void>(hipGetLastError());
+            std::snprintf(state.reason, sizeof(state.reason),
+                          "device 0 properties are unreadable");
+            return;
+        }
+        if (std::strncmp(properties.gcnArchName, "gfx950", 6) != 0) {
+            std::snprintf(state.reason, sizeof(state.reason),
+                          "device 0 is %s; this library carries gfx950 code "
+                          "only",
+                          properties.gcnArchName);
+            return;
+        }
+        state.status = RTHIP_OK;
+        state.count = count;
+        std::snprintf(state.description, sizeof(state.description),
+                      "%s (%s), %d CUs, %.0f GiB", properties.name,
+                      properties.gcnArchName, properties.multiProcessorCount,
+                      static_cast<double>(properties.totalGlobalMem) /
+                          (1024.0 * 1024.0 * 1024.0));
+    });
+    return state;
+}
+
+rthip_status require_device() {
+    const DeviceState& state = device_state();
+    if (state.status != RTHIP_OK) {
+        return fail(RTHIP_UNAVAILABLE, "%s", state.reason);
+    }
+    return RTHIP_OK;
+}
+
+// The block sizes the format allows (src/core/quantization/nf4.cpp:39-53).
+bool block_shift_for(uint64_t block_size, unsigned* shift) {
+    for (unsigned candidate = 5; candidate <= 12; ++candidate) {
+        if (block_size == (1ULL << candidate)) {
+            *shift = candidate;
+            return true;
+        }
+    }
+    return false;
+}
+
+rthip_status make_weight_view(
+    const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, rthip::Nf4WeightView* view
+) {
+    if (codes == nullptr || primary_scales == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "packed codes and primary scales must not be null");
+    }
+    view->codes = codes;
+    view->primary_scales = primary_scales;
+    view->secondary_scales = nullptr;
+    view->encoding = encoding;
+    view->second_level_shift = 0;
+    view->offset = 0.0F;
+    if (encoding == RTHIP_NF4_SCALE_FLOAT32) {
+        return RTHIP_OK;
+    }
+    if (encoding != RTHIP_NF4_SCALE_DOUBLE_QUANTIZED_UINT8) {
+        return fail(RTHIP_INVALID_ARGUMENT, "unknown NF4 scale encoding %d",
+                    static_cast<int>(encoding));
+    }
+    unsigned shift = 0;
+    if (!block_shift_for(second_level_block, &shift)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "second-level scale block %llu is not one of 32..4096",
+                    static_cast<unsigned long long>(second_level_block));
+    }
+    if (secondary_scales == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "double-quantized scales need second-level scales");
+    }
+    view->secondary_scales = secondary_scales;
+    view->second_level_shift = shift;
+    view->offset = offset;
+    return RTHIP_OK;
+}
+
+rthip_status check_dimensions(uint64_t rows, uint64_t input_width,
+                              uint64_t output_width, uint64_t block_size,
+                              unsigned* block_shift) {
+    if (rows == 0 || input_width == 0 || output_width == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "quantized linear dimensions must be positive");
+    }
+    if (!block_shift_for(block_size, block_shift)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "NF4 block size %llu is not one of 32..4096",
+                    static_cast<unsigned long long>(block_size));
+    }
+    constexpr uint64_t kMax = std::numeric_limits<uint64_t>::max() / 4;
+    if (input_width > kMax / output_width || rows > kMax / input_width ||
+        rows > kMax / output_width) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "quantized linear size exceeds addressable storage");
+    }
+    return RTHIP_OK;
+}
+
+rthip_status finish_launch(const char* what) {
+    return from_hip(hipGetLastError(), what);
+}
+
+int32_t select_forward(const rthip::LinearProblem& problem) {
+    if (problem.rows <= rthip::kGemvMaxRows &&
+        rthip::gemv_forward_supports(problem)) {
+        return RTHIP_NF4_ALGORITHM_GEMV;
+    }
+    if (rthip::mfma_forward_supports(problem)) {
+        return RTHIP_NF4_ALGORITHM_MFMA;
+    }
+    return RTHIP_NF4_ALGORITHM_GENERIC;
+}
+
+int32_t select_input_backward(const rthip::LinearProblem& problem) {
+    if (rthip::mfma_input_backward_supports(problem)) {
+        return RTHIP_NF4_ALGORITHM_MFMA;
+    }
+    return RTHIP_NF4_ALGORITHM_GENERIC;
+}
+
+}  // namespace
+
+extern "C" {
+
+uint32_t rthip_abi_version(void) {
+    return (RTHIP_ABI_VERSION_MAJOR << 16) | RTHIP_ABI_VERSION_MINOR;
+}
+
+const char* rthip_last_error(void) { return g_last_error; }
+
+rthip_status rthip_device_count(int32_t* count) {
+    if (count == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "count must not be null");
+    }
+    *count = 0;
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    *count = device_state().count;
+    return ok();
+}
+
+rthip_status rthip_device_description(char* buffer, size_t capacity) {
+    if (buffer == nullptr || capacity == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT, "buffer must not be empty");
+    }
+    buffer[0] = '\0';
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    std::snprintf(buffer, capacity, "%s", device_state().description);
+    return ok();
+}
+
+rthip_status rthip_malloc(void** pointer, size_t bytes) {
+    if (pointer == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "pointer must not be null");
+    }
+    *pointer = nullptr;
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    if (bytes == 0) {
+        return ok();
+    }
+    return from_hip(hipMalloc(pointer, bytes), "device allocation");
+}
+
+rthip_status rthip_free(void* pointer) {
+    if (pointer == nullptr) {
+        return ok();
+    }
+    return from_hip(hipFree(pointer), "device free");
+}
+
+rthip_status rthip_copy_to_device(void* device, const void* host,
+                                  size_t bytes) {
+    if (bytes == 0) {
+        return ok();
+    }
+    if (device == nullptr || host == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "copy pointers must not be null");
+    }
+    return from_hip(hipMemcpy(device, host, bytes, hipMemcpyHostToDevice),
+                    "host-to-device copy");
+}
+
+rthip_status rthip_copy_to_host(void* host, const void* device, size_t bytes) {
+    if (bytes == 0) {
+        return ok();
+    }
+    if (device == nullptr || host == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "copy pointers must not be null");
+    }
+    return from_hip(hipMemcpy(host, device, bytes, hipMemcpyDeviceToHost),
+                    "device-to-host copy");
+}
+
+rthip_status rthip_fill_f32(float* device, float value, uint64_t count,
+                            void* stream) {
+    if (count == 0) {
+        return ok();
+    }
+    if (device == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "fill target must not be null");
+    }
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    rthip::launch_fill(device, value, count,
+                       static_cast<hipStream_t>(stream));
+    return finish_launch("fill kernel launch");
+}
+
+rthip_status rthip_stream_synchronize(void* stream) {
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    return from_hip(hipStreamSynchronize(static_cast<hipStream_t>(stream)),
+                    "stream synchronisation");
+}
+
+rthip_status rthip_nf4_select_algorithm(
+    int32_t direction, uint64_t rows, uint64_t input_width,
+    uint64_t output_width, uint64_t block_size, int32_t* algorithm
+) {
+    if (algorithm == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "algorithm must not be null");
+    }
+    unsigned block_shift = 0;
+    if (const rthip_status status = check_dimensions(
+            rows, input_width, output_width, block_size, &block_shift);
+        status != RTHIP_OK) {
+        return status;
+    }
+    rthip::LinearProblem problem{};
+    problem.rows = rows;
+    problem.input_width = input_width;
+    problem.output_width = output_width;
+    problem.block_shift = block_shift;
+    if (direction == 0) {
+        *algorithm = select_forward(problem);
+    } else if (direction == 1) {
+        *algorithm = select_input_backward(problem);
+    } else {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "direction must be 0 (forward) or 1 (input backward)");
+    }
+    return ok();
+}
+
+rthip_status rthip_nf4_linear_forward_with(
+    int32_t algorithm, const float* x, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset,
+    const float* bias_or_null, float* y, uint64_t rows, uint64_t input_width,
+    uint64_t output_width, uint64_t block_size, void* stream
+) {
+    if (x == nullptr || y == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "input and output must not be null");
+    }
+    if (static_cast<const void*>(x) == static_cast<const void*>(y)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "quantized linear input and output must not alias");
+    }
+    rthip::LinearProblem problem{};
+    if (const rthip_status status = check_dimensions(
+            rows, input_width, output_width, block_size,
+            &problem.block_shift);
+        status != RTHIP_OK) {
+        return status;
+    }
+    if (const rthip_status status = make_weight_view(
+            codes, primary_scales, secondary_scales, encoding,
+            second_level_block, offset, &problem.weight);
+        status != RTHIP_OK) {
+        return status;
+    }
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    problem.activations = x;
+    problem.bias = bias_or_null;
+    problem.result = y;
+    problem.rows = rows;
+    problem.input_width = input_width;
+    problem.output_width = output_width;
+    const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+
+    if (algorithm == RTHIP_NF4_ALGORITHM_AUTO) {
+        algorithm = select_forward(problem);
+    }
+    switch (algorithm) {
+    case RTHIP_NF4_ALGORITHM_GENERIC:
+        rthip::launch_generic_forward(problem, hip_stream);
+        break;
+    case RTHIP_NF4_ALGORITHM_GEMV:
+        if (!rthip::gemv_forward_supports(problem)) {
+            return fail(RTHIP_UNSUPPORTED,
+                        "the GEMV family needs rows <= %zu, a row width that "
+                        "is a multiple of 16 and at most 16384, and aligned "
+                        "pointers",
+                        rthip::kGemvMaxRows);
+        }
+        rthip::launch_gemv_forward(problem, hip_stream);
+        break;
+    case RTHIP_NF4_ALGORITHM_MFMA:
+        if (!rthip::mfma_forward_supports(problem)) {
+            return fail(RTHIP_UNSUPPORTED,
+                        "the MFMA family needs a row width that is a "
+                        "multiple of 32 and aligned pointers");
+        }
+        rthip::launch_mfma_forward(problem, hip_stream);
+        break;
+    default:
+        return fail(RTHIP_INVALID_ARGUMENT, "unknown algorithm %d",
+                    static_cast<int>(algorithm));
+    }
+    return finish_launch("NF4 linear forward launch");
+}
+
+rthip_status rthip_nf4_linear_forward(
+    const float* x, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, const float* bias_or_null,
+    float* y, uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream
+) {
+    return rthip_nf4_linear_forward_with(
+        RTHIP_NF4_ALGORITHM_AUTO, x, codes, primary_scales, secondary_scales,
+        encoding, second_level_block, offset, bias_or_null, y, rows,
+        input_width, output_width, block_size, stream);
+}
+
+rthip_status rthip_nf4_linear_input_backward_with(
+    int32_t algorithm, const float* dy, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset, float* dx,
+    uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream
+) {
+    if (dy == nullptr || dx == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "upstream and input gradient must not be null");
+    }
+    if (static_cast<const void*>(dy) == static_cast<const void*>(dx)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "quantized linear upstream and input gradient must not "
+                    "alias");
+    }
+    rthip::LinearProblem problem{};
+    if (const rthip_status status = check_dimensions(
+            rows, input_width, output_width, block_size,
+            &problem.block_shift);
+        status != RTHIP_OK) {
+        return status;
+    }
+    if (const rthip_status status = make_weight_view(
+            codes, primary_scales, secondary_scales, encoding,
+            second_level_block, offset, &problem.weight);
+        status != RTHIP_OK) {
+        return status;
+    }
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    problem.activations = dy;
+    problem.bias = nullptr;
+    problem.result = dx;
+    problem.rows = rows;
+    problem.input_width = input_width;
+    problem.output_width = output_width;
+    const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+
+    if (algorithm == RTHIP_NF4_ALGORITHM_AUTO) {
+        algorithm = select_input_backward(problem);
+    }
+    switch (algorithm) {
+    case RTHIP_NF4_ALGORITHM_GENERIC:
+        rthip::launch_generic_input_backward(problem, hip_stream);
+        break;
+    case RTHIP_NF4_ALGORITHM_MFMA:
+        if (!rthip::mfma_input_backward_supports(problem)) {
+            return fail(RTHIP_UNSUPPORTED,
+                        "the MFMA family needs an output width that is a "
+                        "multiple of 32, a row width that is a multiple of "
+                        "16 and aligned pointers");
+        }
+        rthip::launch_mfma_input_backward(problem, hip_stream);
+        break;
+    case RTHIP_NF4_ALGORITHM_GEMV:
+        return fail(RTHIP_UNSUPPORTED,
+                    "the GEMV family implements the forward product only");
+    default:
+        return fail(RTHIP_INVALID_ARGUMENT, "unknown algorithm %d",
+                    static_cast<int>(algorithm));
+    }
+    return finish_launch("NF4 linear input-backward launch");
+}
+
+rthip_status rthip_nf4_linear_input_backward(
+    const float* dy, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, float* dx, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream
+) {
+    return rthip_nf4_linear_input_backward_with(
+        RTHIP_NF4_ALGORITHM_AUTO, dy, codes, primary_scales, secondary_scales,
+        encoding, second_level_block, offset, dx, rows, input_width,
+        output_width, block_size, stream);
+}
+
+rthip_status rthip_nf4_dequantize(
+    const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, float* out,
+    uint64_t element_count, uint64_t block_size, void* stream
+) {
+    if (out == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "output must not be null");
+    }
+    if (element_count == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "element count must be positive");
+    }
+    unsigned block_shift = 0;
+    if (!block_shift_for(block_size, &block_shift)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "NF4 block size %llu is not one of 32..4096",
+                    static_cast<unsigned long long>(block_size));
+    }
+    rthip::Nf4WeightView weight{};
+    if (const rthip_status status = make_weight_view(
+            codes, primary_scales, secondary_scales, encoding,
+            second_level_block, offset, &weight);
+        status != RTHIP_OK) {
+        return status;
+    }
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    rthip::launch_dequantize(weight, out, element_count, block_shift,
+                             static_cast<hipStream_t>(stream));
+    return finish_launch("NF4 dequantize launch");
+}
+
+}  // extern "C"

@@ -1,0 +1,79 @@
+"""PyTorch plumbing around the C ABI: torch allocates device memory and owns
+the stream, librthip.so does all the arithmetic.  Importing this module needs
+torch; nothing here computes on the host."""
+from __future__ import annotations
+
+from typing import Optional
+
+import numpy as np
+import torch
+
+from .binding import (
+    SCALE_DOUBLE_QUANTIZED_UINT8,
+    SCALE_FLOAT32,
+    DeviceWeight,
+    load_library,
+)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def upload_weight(output_width: int, input_width: int, block_size: int,
+                  codes: np.ndarray, *, fp32_scales=None, scale_codes=None,
+                  second_level=None, second_level_block: int = 0,
+                  offset: float = 0.0, device="cuda") -> DeviceWeight:
+    """Copies a canonical host payload (the fields of the reference's
+    Nf4Payload) into device memory, byte for byte."""
+    codes_t = torch.from_numpy(np.ascontiguousarray(codes)).to(device)
+    if fp32_scales is not None:
+        primary = torch.from_numpy(
+            np.ascontiguousarray(fp32_scales, dtype=np.float32)).to(device)
+        return DeviceWeight(output_width, input_width, block_size,
+                            SCALE_FLOAT32, codes_t, primary, None)
+    primary = torch.from_numpy(
+        np.ascontiguousarray(scale_codes, dtype=np.uint8)).to(device)
+    secondary = torch.from_numpy(
+        np.ascontiguousarray(second_level, dtype=np.float32)).to(device)
+    return DeviceWeight(output_width, input_width, block_size,
+                        SCALE_DOUBLE_QUANTIZED_UINT8, codes_t, primary,
+                        secondary, second_level_block, float(offset))
+
+
+def linear_forward(x: torch.Tensor, weight: DeviceWeight,
+                   bias: Optional[torch.Tensor] = None,
+                   out: Optional[torch.Tensor] = None,
+                   algorithm: Optional[int] = None) -> torch.Tensor:
+    """y = x . deq(W)^T (+ bias) through rthip_nf4_linear_forward."""
+    assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous()
+    rows = x.numel() // weight.input_width
+    if out is None:
+        out = torch.empty((rows, weight.output_width), dtype=torch.float32,
+                          device=x.device)
+    load_library().linear_forward(
+        x.data_ptr(), weight, None if bias is None else bias.data_ptr(),
+        out.data_ptr(), rows, _stream(), algorithm)
+    return out
+
+
+def linear_input_backward(dy: torch.Tensor, weight: DeviceWeight,
+                          out: Optional[torch.Tensor] = None,
+                          algorithm: Optional[int] = None) -> torch.Tensor:
+    """dx = dy . deq(W) through rthip_nf4_linear_input_backward."""
+    assert dy.is_cuda and dy.dtype == torch.float32 and dy.is_contiguous()
+    rows = dy.numel() // weight.output_width
+    if out is None:
+        out = torch.empty((rows, weight.input_width), dtype=torch.float32,
+                          device=dy.device)
+    load_library().linear_input_backward(
+        dy.data_ptr(), weight, out.data_ptr(), rows, _stream(), algorithm)
+    return out
+
+
+def dequantize(weight: DeviceWeight) -> torch.Tensor:
+    """deq(W) as an fp32 tensor through rthip_nf4_dequantize (checking aid)."""
+    out = torch.empty((weight.output_width, weight.input_width),
+                      dtype=torch.float32, device=weight.codes.device)
+    load_library().dequantize(weight, out.data_ptr(), stream=_stream())
+    return out

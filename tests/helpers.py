@@ -1,0 +1,135 @@
+"""Test helpers: deterministic inputs, the reference tests' closed-form
+fixtures restated as numpy generators, and the error measures of the parity
+bar."""
+from __future__ import annotations
+
+import hashlib
+
+import numpy as np
+
+# The seven Llama-7B projection shapes (output_width, input_width).
+LLAMA_SHAPES = {
+    "q_proj": (4096, 4096),
+    "k_proj": (4096, 4096),
+    "v_proj": (4096, 4096),
+    "o_proj": (4096, 4096),
+    "gate_proj": (11008, 4096),
+    "up_proj": (11008, 4096),
+    "down_proj": (4096, 11008),
+}
+
+
+def normal(seed: int, shape, sigma: float) -> np.ndarray:
+    """N(0, sigma) fp32 values from numpy's PCG64 stream `seed`."""
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal(shape, dtype=np.float32) *
+            np.float32(sigma)).astype(np.float32)
+
+
+def bits(array: np.ndarray) -> np.ndarray:
+    return np.ascontiguousarray(array, dtype=np.float32).view(np.uint32)
+
+
+def sha256(array: np.ndarray) -> str:
+    return hashlib.sha256(np.ascontiguousarray(array).tobytes()).hexdigest()
+
+
+def assert_bit_equal(actual, expected, what: str = "") -> None:
+    a, e = bits(actual), bits(expected)
+    assert a.shape == e.shape, f"{what}: shape {a.shape} != {e.shape}"
+    if not np.array_equal(a, e):
+        bad = np.flatnonzero(a.ravel() != e.ravel())
+        index = int(bad[0])
+        raise AssertionError(
+            f"{what}: {bad.size} of {a.size} values differ bitwise; first at "
+            f"flat index {index}: {np.ravel(actual)[index]!r} != "
+            f"{np.ravel(expected)[index]!r}")
+
+
+# ---- closed-form fixtures ------------------------------------------------
+# Integer-formula tensors of the reference's backend parity test
+# (tests/core/backend/test_quantized_linear_backend.cpp:89-169).
+
+def aligned_weight() -> np.ndarray:  # :89-100
+    index = np.arange(3 * 32)
+    values = ((index % 19) - 9).astype(np.float32) * np.float32(0.1375)
+    values[0] = -2.0
+    values[31] = 1.75
+    values[32] = 3.0
+    values[-1] = -4.0
+    return values.reshape(3, 32)
+
+
+def aligned_input() -> np.ndarray:  # :102-109
+    index = np.arange(2 * 32)
+    return (((index % 11) - 5).astype(np.float32) *
+            np.float32(0.2)).reshape(2, 32)
+
+
+def aligned_upstream() -> np.ndarray:  # :111-124
+    return np.array([[0.25, -0.75, 1.5], [-1.0, 0.5, 0.125]],
+                    dtype=np.float32)
+
+
+EDGE = 33
+
+
+def edge_weight() -> np.ndarray:  # :126-142
+    index = np.arange(EDGE * EDGE)
+    values = ((index % 37) - 18).astype(np.float32) * np.float32(0.0625)
+    values[0] = -3.0
+    values[31] = 2.5
+    values[32] = -2.75
+    values[1023] = 4.0
+    values[1024] = -4.5
+    values[-1] = 5.0
+    return values.reshape(EDGE, EDGE)
+
+
+def edge_input() -> np.ndarray:  # :144-155
+    index = np.arange(2 * EDGE)
+    return (((index % 17) - 8).astype(np.float32) *
+            np.float32(0.125)).reshape(2, EDGE)
+
+
+def edge_upstream() -> np.ndarray:  # :157-168
+    index = np.arange(2 * EDGE)
+    return (((index % 13) - 6).astype(np.float32) *
+            np.float32(0.075)).reshape(2, EDGE)
+
+
+# ---- error measures ------------------------------------------------------
+
+def reference_close(actual, expected, tolerance: float = 3.0e-5) -> bool:
+    """The reference's own check: |a-e| <= tol * max(1, |a|, |e|)
+    (tests/core/backend/test_quantized_linear_backend.cpp:46-70)."""
+    actual = np.asarray(actual, dtype=np.float32)
+    expected = np.asarray(expected, dtype=np.float32)
+    scale = np.maximum(1.0, np.maximum(np.abs(actual), np.abs(expected)))
+    return bool(np.all(np.isfinite(actual)) and
+                np.all(np.abs(actual - expected) <= tolerance * scale))
+
+
+def rms(values) -> float:
+    values = np.asarray(values, dtype=np.float64)
+    return float(np.sqrt(np.mean(values * values)))
+
+
+def normalized_error(actual, expected, contraction: int, activation_rms: float,
+                     weight_rms: float) -> float:
+    """max |a - e| / (sqrt(K) * rms(activations) * rms(deq W)): the error in
+    units of one standard deviation of an output."""
+    difference = np.abs(np.asarray(actual, dtype=np.float64) -
+                        np.asarray(expected, dtype=np.float64)).max()
+    return float(difference /
+                 (np.sqrt(contraction) * activation_rms * weight_rms))
+
+
+def exact_forward(x, dense) -> np.ndarray:
+    """fp64-accumulated x . dense^T."""
+    return np.asarray(x, np.float64) @ np.asarray(dense, np.float64).T
+
+
+def exact_input_backward(dy, dense) -> np.ndarray:
+    """fp64-accumulated dy . dense."""
+    return np.asarray(dy, np.float64) @ np.asarray(dense, np.float64)

@@ -1,0 +1,158 @@
+"""Pins the CPU restatement (oracle/) to the known-answer vectors the
+reference's own unit tests hold.  Each test names the reference test it
+restates (paths under /root/reference)."""
+import numpy as np
+import pytest
+
+from oracle.binding import (SCALE_DOUBLE_QUANTIZED_UINT8, SCALE_FLOAT32,
+                            Nf4Weight)
+
+CODEBOOK = np.array([
+    -1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453,
+    -0.28444138169288635, -0.18477343022823334, -0.09105003625154495, 0.0,
+    0.07958029955625534, 0.16093020141124725, 0.24611230194568634,
+    0.33791524171829224, 0.44070982933044434, 0.5626170039176941,
+    0.7229568362236023, 1.0], dtype=np.float32)
+
+
+def unpack(codes, index):
+    byte = int(codes[index // 2])
+    return byte & 0x0F if index % 2 == 0 else byte >> 4
+
+
+def test_codebook_literals_and_canonical_packing(oracle):
+    # tests/core/test_quantization.cpp:62-112
+    codebook = oracle.codebook()
+    assert np.array_equal(codebook.view(np.uint32), CODEBOOK.view(np.uint32))
+    assert np.all(np.diff(codebook) > 0)
+    assert codebook[7] == 0.0
+    weight = oracle.quantize(CODEBOOK, 32)
+    assert weight.codes.tolist() == [0x10, 0x32, 0x54, 0x76, 0x98, 0xBA,
+                                     0xDC, 0xFE]
+    assert weight.fp32_scales.tolist() == [1.0]
+    restored = oracle.dequantize(weight).ravel()
+    assert np.array_equal(restored.view(np.uint32), CODEBOOK.view(np.uint32))
+
+
+def test_midpoint_tie_chooses_lower_code(oracle):
+    # tests/core/test_quantization.cpp:114-125
+    values = np.zeros(32, dtype=np.float32)
+    values[0] = CODEBOOK[8] * np.float32(0.5)
+    values[-1] = 1.0
+    weight = oracle.quantize(values, 32)
+    assert unpack(weight.codes, 0) == 7
+    assert oracle.nearest_code(CODEBOOK[8] * np.float32(0.5)) == 7
+
+
+def test_zero_blocks_use_code_seven_and_zero_scale(oracle):
+    # tests/core/test_quantization.cpp:127-137
+    weight = oracle.quantize(np.zeros(33, dtype=np.float32), 32)
+    assert weight.fp32_scales.tolist() == [0.0, 0.0]
+    assert all(unpack(weight.codes, i) == 7 for i in range(33))
+    assert weight.codes[-1] == 0x07
+
+
+def test_partial_block_has_its_own_scale(oracle):
+    # tests/core/test_quantization.cpp:139-152
+    values = np.full(33, 0.25, dtype=np.float32)
+    values[0] = -2.0
+    values[-1] = 10.0
+    weight = oracle.quantize(values, 32)
+    assert weight.fp32_scales.tolist() == [2.0, 10.0]
+    assert unpack(weight.codes, 0) == 0 and unpack(weight.codes, 32) == 15
+    restored = oracle.dequantize(weight).ravel()
+    assert restored[0] == -2.0 and restored[32] == 10.0
+
+
+def test_double_quantized_scale_packing_and_bytes(oracle):
+    # tests/core/test_quantization.cpp:155-205
+    values = np.repeat(np.arange(33, dtype=np.float32), 32)
+    weight = oracle.quantize(values, 32, double_quantized=True,
+                             second_level_block=32)
+    assert weight.encoding == SCALE_DOUBLE_QUANTIZED_UINT8
+    assert weight.fp32_scales is None
+    assert weight.scale_codes.size == 33
+    assert weight.second_level.tolist() == [16.0, 16.0]
+    assert weight.offset == 16.0
+    assert weight.scale_codes[0] == 1
+    assert weight.scale_codes[16] == 128
+    assert weight.scale_codes[32] == 255
+    restored = oracle.dequantize(weight).ravel()
+    assert restored[0] == 0.0
+    assert restored[16 * 32] == 16.0
+    assert restored[32 * 32] == 32.0
+    # packed 528, scales 33 + 2*4 + 4 = 45, logical 573, fp32 4224
+    assert weight.codes.size == 528
+    assert oracle.scale_payload_bytes(weight) == 45
+    assert weight.payload_bytes == 573
+    assert weight.element_count * 4 == 4224
+
+
+def test_sixty_four_zeros_use_36_bytes(oracle):
+    # tests/core/test_quantization.cpp:368-376
+    weight = oracle.quantize(np.zeros(64, dtype=np.float32), 64)
+    assert weight.codes.size == 32
+    assert oracle.scale_payload_bytes(weight) == 4
+    assert weight.payload_bytes == 36
+
+
+def scalar_zero():
+    return Nf4Weight(1, 1, 32, np.array([0x07], dtype=np.uint8),
+                     SCALE_FLOAT32, fp32_scales=np.zeros(1, np.float32))
+
+
+def double_scalar_zero():
+    return Nf4Weight(1, 1, 32, np.array([0x07], dtype=np.uint8),
+                     SCALE_DOUBLE_QUANTIZED_UINT8,
+                     scale_codes=np.array([128], dtype=np.uint8),
+                     second_level=np.zeros(1, np.float32),
+                     second_level_block=32, offset=0.0)
+
+
+def test_payload_validation_accepts_canonical_scalars(oracle):
+    # tests/core/test_quantization.cpp:207-223
+    oracle.validate_payload(scalar_zero())
+    oracle.validate_payload(double_scalar_zero())
+    assert oracle.dequantize(scalar_zero()).ravel()[0] == 0.0
+
+
+@pytest.mark.parametrize("mutate", [
+    # tests/core/test_quantization.cpp:225-345, one entry per require_throws
+    lambda w: setattr(w, "codes", np.zeros(0, np.uint8)),
+    lambda w: setattr(w, "fp32_scales", np.zeros(0, np.float32)),
+    lambda w: setattr(w, "codes", np.array([0xF7], np.uint8)),
+    lambda w: setattr(w, "codes", np.array([0x08], np.uint8)),
+    lambda w: setattr(w, "fp32_scales", np.array([-1.0], np.float32)),
+    lambda w: setattr(w, "fp32_scales", np.array([np.inf], np.float32)),
+])
+def test_payload_validation_rejects_legacy(oracle, mutate):
+    weight = scalar_zero()
+    mutate(weight)
+    with pytest.raises(ValueError):
+        oracle.validate_payload(weight)
+
+
+@pytest.mark.parametrize("mutate", [
+    lambda w: setattr(w, "fp32_scales", np.zeros(1, np.float32)),
+    lambda w: setattr(w, "scale_codes", np.zeros(0, np.uint8)),
+    lambda w: setattr(w, "second_level_block", 16),
+    lambda w: setattr(w, "second_level", np.zeros(0, np.float32)),
+    lambda w: setattr(w, "second_level", np.array([-1.0], np.float32)),
+    lambda w: setattr(w, "offset", float("inf")),
+])
+def test_payload_validation_rejects_double_quantized(oracle, mutate):
+    weight = double_scalar_zero()
+    mutate(weight)
+    with pytest.raises(ValueError):
+        oracle.validate_payload(weight)
+
+
+def test_block_sizes_and_nonfinite_sources(oracle):
+    # src/core/quantization/nf4.cpp:39-53; test_quantization.cpp:347-359
+    supported = [32, 64, 128, 256, 512, 1024, 2048, 4096]
+    for size in range(1, 8200):
+        assert oracle.block_size_supported(size) == (size in supported)
+    values = np.zeros(32, dtype=np.float32)
+    values[0] = np.nan
+    with pytest.raises(ValueError):
+        oracle.quantize(values, 32)

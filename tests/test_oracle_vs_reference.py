@@ -1,0 +1,107 @@
+"""Where oracle/_ref was built (the container that holds the reference), diff
+the C restatement against the compiled reference on fresh seeded inputs,
+including error behaviour.  Skipped where the reference build is absent."""
+import numpy as np
+import pytest
+
+import helpers
+from oracle.binding import (SCALE_DOUBLE_QUANTIZED_UINT8, SCALE_FLOAT32,
+                            Nf4Weight)
+
+
+def same_payload(a, b):
+    assert np.array_equal(a.codes, b.codes)
+    if a.encoding == SCALE_FLOAT32:
+        helpers.assert_bit_equal(a.fp32_scales, b.fp32_scales)
+    else:
+        assert np.array_equal(a.scale_codes, b.scale_codes)
+        helpers.assert_bit_equal(a.second_level, b.second_level)
+        helpers.assert_bit_equal(np.float32(a.offset), np.float32(b.offset))
+
+
+@pytest.mark.parametrize("shape,block,second", [
+    ((768, 256), 64, 256), ((33, 33), 32, 32), ((17, 96), 32, 64),
+    ((5, 4096), 4096, 32), ((64, 1000), 128, 32), ((1, 1), 32, 32)])
+@pytest.mark.parametrize("double_quantized", [False, True])
+@pytest.mark.parametrize("sigma", [0.02, 1.0])
+def test_bitwise_agreement(oracle, reference, shape, block, second,
+                           double_quantized, sigma):
+    out_w, in_w = shape
+    dense = helpers.normal(41, shape, sigma)
+    dense.ravel()[::7] = 0.0  # exact zeros and ties at code 7
+    mine = oracle.quantize(dense, block, double_quantized, second)
+    theirs = reference.quantize(dense, block, double_quantized, second)
+    same_payload(mine, theirs)
+    helpers.assert_bit_equal(oracle.dequantize(mine),
+                             reference.dequantize(mine))
+    x = helpers.normal(42, (3, in_w), 1.0)
+    dy = helpers.normal(43, (3, out_w), 1.0e-2)
+    helpers.assert_bit_equal(oracle.forward(x, mine, faithful=True),
+                             reference.forward(x, mine))
+    helpers.assert_bit_equal(oracle.forward(x, mine),
+                             reference.forward(x, mine))
+    helpers.assert_bit_equal(oracle.input_backward(dy, mine, faithful=True),
+                             reference.input_backward(dy, mine))
+    helpers.assert_bit_equal(oracle.input_backward(dy, mine),
+                             reference.input_backward(dy, mine))
+
+
+def test_zero_block_and_constant_scales(oracle, reference):
+    dense = np.zeros((4, 64), np.float32)
+    dense[2] = 0.5
+    for dq in (False, True):
+        same_payload(oracle.quantize(dense, 32, dq, 32),
+                     reference.quantize(dense, 32, dq, 32))
+
+
+def test_validation_agrees(oracle, reference):
+    def legacy(codes, scales):
+        return Nf4Weight(1, 1, 32, np.array(codes, np.uint8), SCALE_FLOAT32,
+                         fp32_scales=np.array(scales, np.float32))
+
+    def nested(**changes):
+        weight = Nf4Weight(1, 1, 32, np.array([0x07], np.uint8),
+                           SCALE_DOUBLE_QUANTIZED_UINT8,
+                           scale_codes=np.array([128], np.uint8),
+                           second_level=np.zeros(1, np.float32),
+                           second_level_block=32, offset=0.0)
+        for key, value in changes.items():
+            setattr(weight, key, value)
+        return weight
+
+    good = [legacy([0x07], [0.0]), nested()]
+    bad = [
+        legacy([], [0.0]), legacy([0x07], []), legacy([0xF7], [0.0]),
+        legacy([0x08], [0.0]), legacy([0x07], [-1.0]),
+        legacy([0x07], [np.inf]),
+        nested(fp32_scales=np.zeros(1, np.float32)),
+        nested(scale_codes=np.zeros(0, np.uint8)),
+        nested(second_level_block=16),
+        nested(second_level=np.zeros(0, np.float32)),
+        nested(second_level=np.array([-1.0], np.float32)),
+        nested(offset=float("inf")),
+    ]
+    for weight in good:
+        oracle.validate_payload(weight)
+        reference.validate_payload(weight)
+    for weight in bad:
+        with pytest.raises(ValueError) as mine:
+            oracle.validate_payload(weight)
+        with pytest.raises(ValueError) as theirs:
+            reference.validate_payload(weight)
+        assert str(mine.value) == str(theirs.value)
+
+
+def test_memory_usage_known_answers(oracle, reference):
+    # tests/core/test_quantization.cpp:188-198 and :368-376
+    values = np.repeat(np.arange(33, dtype=np.float32), 32)
+    weight = oracle.quantize(values, 32, True, 32)
+    usage = reference.memory_usage(weight)
+    assert usage == {
+        "packed_code_bytes": 528, "scale_bytes": 45,
+        "logical_payload_bytes": 573, "resident_payload_bytes": 573,
+        "fp32_equivalent_bytes": 4224, "fp32_scale_bytes": 0,
+        "scale_code_bytes": 33, "second_level_scale_bytes": 8,
+        "scale_offset_bytes": 4}
+    assert oracle.scale_payload_bytes(weight) == usage["scale_bytes"]
+    assert weight.payload_bytes == usage["logical_payload_bytes"]
