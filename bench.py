@@ -1,0 +1,317 @@
+"""Benchmark of the packed NF4 linear path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L]
+
+Headline workload (the configuration the metric is quoted on): decode GEMV,
+M = 1, the seven Llama-7B projection shapes per layer (q/k/v/o 4096x4096,
+gate/up 11008x4096, down 4096x11008), NF4 block 64 with fp32 absmax scales, no
+bias.  One step = one token through all 7 projections of L layers, every layer
+holding its own packed weights, so the working set (L x 113.8 MB) is far
+larger than the 256 MB last-level cache and every step streams it from HBM.
+`value` = algorithmic bytes (packed codes + scale payload) per second with
+everything resident in HBM before the timed region.
+
+The same JSON line carries
+  roofline      HBM roofline of the GEMV kernel (bytes per launch / average
+                launch duration from HIP events on the launch stream)
+  gemm          M = 2048 forward and input-backward GEMMs of BASELINE configs 4
+                and 5 with their fp32-MFMA rooflines
+  small_batch   M in {4, 16, 64} on the three distinct shapes (config 3)
+  cpu_baseline  the reference CPU backend (oracle/_ref, else the C
+                restatement) timed on this host, single thread, on one layer
+
+Packed payloads are synthetic: uniformly random nibbles (NF4 codes of normal
+weights are close to uniform by construction) and block scales drawn around
+the absmax of 64 samples of N(0, 0.02), generated on the device.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
+
+LAYER_SHAPES = [  # (name, output_width, input_width)
+    ("q_proj", 4096, 4096), ("k_proj", 4096, 4096), ("v_proj", 4096, 4096),
+    ("o_proj", 4096, 4096), ("gate_proj", 11008, 4096),
+    ("up_proj", 11008, 4096), ("down_proj", 4096, 11008),
+]
+BLOCK = 64
+SECOND_LEVEL_BLOCK = 256
+
+
+def synthetic_weight(package, torch, out_w, in_w, double_quantized, seed):
+    """A packed weight generated directly in HBM."""
+    generator = torch.Generator(device="cuda")
+    generator.manual_seed(seed)
+    count = out_w * in_w
+    blocks = count // BLOCK
+    codes = torch.randint(0, 256, (count // 2,), dtype=torch.uint8,
+                          device="cuda", generator=generator)
+    if not double_quantized:
+        scales = (torch.rand(blocks, device="cuda", generator=generator) *
+                  0.03 + 0.035)
+        return package.DeviceWeight(out_w, in_w, BLOCK, package.SCALE_FLOAT32,
+                                    codes, scales, None)
+    scale_codes = torch.randint(1, 256, (blocks,), dtype=torch.uint8,
+                                device="cuda", generator=generator)
+    groups = -(-blocks // SECOND_LEVEL_BLOCK)
+    second = (torch.rand(groups, device="cuda", generator=generator) *
+              0.01 + 0.02)
+    return package.DeviceWeight(
+        out_w, in_w, BLOCK, package.SCALE_DOUBLE_QUANTIZED_UINT8, codes,
+        scale_codes, second, SECOND_LEVEL_BLOCK, 0.05)
+
+
+def capture(torch, body):
+    """Records body()'s launches into a HIP graph and returns its replay.  The
+    decode kernels last microseconds, far less than a Python-level launch, so
+    the launch-bound loops are replayed as graphs (kernel nodes only)."""
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        body()
+    return graph.replay
+
+
+def time_region(torch, body, repeats):
+    """Milliseconds for `repeats` calls of body(), bracketed by HIP events on
+    the stream the kernels are launched on."""
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(repeats):
+        body()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop)
+
+
+def bench_decode(package, device, torch, layers, steps, warmup, use_graph):
+    library = package.load_library()
+    weights = []
+    for layer in range(layers):
+        for index, (_, out_w, in_w) in enumerate(LAYER_SHAPES):
+            weights.append(synthetic_weight(package, torch, out_w, in_w,
+                                            False, 1000 * layer + index))
+    x = {width: torch.randn(1, width, device="cuda")
+         for width in (4096, 11008)}
+    y = {width: torch.empty(1, width, device="cuda")
+         for width in (4096, 11008)}
+    launches = [(x[w.input_width].data_ptr(), w, y[w.output_width].data_ptr())
+                for w in weights]
+
+    def launch_all(items):
+        stream = torch.cuda.current_stream().cuda_stream
+        for x_ptr, weight, y_ptr in items:
+            library.linear_forward(x_ptr, weight, None, y_ptr, 1, stream)
+
+    launch_all(launches)  # first use outside any capture
+    torch.cuda.synchronize()
+    step = lambda: launch_all(launches)
+    if use_graph:
+        step = capture(torch, step)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter()
+    milliseconds = time_region(torch, step, steps)
+    wall = time.perf_counter() - wall
+    bytes_per_step = sum(w.payload_bytes for w in weights)
+    launches_per_step = len(weights)
+    seconds = milliseconds / 1e3
+    gbs = bytes_per_step * steps / seconds / 1e9
+
+    # The dominant kernel: the K = 4096 instantiation (6 of 7 projections).
+    dominant = [item for item in launches if item[1].input_width == 4096]
+
+    dominant_pass = lambda: launch_all(dominant)
+    if use_graph:
+        dominant_pass = capture(torch, dominant_pass)
+    dominant_pass()
+    dominant_ms = time_region(torch, dominant_pass, steps)
+    dominant_bytes = sum(item[1].payload_bytes for item in dominant)
+    average_us = dominant_ms * 1e3 / (steps * len(dominant))
+    achieved = dominant_bytes * steps / (dominant_ms / 1e3) / 1e9
+    return {
+        "value": gbs,
+        "ms_per_step": milliseconds / steps,
+        "wall_seconds": wall,
+        "bytes_per_step": bytes_per_step,
+        "launches_per_step": launches_per_step,
+        "roofline": {
+            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "kernel": "gemv_forward_kernel<rows=1, K=4096>",
+            "bytes_per_launch": dominant_bytes / len(dominant),
+            "avg_launch_us": average_us,
+        },
+    }
+
+
+def bench_gemm(package, device, torch, steps):
+    """BASELINE configs 4 and 5: M = 2048."""
+    rows = 2048
+    results = []
+    cases = [
+        ("forward", 11008, 4096, False), ("forward", 11008, 4096, True),
+        ("forward", 4096, 4096, False), ("forward", 4096, 4096, True),
+        ("input_backward", 4096, 11008, True),
+        ("input_backward", 11008, 4096, True),
+    ]
+    for direction, out_w, in_w, double_quantized in cases:
+        weight = synthetic_weight(package, torch, out_w, in_w,
+                                  double_quantized, 77)
+        if direction == "forward":
+            source = torch.randn(rows, in_w, device="cuda")
+            target = torch.empty(rows, out_w, device="cuda")
+            body = lambda: device.linear_forward(source, weight, out=target)
+        else:
+            source = torch.randn(rows, out_w, device="cuda") * 1e-2
+            target = torch.empty(rows, in_w, device="cuda")
+            body = lambda: device.linear_input_backward(source, weight,
+                                                        out=target)
+        body()
+        body()
+        milliseconds = time_region(torch, body, steps) / steps
+        flops = 2.0 * rows * out_w * in_w
+        tflops = flops / (milliseconds / 1e3) / 1e12
+        results.append({
+            "direction": direction, "rows": rows, "output_width": out_w,
+            "input_width": in_w,
+            "scales": "double_quantized" if double_quantized else "fp32",
+            "ms": milliseconds,
+            "roofline": {"bound": "mfma", "achieved": tflops,
+                         "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
+                         "traffic": None},
+        })
+        del source, target, weight
+    return results
+
+
+def bench_small_batch(package, device, torch, steps):
+    """BASELINE config 3: M in {4, 16, 64}, fp32 scales; rotating weights."""
+    results = []
+    copies = 12  # 12 x >= 9.4 MB per shape: beyond the last-level cache
+    for name, out_w, in_w in (LAYER_SHAPES[0], LAYER_SHAPES[4],
+                              LAYER_SHAPES[6]):
+        weights = [synthetic_weight(package, torch, out_w, in_w, False, 500 + i)
+                   for i in range(copies * (3 if out_w * in_w < 2 ** 25 else 1))]
+        for rows in (1, 4, 16, 64):
+            source = torch.randn(rows, in_w, device="cuda")
+            target = torch.empty(rows, out_w, device="cuda")
+
+            def body():
+                for weight in weights:
+                    device.linear_forward(source, weight, out=target)
+
+            body()
+            torch.cuda.synchronize()
+            body = capture(torch, body)
+            body()
+            milliseconds = time_region(torch, body, steps) / (
+                steps * len(weights))
+            results.append({
+                "shape": name, "rows": rows, "us": milliseconds * 1e3,
+                "gb_per_s": weights[0].payload_bytes / milliseconds / 1e6,
+                "tflop_per_s": 2.0 * rows * out_w * in_w / milliseconds / 1e9,
+            })
+        del weights
+    return results
+
+
+def cpu_baseline():
+    """One Llama-7B layer (7 projections, M = 1) on the host, single thread."""
+    import numpy as np
+    from oracle.binding import Nf4Weight, Oracle, Reference
+    backend = Reference() if Reference.available() else Oracle()
+    rng = np.random.default_rng(3)
+    total_bytes = 0
+    seconds = 0.0
+    for _, out_w, in_w in LAYER_SHAPES:
+        count = out_w * in_w
+        codes = rng.integers(0, 256, count // 2, dtype=np.uint8)
+        scales = (rng.random(count // BLOCK, dtype=np.float32) *
+                  np.float32(0.03) + np.float32(0.035))
+        weight = Nf4Weight(out_w, in_w, BLOCK, codes, 0, fp32_scales=scales)
+        x = rng.standard_normal((1, in_w), dtype=np.float32)
+        begin = time.perf_counter()
+        backend.forward(x, weight, faithful=True)
+        seconds += time.perf_counter() - begin
+        total_bytes += weight.payload_bytes
+    return {
+        "value": total_bytes / seconds / 1e9, "unit": "GB/s", "cores": 1,
+        "kind": backend.kind, "seconds": seconds,
+        "sample": "one Llama-7B layer: 7 projections at M=1, fp32 scales, "
+                  "one pass (%.1f MB packed)" % (total_bytes / 1e6),
+    }
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--layers", type=int, default=32)
+    parser.add_argument("--skip-extras", action="store_true",
+                        help="only the headline decode workload")
+    parser.add_argument("--skip-cpu", action="store_true")
+    parser.add_argument("--no-graph", action="store_true",
+                        help="launch the decode kernels one by one from "
+                             "Python instead of replaying a HIP graph")
+    arguments = parser.parse_args()
+    if arguments.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; the path has no "
+                 "collectives or sharding (--gpus %d refused)" % arguments.gpus)
+
+    import torch
+    package = importlib.import_module("riftco-transformer_amd")
+    device = importlib.import_module("riftco-transformer_amd.device")
+    library = package.load_library()
+    if not torch.cuda.is_available() or not library.is_available():
+        sys.exit("bench.py: no usable MI355X: " + library.last_error())
+
+    decode = bench_decode(package, device, torch, arguments.layers,
+                          arguments.steps, arguments.warmup,
+                          not arguments.no_graph)
+    line = {
+        "metric": "NF4 linear: HBM GB/s at M=1, TFLOP/s at M=2048, % of "
+                  "MI355X roofline",
+        "value": decode["value"], "unit": "GB/s", "n_gpus": 1,
+        "steps": arguments.steps, "warmup": arguments.warmup,
+        "ms_per_step": decode["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "decode GEMV M=1, Llama-7B layer shapes "
+                        "(q/k/v/o 4096x4096, gate/up 11008x4096, down "
+                        "4096x11008), NF4 block 64, fp32 absmax scales, "
+                        "%d layers x 7 projections per step" % arguments.layers,
+            "layers": arguments.layers,
+            "bytes_per_step": decode["bytes_per_step"],
+            "launches_per_step": decode["launches_per_step"],
+            "launch": "per-kernel" if arguments.no_graph else "hip-graph",
+            "device": library.device_description(),
+        },
+        "roofline": decode["roofline"],
+    }
+    if not arguments.skip_extras:
+        line["gemm"] = bench_gemm(package, device, torch,
+                                  max(3, arguments.steps // 4))
+        line["small_batch"] = bench_small_batch(package, device, torch,
+                                                max(3, arguments.steps // 4))
+    if not arguments.skip_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -143,6 +143,14 @@ class Library:
                 f"{path} is missing: build it with "
                 "`make -C riftco-transformer_amd` (or __graft_entry__.build())")
         self.path = path
+        # PyTorch wheels bundle their own HIP runtime under the same SONAME.
+        # Loading torch first makes this library bind to that one runtime, so
+        # that torch's device pointers and streams are valid here; without
+        # torch the system runtime is used.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         self._lib = ctypes.CDLL(path)
         for name, (restype, argtypes) in _PROTOTYPES.items():
             function = getattr(self._lib, name)  # AttributeError if absent

@@ -58,19 +58,23 @@ __device__ __forceinline__ void load_codebook_to_lds(float* table) {
     }
 }
 
-// Block scale for scale index `block` of a double-quantised weight.
+// Block scale of a double-quantised weight.  Every operation below must round
+// on its own: the pragma keeps the compiler from contracting the multiply and
+// the add into one fused multiply-add, and plain operators are used because
+// only code written inside this scope is covered by it.  Division of fp32 is
+// correctly rounded in HIP by default.
 __device__ __forceinline__ float decode_double_quantized_scale(
     std::uint8_t scale_code, float second_level, float offset
 ) {
 #pragma clang fp contract(off)
     const int centered = static_cast<int>(scale_code) - 128;
-    const float factor = __fdiv_rn(static_cast<float>(centered), 127.0F);
-    const float delta = __fmul_rn(second_level, factor);
+    const float factor = static_cast<float>(centered) / 127.0F;
+    const float delta = second_level * factor;
     constexpr float kMaxFinite = 0x1.fffffep+127F;
-    if (delta > 0.0F && offset > __fsub_rn(kMaxFinite, delta)) {
+    if (delta > 0.0F && offset > kMaxFinite - delta) {
         return kMaxFinite;
     }
-    const float reconstructed = __fadd_rn(offset, delta);
+    const float reconstructed = offset + delta;
     return reconstructed > 0.0F ? reconstructed : 0.0F;
 }
 

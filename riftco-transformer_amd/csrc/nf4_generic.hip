@@ -82,12 +82,26 @@ __global__ __launch_bounds__(256) void generic_input_backward_kernel(
         const std::size_t row = index / input_width;
         const std::size_t column = index % input_width;
         const float* upstream = dy + row * output_width;
-        float total = 0.0F;
-        for (std::size_t o = 0; o < output_width; ++o) {
-            total += upstream[o] *
-                     decode_weight_any(weight, block_shift,
-                                       o * input_width + column);
+        // Eight interleaved partial sums: shorter rounding walks than one
+        // long chain, and independent multiply-adds in flight.
+        float partial[8] = {0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F};
+        std::size_t o = 0;
+        for (; o + 8 <= output_width; o += 8) {
+#pragma unroll
+            for (int lane = 0; lane < 8; ++lane) {
+                partial[lane] += upstream[o + lane] *
+                    decode_weight_any(weight, block_shift,
+                                      (o + lane) * input_width + column);
+            }
         }
+        for (; o < output_width; ++o) {
+            partial[o % 8] += upstream[o] *
+                decode_weight_any(weight, block_shift,
+                                  o * input_width + column);
+        }
+        const float total =
+            ((partial[0] + partial[1]) + (partial[2] + partial[3])) +
+            ((partial[4] + partial[5]) + (partial[6] + partial[7]));
         dx[index] = total;
     }
 }

@@ -40,6 +40,7 @@ constexpr int kTileN = 128;       // output columns per workgroup
 constexpr int kTileK = 32;        // contraction per step
 constexpr int kStride = 36;       // padded LDS row stride in floats
 constexpr int kChunk = 16;        // weights decoded per thread per step
+constexpr unsigned kFlushSteps = 8;  // steps per first-level accumulation
 
 struct GemmShape {
     unsigned rows;         // M
@@ -196,7 +197,13 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
     const unsigned row0 = blockIdx.y * kTileM;
     const unsigned col0 = blockIdx.x * kTileN;
 
+    // Two-level accumulation: the matrix cores add into `acc` for
+    // kFlushSteps steps (256 contraction values), then `acc` is folded into
+    // `total` and cleared.  One long fp32 chain over K = 11008 drifts about as
+    // far as the CPU's sequential sum (~1e-5 of an output's standard
+    // deviation); chains of 256 stay an order of magnitude below that.
     floatx16 acc[2][2];
+    floatx16 total[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -204,9 +211,11 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 acc[i][j][e] = 0.0F;
+                total[i][j][e] = 0.0F;
             }
         }
     }
+    unsigned steps_since_flush = 0;
 
     Staged staged;
     load_activation_tile(staged, activations, shape, row0, 0);
@@ -269,6 +278,31 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
                 }
             }
         }
+
+        if (++steps_since_flush == kFlushSteps) {
+            steps_since_flush = 0;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        total[i][j][e] += acc[i][j][e];
+                        acc[i][j][e] = 0.0F;
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                total[i][j][e] += acc[i][j][e];
+            }
+        }
     }
 
     // Accumulator element e of lane l is output row 8*(e/4) + 4*(l/32) + e%4,
@@ -293,7 +327,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
                                      8 * (e / 4) + 4 * (lane / 32) + e % 4;
                 if (row < shape.rows) {
                     result[static_cast<std::size_t>(row) * shape.columns +
-                           column] = acc[i][j][e] + addend;
+                           column] = total[i][j][e] + addend;
                 }
             }
         }

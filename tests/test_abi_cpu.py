@@ -1,0 +1,84 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol that
+include/rthip.h declares, validates arguments, and reports 'unavailable'
+instead of computing anything when no device is present."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "rthip.h")
+
+
+def declared_symbols():
+    with open(HEADER) as handle:
+        text = handle.read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rthip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(package, library):
+    raw = ctypes.CDLL(package.LIBRARY_PATH)
+    declared = declared_symbols()
+    assert len(declared) >= 16
+    for name in declared:
+        assert hasattr(raw, name), f"{name} is declared but not exported"
+    # and the Python prototypes cover exactly the declared set
+    assert sorted(package.EXPORTED_SYMBOLS) == declared
+
+
+def test_abi_version(package, library):
+    assert library.abi_version() == (1, 0)
+
+
+def test_select_algorithm_is_pure_host_logic(package, library):
+    select = library.select_algorithm
+    fwd, bwd = package.FORWARD, package.INPUT_BACKWARD
+    # decode shapes -> streaming GEMV
+    assert select(fwd, 1, 4096, 4096, 64) == package.ALGORITHM_GEMV
+    assert select(fwd, 1, 4096, 11008, 64) == package.ALGORITHM_GEMV
+    assert select(fwd, 1, 11008, 4096, 64) == package.ALGORITHM_GEMV
+    # prefill / training -> MFMA GEMM, both directions
+    assert select(fwd, 2048, 4096, 11008, 64) == package.ALGORITHM_MFMA
+    assert select(fwd, 16, 256, 768, 64) == package.ALGORITHM_MFMA
+    assert select(bwd, 2048, 4096, 11008, 64) == package.ALGORITHM_MFMA
+    assert select(bwd, 2048, 11008, 4096, 64) == package.ALGORITHM_MFMA
+    # the reference's edge layout -> shape-agnostic kernels
+    assert select(fwd, 2, 33, 33, 32) == package.ALGORITHM_GENERIC
+    assert select(bwd, 2, 33, 33, 32) == package.ALGORITHM_GENERIC
+
+
+def test_argument_validation_needs_no_device(package, library):
+    with pytest.raises(package.InvalidArgument):
+        library.select_algorithm(package.FORWARD, 0, 64, 64, 64)
+    with pytest.raises(package.InvalidArgument):
+        library.select_algorithm(package.FORWARD, 1, 64, 64, 48)
+    with pytest.raises(package.InvalidArgument):
+        library.select_algorithm(2, 1, 64, 64, 64)
+    assert "block size" in library.last_error() or library.last_error()
+
+
+def test_reports_unavailable_without_a_device(package, library):
+    if library.is_available():
+        pytest.skip("a device is present")
+    with pytest.raises(package.Unavailable) as error:
+        library.device_count()
+    assert "device" in error.value.message
+    with pytest.raises(package.Unavailable):
+        library.malloc(64)
+    # a compute call is refused before anything is launched
+    weight = package.DeviceWeight(
+        64, 64, 64, package.SCALE_FLOAT32, _Fake(0x1000), _Fake(0x2000), None)
+    with pytest.raises(package.Unavailable):
+        library.linear_forward(0x3000, weight, None, 0x4000, 1)
+
+
+class _Fake:
+    """Stands in for a tensor: only its address is ever passed on."""
+
+    def __init__(self, address):
+        self._address = address
+
+    def data_ptr(self):
+        return self._address

@@ -1,0 +1,378 @@
+"""Parity of the HIP kernels with the CPU oracle, through the C ABI, on a real
+MI355X.
+
+The bar:
+  * nibble unpack, codebook lookup, scale decode, deq(W): bit-exact;
+  * y and dx: the reference's own |a-e| <= 3e-5*max(1,|a|,|e|) on its small
+    fixtures, and on transformer-sized layers
+        max|gpu - exact| / (sqrt(K) * rms(act) * rms(deq W)) <= 1e-5
+    against an fp64 accumulation over the bit-exact dequantised weights, plus
+        max|gpu - cpu|   / (sqrt(K) * rms(act) * rms(deq W))
+            <= 1e-5 + (the same measure of cpu against fp64)
+    for the oracle's sequential fp32 sums, whose own rounding walk reaches
+    ~1.2e-5 at K = 11008.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import helpers
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+TOLERANCE = 1.0e-5
+
+
+def upload(gpu, weight):
+    return gpu.upload_weight(
+        weight.output_width, weight.input_width, weight.block_size,
+        weight.codes, fp32_scales=weight.fp32_scales,
+        scale_codes=weight.scale_codes, second_level=weight.second_level,
+        second_level_block=weight.second_level_block, offset=weight.offset)
+
+
+def to_device(array):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(array)).cuda()
+
+
+def host(tensor):
+    import torch
+    torch.cuda.synchronize()
+    return tensor.cpu().numpy()
+
+
+def families(package):
+    """AUTO plus every pinned kernel family; a family that does not accept a
+    shape answers RTHIP_UNSUPPORTED and is skipped by `run`."""
+    return (None, package.ALGORITHM_GENERIC, package.ALGORITHM_GEMV,
+            package.ALGORITHM_MFMA)
+
+
+def run(package, function, *args, algorithm):
+    """One launch with the family pinned; None when it refuses the shape."""
+    try:
+        return host(function(*args, algorithm=algorithm))
+    except package.Unsupported:
+        assert algorithm is not None, "AUTO must accept every shape"
+        return None
+
+
+def check_layer(gpu, package, library, oracle, weight, x, dy, bias=None,
+                oracle_rows=None):
+    """Both products of one layer, every applicable kernel family."""
+    device_weight = upload(gpu, weight)
+    dense = oracle.dequantize(weight)
+    helpers.assert_bit_equal(host(gpu.dequantize(device_weight)), dense,
+                             "deq(W) on the GPU")
+    weight_rms = helpers.rms(dense)
+    rows = x.shape[0]
+    sample = slice(0, rows if oracle_rows is None else oracle_rows)
+
+    exact = helpers.exact_forward(x, dense)
+    if bias is not None:
+        exact = exact + bias.astype(np.float64)[None, :]
+    cpu = oracle.forward(x[sample], weight, bias)
+    cpu_error = helpers.normalized_error(
+        cpu, exact[sample], weight.input_width, helpers.rms(x), weight_rms)
+    x_device = to_device(x)
+    bias_device = None if bias is None else to_device(bias)
+    for family in families(package):
+        y = run(package, gpu.linear_forward, x_device, device_weight,
+                bias_device, algorithm=family)
+        if y is None:
+            continue
+        name = package.ALGORITHM_NAMES[family or 0]
+        error = helpers.normalized_error(
+            y, exact, weight.input_width, helpers.rms(x), weight_rms)
+        assert error <= TOLERANCE, f"forward/{name} vs fp64: {error:.3g}"
+        drift = helpers.normalized_error(
+            y[sample], cpu, weight.input_width, helpers.rms(x), weight_rms)
+        assert drift <= TOLERANCE + cpu_error, \
+            f"forward/{name} vs CPU oracle: {drift:.3g} (cpu {cpu_error:.3g})"
+
+    exact = helpers.exact_input_backward(dy, dense)
+    cpu = oracle.input_backward(dy[sample], weight)
+    cpu_error = helpers.normalized_error(
+        cpu, exact[sample], weight.output_width, helpers.rms(dy), weight_rms)
+    dy_device = to_device(dy)
+    for family in families(package):
+        dx = run(package, gpu.linear_input_backward, dy_device,
+                 device_weight, algorithm=family)
+        if dx is None:
+            continue
+        name = package.ALGORITHM_NAMES[family or 0]
+        error = helpers.normalized_error(
+            dx, exact, weight.output_width, helpers.rms(dy), weight_rms)
+        assert error <= TOLERANCE, f"backward/{name} vs fp64: {error:.3g}"
+        drift = helpers.normalized_error(
+            dx[sample], cpu, weight.output_width, helpers.rms(dy), weight_rms)
+        assert drift <= TOLERANCE + cpu_error, \
+            f"backward/{name} vs CPU oracle: {drift:.3g} (cpu {cpu_error:.3g})"
+
+
+# ---- the reference's own fixtures ------------------------------------------
+
+CLOSED_FORM = {
+    "aligned": (helpers.aligned_weight, helpers.aligned_input,
+                helpers.aligned_upstream),
+    "edge": (helpers.edge_weight, helpers.edge_input, helpers.edge_upstream),
+}
+
+
+@pytest.mark.parametrize("name", ["aligned", "edge"])
+@pytest.mark.parametrize("double_quantized", [False, True])
+def test_reference_fixtures(gpu, package, library, oracle, name,
+                            double_quantized):
+    """Counterpart of run_accelerator_oracle
+    (tests/core/backend/test_quantized_linear_backend.cpp:382-453): aligned
+    [3 x 32] and edge [33 x 33] layouts, block 32, both scale encodings,
+    against the golden outputs of the compiled reference at its tolerance."""
+    golden = np.load(os.path.join(GOLDEN, "closed_form.npz"))
+    make_weight, make_input, make_upstream = CLOSED_FORM[name]
+    tag = f"{name}_{'dq' if double_quantized else 'fp32'}"
+    weight = oracle.quantize(make_weight(), 32, double_quantized, 32)
+    device_weight = upload(gpu, weight)
+    helpers.assert_bit_equal(host(gpu.dequantize(device_weight)),
+                             golden[f"{tag}_dequantized"], "deq(W)")
+    x, dy = make_input(), make_upstream()
+    for family in families(package):
+        y = run(package, gpu.linear_forward, to_device(x), device_weight,
+                algorithm=family)
+        assert y is None or \
+            helpers.reference_close(y, golden[f"{tag}_forward"])
+        dx = run(package, gpu.linear_input_backward, to_device(dy),
+                 device_weight, algorithm=family)
+        assert dx is None or \
+            helpers.reference_close(dx, golden[f"{tag}_input_backward"])
+
+
+@pytest.mark.parametrize("double_quantized", [False, True])
+def test_config1_tiny_layer_with_bias(gpu, package, library, oracle,
+                                      double_quantized):
+    """BASELINE config 1 against the compiled reference's stored outputs."""
+    golden = np.load(os.path.join(GOLDEN, "config1.npz"))
+    x = helpers.normal(1, (16, 256), 1.0)
+    dense = helpers.normal(2, (768, 256), 0.02)
+    bias = helpers.normal(3, (768,), 0.01)
+    dy = helpers.normal(4, (16, 768), 1.0e-2)
+    tag = "dq" if double_quantized else "fp32"
+    weight = oracle.quantize(dense, 64, double_quantized, 256)
+    device_weight = upload(gpu, weight)
+    y = host(gpu.linear_forward(to_device(x), device_weight, to_device(bias)))
+    assert helpers.reference_close(y, golden[f"{tag}_forward_bias"])
+    dx = host(gpu.linear_input_backward(to_device(dy), device_weight))
+    assert helpers.reference_close(dx, golden[f"{tag}_input_backward"])
+    check_layer(gpu, package, library, oracle, weight, x, dy, bias)
+
+
+# ---- transformer-sized layers --------------------------------------------
+
+@pytest.mark.parametrize("name,out_w,in_w,seed", [
+    ("q_proj", 4096, 4096, 11),
+    ("gate_proj", 11008, 4096, 12),
+    ("down_proj", 4096, 11008, 13),
+])
+@pytest.mark.parametrize("double_quantized", [False, True])
+def test_llama_rows_against_golden(gpu, package, library, oracle, name,
+                                   out_w, in_w, seed, double_quantized):
+    """One row (the decode GEMV) through each distinct Llama-7B projection:
+    deq(W) digest and outputs against the compiled reference's vectors."""
+    golden = np.load(os.path.join(GOLDEN, "llama_rows.npz"))
+    with open(os.path.join(GOLDEN, "digests.json")) as handle:
+        meta = json.load(handle)["llama"][name]
+    tag = "dq" if double_quantized else "fp32"
+    dense = helpers.normal(seed, (out_w, in_w), 0.02)
+    x = helpers.normal(seed + 100, (1, in_w), 1.0)
+    dy = helpers.normal(seed + 200, (1, out_w), 1.0e-2)
+    weight = oracle.quantize(dense, 64, double_quantized, 256)
+    device_weight = upload(gpu, weight)
+    assert device_weight.payload_bytes == meta[tag]["payload_bytes"]
+    deq = host(gpu.dequantize(device_weight))
+    assert helpers.sha256(deq) == meta[tag]["dequantized_sha256"]
+    weight_rms = helpers.rms(deq)
+    y = host(gpu.linear_forward(to_device(x), device_weight))
+    expected = golden[f"{name}_{tag}_forward"]
+    exact = helpers.exact_forward(x, deq)
+    own = helpers.normalized_error(expected, exact, in_w, helpers.rms(x),
+                                   weight_rms)
+    assert helpers.normalized_error(y, exact, in_w, helpers.rms(x),
+                                    weight_rms) <= TOLERANCE
+    assert helpers.normalized_error(y, expected, in_w, helpers.rms(x),
+                                    weight_rms) <= TOLERANCE + own
+    dx = host(gpu.linear_input_backward(to_device(dy), device_weight))
+    expected = golden[f"{name}_{tag}_input_backward"]
+    exact = helpers.exact_input_backward(dy, deq)
+    own = helpers.normalized_error(expected, exact, out_w, helpers.rms(dy),
+                                   weight_rms)
+    assert helpers.normalized_error(dx, exact, out_w, helpers.rms(dy),
+                                    weight_rms) <= TOLERANCE
+    assert helpers.normalized_error(dx, expected, out_w, helpers.rms(dy),
+                                    weight_rms) <= TOLERANCE + own
+
+
+@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 16, 64, 130])
+@pytest.mark.parametrize("double_quantized", [False, True])
+def test_row_counts_across_the_gemv_mfma_crossover(
+        gpu, package, library, oracle, rows, double_quantized):
+    dense = helpers.normal(50, (1024, 2048), 0.02)
+    weight = oracle.quantize(dense, 64, double_quantized, 256)
+    x = helpers.normal(51 + rows, (rows, 2048), 1.0)
+    dy = helpers.normal(52 + rows, (rows, 1024), 1.0e-2)
+    check_layer(gpu, package, library, oracle, weight, x, dy)
+
+
+@pytest.mark.parametrize("out_w,in_w,block,second", [
+    (96, 160, 32, 32),      # narrow rows, tiles mostly empty
+    (200, 352, 32, 64),     # output width not a multiple of the tile
+    (128, 4096, 4096, 32),  # one block per row
+    (64, 96, 64, 32),       # blocks straddle rows (96 % 64 != 0)
+    (32, 11008, 128, 256),
+    (136, 48, 32, 32),      # row width a multiple of 16 only
+    (40, 50, 32, 32),       # nothing aligned
+])
+@pytest.mark.parametrize("double_quantized", [False, True])
+def test_ragged_shapes_and_block_sizes(gpu, package, library, oracle, out_w,
+                                       in_w, block, second, double_quantized):
+    dense = helpers.normal(60, (out_w, in_w), 0.05)
+    dense[::3, ::5] = 0.0
+    weight = oracle.quantize(dense, block, double_quantized, second)
+    for rows in (1, 3, 37):
+        x = helpers.normal(61 + rows, (rows, in_w), 1.0)
+        dy = helpers.normal(62 + rows, (rows, out_w), 1.0e-2)
+        check_layer(gpu, package, library, oracle, weight, x, dy)
+
+
+def test_zero_scale_blocks_and_saturated_scales(gpu, package, library,
+                                                oracle):
+    dense = helpers.normal(70, (64, 128), 0.02)
+    dense[5] = 0.0          # zero blocks: scale 0, code 7
+    dense[9, :64] = 0.0
+    for dq in (False, True):
+        weight = oracle.quantize(dense, 64, dq, 32)
+        x = helpers.normal(71, (4, 128), 1.0)
+        dy = helpers.normal(72, (4, 64), 1.0e-2)
+        check_layer(gpu, package, library, oracle, weight, x, dy)
+
+
+# ---- full-size properties -----------------------------------------------
+
+@pytest.mark.parametrize("out_w,in_w,double_quantized", [
+    (11008, 4096, False), (11008, 4096, True), (4096, 4096, True),
+    (4096, 11008, True)])
+def test_prefill_shapes_at_full_size(gpu, package, library, oracle, out_w,
+                                     in_w, double_quantized):
+    """M = 2048 at BASELINE's shapes.  Size-independent checks: every output
+    against an fp64 product over the bit-exact deq(W) (computed on the device
+    by the vendor BLAS, an independent path), 32 seeded rows against the CPU
+    oracle, and linearity y(a*x1 + x2) = a*y(x1) + y(x2) for a power of two."""
+    import torch
+    rows = 2048
+    dense = helpers.normal(80, (out_w, in_w), 0.02)
+    weight = oracle.quantize(dense, 64, double_quantized, 256)
+    device_weight = upload(gpu, weight)
+    deq = gpu.dequantize(device_weight)
+    helpers.assert_bit_equal(host(deq), oracle.dequantize(weight), "deq(W)")
+    weight_rms = helpers.rms(host(deq))
+    picked = np.sort(np.random.default_rng(81).choice(rows, 32, replace=False))
+
+    x = helpers.normal(82, (rows, in_w), 1.0)
+    x_device = to_device(x)
+    y = gpu.linear_forward(x_device, device_weight)
+    exact = (x_device.double() @ deq.double().T)
+    scale = np.sqrt(in_w) * helpers.rms(x) * weight_rms
+    error = float((y.double() - exact).abs().max()) / scale
+    assert error <= TOLERANCE, f"forward vs fp64: {error:.3g}"
+    cpu = oracle.forward(x[picked], weight)
+    cpu_error = helpers.normalized_error(
+        cpu, host(exact)[picked], in_w, helpers.rms(x), weight_rms)
+    drift = helpers.normalized_error(host(y)[picked], cpu, in_w,
+                                     helpers.rms(x), weight_rms)
+    assert drift <= TOLERANCE + cpu_error
+    y2 = gpu.linear_forward(x_device * 4.0, device_weight)
+    assert torch.equal(y2, y * 4.0), "scaling x by 4 must scale y exactly"
+    del exact, y2
+
+    dy = helpers.normal(83, (rows, out_w), 1.0e-2)
+    dy_device = to_device(dy)
+    dx = gpu.linear_input_backward(dy_device, device_weight)
+    exact = (dy_device.double() @ deq.double())
+    scale = np.sqrt(out_w) * helpers.rms(dy) * weight_rms
+    error = float((dx.double() - exact).abs().max()) / scale
+    assert error <= TOLERANCE, f"backward vs fp64: {error:.3g}"
+    cpu = oracle.input_backward(dy[picked], weight)
+    cpu_error = helpers.normalized_error(
+        cpu, host(exact)[picked], out_w, helpers.rms(dy), weight_rms)
+    drift = helpers.normalized_error(host(dx)[picked], cpu, out_w,
+                                     helpers.rms(dy), weight_rms)
+    assert drift <= TOLERANCE + cpu_error
+    # <dy, y(x)> == <dx(dy), x>: the two kernels are adjoint to each other
+    lhs = float((dy_device.double() * y.double()).sum())
+    rhs = float((dx.double() * x_device.double()).sum())
+    assert abs(lhs - rhs) <= 1e-6 * max(abs(lhs), abs(rhs), 1.0)
+
+
+def test_decode_shapes_small_batches(gpu, package, library, oracle):
+    """M in {1, 4, 16, 64} on the three distinct Llama-7B shapes."""
+    for name, (out_w, in_w) in (("q_proj", (4096, 4096)),
+                                ("gate_proj", (11008, 4096)),
+                                ("down_proj", (4096, 11008))):
+        dense = helpers.normal(90, (out_w, in_w), 0.02)
+        weight = oracle.quantize(dense, 64)
+        for rows in (1, 4, 16, 64):
+            x = helpers.normal(91 + rows, (rows, in_w), 1.0)
+            dy = helpers.normal(92 + rows, (rows, out_w), 1.0e-2)
+            check_layer(gpu, package, library, oracle, weight, x, dy,
+                        oracle_rows=min(rows, 4))
+
+
+# ---- the ABI's error behaviour on a live device --------------------------
+
+def test_abi_rejects_bad_arguments(gpu, package, library, oracle):
+    import torch
+    weight = oracle.quantize(helpers.normal(95, (64, 64), 0.02), 64)
+    device_weight = upload(gpu, weight)
+    x = torch.zeros(64, device="cuda")
+    y = torch.zeros(64, device="cuda")
+    with pytest.raises(package.InvalidArgument):
+        library.linear_forward(x.data_ptr(), device_weight, None,
+                               x.data_ptr(), 1)           # aliasing
+    with pytest.raises(package.InvalidArgument):
+        library.linear_forward(0, device_weight, None, y.data_ptr(), 1)
+    with pytest.raises(package.InvalidArgument):
+        library.linear_forward(x.data_ptr(), device_weight, None,
+                               y.data_ptr(), 0)           # zero rows
+    bad = package.DeviceWeight(64, 64, 48, 0, device_weight.codes,
+                               device_weight.primary_scales, None)
+    with pytest.raises(package.InvalidArgument):
+        library.linear_forward(x.data_ptr(), bad, None, y.data_ptr(), 1)
+    with pytest.raises(package.Unsupported):
+        library.linear_input_backward(x.data_ptr(), device_weight,
+                                      y.data_ptr(), 1,
+                                      algorithm=package.ALGORITHM_GEMV)
+    odd = oracle.quantize(helpers.normal(96, (3, 33), 0.02), 32)
+    with pytest.raises(package.Unsupported):
+        library.linear_forward(x.data_ptr(), upload(gpu, odd), None,
+                               y.data_ptr(), 1,
+                               algorithm=package.ALGORITHM_MFMA)
+
+
+def test_memory_entry_points(gpu, package, library):
+    import torch
+    pointer = library.malloc(4096)
+    assert pointer % 256 == 0
+    source = np.arange(1024, dtype=np.float32)
+    library.copy_to_device(pointer, source.ctypes.data, 4096)
+    back = np.zeros(1024, dtype=np.float32)
+    library.copy_to_host(back.ctypes.data, pointer, 4096)
+    assert np.array_equal(source, back)
+    library.fill_f32(pointer, 2.5, 1024)
+    library.synchronize()
+    library.copy_to_host(back.ctypes.data, pointer, 4096)
+    assert np.all(back == 2.5)
+    library.free(pointer)
+    assert "MI355X" in library.device_description() or \
+        "gfx950" in library.device_description()
