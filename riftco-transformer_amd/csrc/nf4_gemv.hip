@@ -5,20 +5,44 @@
 // HBM-bound case, where the only traffic that matters is the packed codes and
 // their scales, each read exactly once.
 //
-// Work split.  A workgroup of four wavefronts owns kRows consecutive weight
-// rows.  The contraction axis is cut into 16-weight segments (8 bytes of
-// codes); thread t owns segments t, t + 256, ... of EVERY row, so
+// Work split.  One persistent workgroup per CU holds kTeams teams of four
+// wavefronts.  A team owns batches of kRows consecutive weight rows; the
+// contraction axis is cut into 16-weight segments (8 bytes of codes) and thread
+// t of a team owns segments t, t + 256, ... of EVERY row, so
 //   * a wavefront's loads of one row are 512 contiguous bytes,
 //   * the x values a thread needs never change: they are loaded once into
-//     registers and reused for all rows (x costs no LDS or cache bandwidth in
-//     the row loop),
+//     registers and reused for all rows,
 //   * a segment lies inside one quantisation block (block sizes are powers of
 //     two >= 32 and the row width is a multiple of 16), so a thread applies
 //     one scale per segment:  acc += scale * sum_i x_i * codebook[c_i].
-// All loads of a workgroup's rows are issued before the first use, which
-// keeps ~32 KB per CU in flight.  Nibble -> fp32 goes through a 16-entry LDS
-// table (conflict-free by construction).  Row sums are reduced across the
-// wavefront with shuffles and across the four wavefronts through LDS.
+// The loads of batch b + 1 are issued before batch b is computed, and the
+// wavefronts never wait for each other inside the loop, so HBM requests are in
+// flight for the whole life of the workgroup.
+//
+// Decode.  Nibble -> fp32 is a table lookup, and the LDS (128 B per clock per
+// CU) is the unit that bounds this kernel once the loads stream: 4 bytes of
+// table per weight.  Nibbles are therefore decoded two at a time -- a code BYTE
+// indexes a table of (codebook[low nibble], codebook[high nibble]) pairs, one
+// ds_read_b64 per two weights -- and everything else is kept off the LDS.
+// The table is stored entry-major with 16 interleaved replicas: replica k of
+// entry e sits at byte e * 256 + k * 8, and lane l reads replica l % 16.  The 16
+// lanes the LDS serves per clock therefore always touch 16 different bank pairs
+// whatever their codes are, and an entry's address is
+// (byte << 8) | ((l % 16) << 3): ONE v_perm_b32 that drops the code byte into
+// bits 8..15 above the lane's fixed low byte.  The table is built from
+// instruction literals while the first loads are in flight.
+//
+// Weight bytes and scales are fetched with buffer loads: the address is a
+// per-lane constant offset plus a per-row SCALAR offset, so stepping to the next
+// row costs no vector arithmetic, and the hardware range check turns reads past
+// the end of the payload into zeros.  Nothing branches on data or on bounds:
+// segments past the row end carry x = 0 and rows past the output width are
+// computed on whatever was read and never written.
+//
+// Reduction.  Row sums are reduced inside each 16-lane DPP row with a transposed
+// butterfly of DPP moves (vector ALU only, no LDS round trips); the 16 row
+// partials per team and batch are parked in LDS, and after ONE barrier at the
+// end of the kernel the team adds them up and writes y.
 
 #include "kernels.hpp"
 #include "nf4_decode.hpp"
@@ -26,166 +50,452 @@
 namespace rthip {
 namespace {
 
-constexpr int kThreads = 256;
 constexpr int kWave = 64;
-constexpr int kWaves = kThreads / kWave;
-constexpr int kSegment = 16;  // weights per thread per row visit
+constexpr int kTeamThreads = 256;  // threads that share one weight row
+constexpr int kSegment = 16;       // weights per thread per row visit
+constexpr int kReplicas = 16;      // interleaved copies of the pair table
+constexpr int kEntryStride = 256;  // bytes between table entries
+constexpr int kRowLanes = 16;      // lanes of one DPP row
+constexpr int kTeamDppRows = kTeamThreads / kRowLanes;
+constexpr unsigned kComputeUnits = 256;
+constexpr unsigned kMaxIterations = 8;  // batches per team kept in LDS
+#ifndef RTHIP_GEMV_TEAMS
+#define RTHIP_GEMV_TEAMS 2
+#endif
+#ifndef RTHIP_GEMV_ROWS
+#define RTHIP_GEMV_ROWS 4
+#endif
 
-__device__ __forceinline__ float wave_sum(float value) {
-#pragma unroll
-    for (int offset = kWave / 2; offset > 0; offset >>= 1) {
-        value += __shfl_xor(value, offset, kWave);
-    }
-    return value;
+// codebook[n] selected with compare/select on instruction literals (no memory
+// access, so it cannot stall behind the streaming loads).
+__device__ __forceinline__ float codebook_literal(unsigned n) {
+    const float lo0 = (n & 1U) ? -0.6961928009986877F : -1.0F;
+    const float lo1 = (n & 1U) ? -0.39491748809814453F : -0.5250730514526367F;
+    const float lo2 = (n & 1U) ? -0.18477343022823334F : -0.28444138169288635F;
+    const float lo3 = (n & 1U) ? 0.0F : -0.09105003625154495F;
+    const float hi0 = (n & 1U) ? 0.16093020141124725F : 0.07958029955625534F;
+    const float hi1 = (n & 1U) ? 0.33791524171829224F : 0.24611230194568634F;
+    const float hi2 = (n & 1U) ? 0.5626170039176941F : 0.44070982933044434F;
+    const float hi3 = (n & 1U) ? 1.0F : 0.7229568362236023F;
+    const float a = (n & 2U) ? lo1 : lo0;
+    const float b = (n & 2U) ? lo3 : lo2;
+    const float c = (n & 2U) ? hi1 : hi0;
+    const float d = (n & 2U) ? hi3 : hi2;
+    const float low = (n & 4U) ? b : a;
+    const float high = (n & 4U) ? d : c;
+    return (n & 8U) ? high : low;
 }
 
-template <int kX, int kSegments, int kRows, bool kDoubleQuantized>
-__global__ __launch_bounds__(kThreads) void gemv_forward_kernel(
-    const float* __restrict__ x, Nf4WeightView weight,
-    const float* __restrict__ bias, float* __restrict__ y,
-    unsigned input_width, unsigned output_width, unsigned block_shift
-) {
-    __shared__ float table[16];
-    __shared__ float partial[kWaves][kRows][kX];
-    load_codebook_to_lds(table);
+// Level of nibble 4 * quarter + i (i is a compile-time constant).
+template <int kIndex>
+__device__ __forceinline__ float level_in_quarter(unsigned quarter) {
+    constexpr float kLevels[16] = {
+        -1.0F, -0.6961928009986877F, -0.5250730514526367F,
+        -0.39491748809814453F, -0.28444138169288635F, -0.18477343022823334F,
+        -0.09105003625154495F, 0.0F, 0.07958029955625534F,
+        0.16093020141124725F, 0.24611230194568634F, 0.33791524171829224F,
+        0.44070982933044434F, 0.5626170039176941F, 0.7229568362236023F, 1.0F};
+    const float low = (quarter & 1U) ? kLevels[4 + kIndex] : kLevels[kIndex];
+    const float high =
+        (quarter & 1U) ? kLevels[12 + kIndex] : kLevels[8 + kIndex];
+    return (quarter & 2U) ? high : low;
+}
 
-    const unsigned thread = threadIdx.x;
+// Builds the replicated pair table with all kThreads threads of the
+// workgroup.  A thread fills one replica of 4096 / kThreads consecutive
+// entries, in groups of four that share a high nibble and a low-nibble
+// quarter.
+template <int kThreads>
+__device__ __forceinline__ void build_pair_table(char* table) {
+    constexpr int kEntries = 256 * kReplicas / kThreads;  // per thread
+    static_assert(kEntries >= 4 && kEntries % 4 == 0);
+    const unsigned replica = threadIdx.x % kReplicas;
+    const unsigned first_entry = (threadIdx.x / kReplicas) * kEntries;
+    char* slot = table + replica * sizeof(float2);
+#pragma unroll
+    for (int group = 0; group < kEntries / 4; ++group) {
+        const unsigned entry = first_entry + 4 * group;
+        const float high_level = codebook_literal(entry >> 4);
+        const unsigned quarter = (entry >> 2) & 3U;
+        float2* target =
+            reinterpret_cast<float2*>(slot + entry * kEntryStride);
+        constexpr int kStep = kEntryStride / sizeof(float2);
+        target[0 * kStep] =
+            make_float2(level_in_quarter<0>(quarter), high_level);
+        target[1 * kStep] =
+            make_float2(level_in_quarter<1>(quarter), high_level);
+        target[2 * kStep] =
+            make_float2(level_in_quarter<2>(quarter), high_level);
+        target[3 * kStep] =
+            make_float2(level_in_quarter<3>(quarter), high_level);
+    }
+}
+
+// value of lane (l ^ kXor) within the 16-lane DPP row, vector ALU only.
+template <int kXor>
+__device__ __forceinline__ float dpp_xor(float value) {
+    const int bits = __builtin_bit_cast(int, value);
+    int moved;
+    if constexpr (kXor == 1) {
+        moved = __builtin_amdgcn_update_dpp(0, bits, 0xB1, 0xF, 0xF, false);
+    } else if constexpr (kXor == 2) {
+        moved = __builtin_amdgcn_update_dpp(0, bits, 0x4E, 0xF, 0xF, false);
+    } else if constexpr (kXor == 4) {
+        // lanes 0-3 and 8-11 read four lanes up, the others four lanes down
+        moved = __builtin_amdgcn_update_dpp(0, bits, 0x104, 0xF, 0x5, false);
+        moved =
+            __builtin_amdgcn_update_dpp(moved, bits, 0x114, 0xF, 0xA, false);
+    } else {
+        static_assert(kXor == 8);
+        moved = __builtin_amdgcn_update_dpp(0, bits, 0x128, 0xF, 0xF, false);
+    }
+    return __builtin_bit_cast(float, moved);
+}
+
+template <int kXor, int kHalf, int kValues>
+__device__ __forceinline__ void transposed_step(float (&values)[kValues],
+                                                unsigned lane) {
+    if constexpr (kHalf >= 1) {
+        // Lanes with bit kXor set keep the upper half of the values and hand
+        // the lower half to their partner, and vice versa.
+        const bool upper = (lane & kXor) != 0;
+#pragma unroll
+        for (int j = 0; j < kHalf; ++j) {
+            float low = values[j];
+            float high = values[j + kHalf];
+            // Keep the two operands as plain registers: without this the
+            // selects below are rewritten into a dynamically indexed read of
+            // `values`, which costs a compare/select chain over the array.
+            asm volatile("" : "+v"(low), "+v"(high));
+            const float keep = upper ? high : low;
+            const float send = upper ? low : high;
+            values[j] = keep + dpp_xor<kXor>(send);
+        }
+    } else {
+        values[0] += dpp_xor<kXor>(values[0]);
+    }
+}
+
+// Sum over each 16-lane DPP row of kValues per-lane values.  On return every
+// lane holds the row total of value `slot_of_lane(lane)`.
+template <int kValues>
+__device__ __forceinline__ float transposed_row_sum(float (&values)[kValues],
+                                                    unsigned lane) {
+    static_assert((kValues & (kValues - 1)) == 0 && kValues <= kRowLanes);
+    transposed_step<1, kValues / 2>(values, lane);
+    transposed_step<2, kValues / 4>(values, lane);
+    transposed_step<4, kValues / 8>(values, lane);
+    transposed_step<8, kValues / 16>(values, lane);
+    return values[0];
+}
+
+// Which value a lane ends up holding after transposed_row_sum: lane bit s
+// selected the upper half at step s.
+template <int kValues>
+__device__ __forceinline__ unsigned slot_of_lane(unsigned lane) {
+    unsigned slot = 0;
+    unsigned bit = 1;
+#pragma unroll
+    for (int half = kValues / 2; half >= 1; half /= 2) {
+        if (lane & bit) {
+            slot += half;
+        }
+        bit *= 2;
+    }
+    return slot;
+}
+
+typedef unsigned uint2_vec __attribute__((ext_vector_type(2)));
+
+template <int kRows, int kSegments>
+struct RowBatch {
+    uint2_vec codes[kRows][kSegments];
+    float scales[kRows][kSegments];
+};
+
+// Buffer descriptors of one packed weight; sizes are in bytes.
+struct GemvBuffers {
+    unsigned code_bytes;
+    unsigned primary_bytes;
+    unsigned secondary_bytes;
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base,
+                                                             unsigned bytes) {
+    // Raw (untyped, stride 0) buffer with range checking on `bytes`.
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0,
+                                             static_cast<int>(bytes),
+                                             0x00020000);
+}
+
+// kX: x rows held per thread (1, 2 or 4; a 3-row call runs as 4 with a zero
+// row).  kSegments: segments per thread.  kRows: weight rows per batch.
+// kTeams: teams per workgroup.
+template <int kX, int kSegments, int kRows, int kTeams, bool kDoubleQuantized>
+__global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
+    const float* __restrict__ x, Nf4WeightView weight, GemvBuffers sizes,
+    const float* __restrict__ bias, float* __restrict__ y, unsigned x_rows,
+    unsigned input_width, unsigned output_width, unsigned block_shift,
+    unsigned batch_count, unsigned iterations
+) {
+    constexpr int kThreads = kTeamThreads * kTeams;
+    constexpr int kValues = kRows * kX;
+    __shared__ __attribute__((aligned(256))) char table[256 * kEntryStride];
+    __shared__ float partial[kTeams][kMaxIterations][kTeamDppRows][kValues];
+
+    const unsigned team =
+        __builtin_amdgcn_readfirstlane(threadIdx.x / kTeamThreads);
+    const unsigned thread = threadIdx.x % kTeamThreads;  // within the team
+    const unsigned lane = thread % kWave;
     const unsigned segment_count = input_width / kSegment;
 
-    // This thread's slice of x, resident for the whole kernel.
+    const __amdgpu_buffer_rsrc_t code_buffer =
+        make_buffer(weight.codes, sizes.code_bytes);
+    const __amdgpu_buffer_rsrc_t primary_buffer =
+        make_buffer(weight.primary_scales, sizes.primary_bytes);
+    const __amdgpu_buffer_rsrc_t secondary_buffer =
+        make_buffer(weight.secondary_scales, sizes.secondary_bytes);
+
+    // Per-lane constants: where this thread's segments sit inside a row.  The
+    // row width is a multiple of the block size, so a row starts on a block
+    // boundary and (row block) + (segment block) is the flat block index.
+    unsigned segment_weights[kSegments];
+#pragma unroll
+    for (int j = 0; j < kSegments; ++j) {
+        segment_weights[j] = (thread + kTeamThreads * j) * kSegment;
+    }
+
+    // All indices fit 32 bits (the launcher checks O * I < 2^32).
+    const auto load_batch = [&](RowBatch<kRows, kSegments>& batch,
+                                unsigned batch_index) {
+#pragma unroll
+        for (int row = 0; row < kRows; ++row) {
+            const unsigned o = batch_index * kRows + row;  // scalar
+            const unsigned row_start = o * input_width;
+            const unsigned row_block = row_start >> block_shift;
+#pragma unroll
+            for (int j = 0; j < kSegments; ++j) {
+#ifdef RTHIP_GEMV_DEBUG_NOLOAD
+                batch.codes[row][j].x = thread * 2654435761u + row_start;
+                batch.codes[row][j].y = thread * 40503u + row_start;
+                batch.scales[row][j] = 1.0F;
+                continue;
+#endif
+                batch.codes[row][j] = __builtin_amdgcn_raw_buffer_load_b64(
+                    code_buffer, segment_weights[j] >> 1, row_start >> 1, 0);
+                const unsigned segment_block =
+                    segment_weights[j] >> block_shift;
+                if constexpr (!kDoubleQuantized) {
+                    batch.scales[row][j] = __builtin_bit_cast(
+                        float, __builtin_amdgcn_raw_buffer_load_b32(
+                                   primary_buffer, segment_block * 4,
+                                   row_block * 4, 0));
+                } else {
+                    const std::uint8_t scale_code =
+                        __builtin_amdgcn_raw_buffer_load_b8(
+                            primary_buffer, segment_block, row_block, 0);
+                    const unsigned group = (row_block + segment_block) >>
+                                           weight.second_level_shift;
+                    const float second = __builtin_bit_cast(
+                        float, __builtin_amdgcn_raw_buffer_load_b32(
+                                   secondary_buffer, group * 4, 0, 0));
+                    batch.scales[row][j] = decode_double_quantized_scale(
+                        scale_code, second, weight.offset);
+                }
+            }
+        }
+    };
+
+    // Batches are dealt round-robin: iteration i of workgroup g, team t takes
+    // batch (i * gridDim.x + g) * kTeams + t.
+    const unsigned stride = gridDim.x * kTeams;
+    const unsigned first_batch = blockIdx.x * kTeams + team;
+
+    RowBatch<kRows, kSegments> ping;
+    RowBatch<kRows, kSegments> pong;
+    load_batch(ping, first_batch);
+
+    // This thread's slice of x, resident for the whole kernel.  Segments past
+    // the row end and rows past x_rows read as zero.
     float xs[kX][kSegments][kSegment];
 #pragma unroll
     for (int j = 0; j < kSegments; ++j) {
-        const unsigned segment = thread + kThreads * j;
-        const bool valid = segment < segment_count;
+        const bool segment_valid = thread + kTeamThreads * j < segment_count;
+        const unsigned clamped =
+            min(thread + kTeamThreads * j, segment_count - 1) * kSegment;
 #pragma unroll
         for (int r = 0; r < kX; ++r) {
+            const bool valid =
+                segment_valid && static_cast<unsigned>(r) < x_rows;
+            const unsigned source_row =
+                min(static_cast<unsigned>(r), x_rows - 1);
             const float4* source = reinterpret_cast<const float4*>(
-                x + static_cast<std::size_t>(r) * input_width +
-                static_cast<std::size_t>(segment) * kSegment);
+                x + source_row * input_width + clamped);
 #pragma unroll
             for (int q = 0; q < kSegment / 4; ++q) {
-                const float4 v =
-                    valid ? source[q] : make_float4(0.0F, 0.0F, 0.0F, 0.0F);
-                xs[r][j][4 * q + 0] = v.x;
-                xs[r][j][4 * q + 1] = v.y;
-                xs[r][j][4 * q + 2] = v.z;
-                xs[r][j][4 * q + 3] = v.w;
+                const float4 v = source[q];
+                xs[r][j][4 * q + 0] = valid ? v.x : 0.0F;
+                xs[r][j][4 * q + 1] = valid ? v.y : 0.0F;
+                xs[r][j][4 * q + 2] = valid ? v.z : 0.0F;
+                xs[r][j][4 * q + 3] = valid ? v.w : 0.0F;
             }
         }
     }
 
-    const unsigned first_row = blockIdx.x * kRows;
+    build_pair_table<kThreads>(table);
+    __syncthreads();
 
-    // Issue every load of this workgroup's rows before any use.
-    uint2 codes[kRows][kSegments];
-    float scales[kRows][kSegments];
-#pragma unroll
-    for (int row = 0; row < kRows; ++row) {
-        const unsigned o = first_row + row;
-#pragma unroll
-        for (int j = 0; j < kSegments; ++j) {
-            const unsigned segment = thread + kThreads * j;
-            const bool valid = segment < segment_count && o < output_width;
-            const std::size_t flat =
-                static_cast<std::size_t>(o) * input_width +
-                static_cast<std::size_t>(segment) * kSegment;
-            // An absent segment decodes to code 7 (0.0) with scale 0.
-            codes[row][j] = valid
-                ? *reinterpret_cast<const uint2*>(weight.codes + (flat >> 1))
-                : make_uint2(0x77777777U, 0x77777777U);
-            scales[row][j] = valid
-                ? load_block_scale<kDoubleQuantized>(weight,
-                                                     flat >> block_shift)
-                : 0.0F;
+    const unsigned lane_bits = (lane % kReplicas) * sizeof(float2);  // < 128
+    // v_perm_b32 selectors: (byte b of the code word) << 8 | lane_bits.
+    constexpr unsigned kSelect[4] = {0x0C0C0400U, 0x0C0C0500U, 0x0C0C0600U,
+                                     0x0C0C0700U};
+
+    // One batch: prefetch `next`, compute `current`, reduce, write.
+    const auto step = [&](const RowBatch<kRows, kSegments>& current,
+                          RowBatch<kRows, kSegments>& next,
+                          unsigned iteration) {
+        const unsigned batch_index = first_batch + iteration * stride;
+        if (iteration + 1 < iterations) {
+            load_batch(next, batch_index + stride);
         }
-    }
 
-    __syncthreads();  // codebook table visible
-
-    float acc[kRows][kX];
+        float acc[kValues];
 #pragma unroll
-    for (int row = 0; row < kRows; ++row) {
-#pragma unroll
-        for (int r = 0; r < kX; ++r) {
-            acc[row][r] = 0.0F;
-        }
-#pragma unroll
-        for (int j = 0; j < kSegments; ++j) {
-            float sums[kX];
+        for (int row = 0; row < kRows; ++row) {
+            float row_acc[kX];
 #pragma unroll
             for (int r = 0; r < kX; ++r) {
-                sums[r] = 0.0F;
+                row_acc[r] = 0.0F;
             }
-            const unsigned words[2] = {codes[row][j].x, codes[row][j].y};
 #pragma unroll
-            for (int w = 0; w < 2; ++w) {
+            for (int j = 0; j < kSegments; ++j) {
+                float even[kX];
+                float odd[kX];
 #pragma unroll
-                for (int n = 0; n < 8; ++n) {
-                    const float level = table[(words[w] >> (4 * n)) & 0xFU];
+                for (int r = 0; r < kX; ++r) {
+                    even[r] = 0.0F;
+                    odd[r] = 0.0F;
+                }
+                const unsigned words[2] = {current.codes[row][j].x,
+                                           current.codes[row][j].y};
+#ifdef RTHIP_GEMV_DEBUG_NOCOMPUTE
+                even[0] = __builtin_bit_cast(float, words[0] & 0x3FFFFFFFU);
+                odd[0] = __builtin_bit_cast(float, words[1] & 0x3FFFFFFFU);
+#else
 #pragma unroll
-                    for (int r = 0; r < kX; ++r) {
-                        sums[r] += xs[r][j][8 * w + n] * level;
+                for (int w = 0; w < 2; ++w) {
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        const unsigned address = __builtin_amdgcn_perm(
+                            words[w], lane_bits, kSelect[b]);
+                        const float2 levels =
+                            *reinterpret_cast<const float2*>(table + address);
+#pragma unroll
+                        for (int r = 0; r < kX; ++r) {
+                            even[r] += xs[r][j][8 * w + 2 * b] * levels.x;
+                            odd[r] += xs[r][j][8 * w + 2 * b + 1] * levels.y;
+                        }
                     }
+                }
+#endif
+#pragma unroll
+                for (int r = 0; r < kX; ++r) {
+                    row_acc[r] += (even[r] + odd[r]) * current.scales[row][j];
                 }
             }
 #pragma unroll
             for (int r = 0; r < kX; ++r) {
-                acc[row][r] += sums[r] * scales[row][j];
+                acc[row * kX + r] = row_acc[r];
             }
+        }
+
+        // Park this DPP row's totals; nobody waits here.
+        const float total = transposed_row_sum<kValues>(acc, lane);
+        if (lane % kRowLanes < kValues) {
+            partial[team][iteration][thread / kRowLanes]
+                   [slot_of_lane<kValues>(lane % kRowLanes)] = total;
+        }
+    };
+
+    // Ping-pong between the two register batches (no copies).
+    for (unsigned iteration = 0; iteration < iterations; iteration += 2) {
+        step(ping, pong, iteration);
+        if (iteration + 1 < iterations) {
+            step(pong, ping, iteration + 1);
         }
     }
 
-    const unsigned wave = thread / kWave;
-    const unsigned lane = thread % kWave;
-#pragma unroll
-    for (int row = 0; row < kRows; ++row) {
-#pragma unroll
-        for (int r = 0; r < kX; ++r) {
-            const float total = wave_sum(acc[row][r]);
-            if (lane == 0) {
-                partial[wave][row][r] = total;
-            }
-        }
-    }
+    // The only barrier after the table build: every batch of this workgroup
+    // has been parked.  Each team adds up its 16 row partials per value and
+    // writes y.
     __syncthreads();
-
-    if (thread < kRows * kX) {
-        const unsigned row = thread / kX;
-        const unsigned r = thread % kX;
-        const unsigned o = first_row + row;
-        if (o < output_width) {
-            float total = 0.0F;
+    for (unsigned index = thread; index < iterations * kValues;
+         index += kTeamThreads) {
+        const unsigned iteration = index / kValues;
+        const unsigned value = index % kValues;
+        const unsigned batch_index = first_batch + iteration * stride;
+        const unsigned o = batch_index * kRows + value / kX;
+        const unsigned r = value % kX;
+        if (batch_index < batch_count && o < output_width && r < x_rows) {
+            float sum = 0.0F;
 #pragma unroll
-            for (int w = 0; w < kWaves; ++w) {
-                total += partial[w][row][r];
+            for (int row = 0; row < kTeamDppRows; ++row) {
+                sum += partial[team][iteration][row][value];
             }
             if (bias != nullptr) {
-                total += bias[o];
+                sum += bias[o];
             }
-            y[static_cast<std::size_t>(r) * output_width + o] = total;
+            y[r * output_width + o] = sum;
         }
     }
+}
+
+std::size_t segments_per_thread(const LinearProblem& p) {
+    return (p.input_width / kSegment + kTeamThreads - 1) / kTeamThreads;
 }
 
 template <int kX, int kSegments, bool kDoubleQuantized>
 void launch_instance(const LinearProblem& p, hipStream_t stream) {
-    // Fewer rows per workgroup when a thread carries more state.
-    constexpr int kRows = (kX * kSegments <= 2) ? 8 : 4;
-    const unsigned blocks =
+    // Two teams (eight wavefronts) per workgroup measured best on MI355X; a
+    // thread that carries more x rows or segments takes fewer weight rows per
+    // batch so that its registers fit.
+    constexpr bool kLight = kX * kSegments == 1;
+    constexpr int kTeams = kLight ? RTHIP_GEMV_TEAMS : 2;
+    constexpr int kRows = kLight ? RTHIP_GEMV_ROWS : (kX * kSegments <= 4 ? 4 : 2);
+    const std::size_t elements = p.output_width * p.input_width;
+    const std::size_t block_count = elements >> p.block_shift;
+    GemvBuffers sizes;
+    sizes.code_bytes = static_cast<unsigned>(elements / 2);
+    if constexpr (!kDoubleQuantized) {
+        sizes.primary_bytes = static_cast<unsigned>(block_count * 4);
+        sizes.secondary_bytes = 0;
+    } else {
+        sizes.primary_bytes = static_cast<unsigned>(block_count);
+        sizes.secondary_bytes = static_cast<unsigned>(
+            (((block_count - 1) >> p.weight.second_level_shift) + 1) * 4);
+    }
+    const unsigned batch_count =
         static_cast<unsigned>((p.output_width + kRows - 1) / kRows);
-    gemv_forward_kernel<kX, kSegments, kRows, kDoubleQuantized>
-        <<<blocks, kThreads, 0, stream>>>(
-            p.activations, p.weight, p.bias, p.result,
+    const unsigned team_groups = (batch_count + kTeams - 1) / kTeams;
+    // One workgroup per CU; more when a team would otherwise need more
+    // batches than its LDS parking space holds.
+    unsigned blocks = team_groups < kComputeUnits ? team_groups : kComputeUnits;
+    if ((team_groups + blocks - 1) / blocks > kMaxIterations) {
+        blocks = (team_groups + kMaxIterations - 1) / kMaxIterations;
+    }
+    const unsigned iterations = (team_groups + blocks - 1) / blocks;
+    gemv_forward_kernel<kX, kSegments, kRows, kTeams, kDoubleQuantized>
+        <<<blocks, kTeamThreads * kTeams, 0, stream>>>(
+            p.activations, p.weight, sizes, p.bias, p.result,
+            static_cast<unsigned>(p.rows),
             static_cast<unsigned>(p.input_width),
-            static_cast<unsigned>(p.output_width), p.block_shift);
+            static_cast<unsigned>(p.output_width), p.block_shift, batch_count,
+            iterations);
 }
 
 template <int kX, bool kDoubleQuantized>
 void launch_segments(const LinearProblem& p, hipStream_t stream) {
-    const std::size_t per_thread =
-        (p.input_width / kSegment + kThreads - 1) / kThreads;
-    switch (per_thread) {
+    switch (segments_per_thread(p)) {
     case 1: launch_instance<kX, 1, kDoubleQuantized>(p, stream); break;
     case 2: launch_instance<kX, 2, kDoubleQuantized>(p, stream); break;
     case 3: launch_instance<kX, 3, kDoubleQuantized>(p, stream); break;
@@ -198,7 +508,6 @@ void launch_rows(const LinearProblem& p, hipStream_t stream) {
     switch (p.rows) {
     case 1: launch_segments<1, kDoubleQuantized>(p, stream); break;
     case 2: launch_segments<2, kDoubleQuantized>(p, stream); break;
-    case 3: launch_segments<3, kDoubleQuantized>(p, stream); break;
     default: launch_segments<4, kDoubleQuantized>(p, stream); break;
     }
 }
@@ -207,14 +516,18 @@ void launch_rows(const LinearProblem& p, hipStream_t stream) {
 
 bool gemv_forward_supports(const LinearProblem& p) {
     constexpr std::size_t kMaxWidth =
-        static_cast<std::size_t>(kSegment) * kThreads * 4;
-    // x rows times segments per thread bounds the register-resident x slice.
-    const std::size_t per_thread =
-        (p.input_width / kSegment + kThreads - 1) / kThreads;
+        static_cast<std::size_t>(kSegment) * kTeamThreads * 4;
+    // x rows (3 runs as 4) times segments per thread bounds the
+    // register-resident x slice.
+    const std::size_t held_rows = p.rows == 3 ? 4 : p.rows;
     return p.rows >= 1 && p.rows <= kGemvMaxRows &&
-           p.rows * per_thread <= 8 &&
+           held_rows * segments_per_thread(p) <= 8 &&
            p.input_width % kSegment == 0 && p.input_width <= kMaxWidth &&
-           p.output_width < (1ULL << 31) &&
+           // rows start on block boundaries (scalar row offset into scales)
+           p.input_width % (std::size_t{1} << p.block_shift) == 0 &&
+           p.output_width * p.input_width < (1ULL << 32) &&
+           p.rows * p.input_width < (1ULL << 32) &&
+           p.rows * p.output_width < (1ULL << 32) &&
            reinterpret_cast<std::uintptr_t>(p.weight.codes) % 8 == 0 &&
            reinterpret_cast<std::uintptr_t>(p.activations) % 16 == 0;
 }
