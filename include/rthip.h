@@ -95,6 +95,16 @@ rthip_status rthip_device_count(int32_t* count);
 /* Human-readable device description, e.g. "AMD Instinct MI355X (gfx950), 256 CUs". */
 rthip_status rthip_device_description(char* buffer, size_t capacity);
 
+/* *visible = 1 when pointers returned by rthip_malloc can be dereferenced by
+ * the host (the whole HBM is mapped through a large PCIe BAR, the normal
+ * configuration of MI300/MI350-class servers), 0 otherwise.  The adapter uses
+ * it to decide whether packed-weight storage can serve the host-readable spans
+ * of QuantizedWeightStorage
+ * (src/core/backend/nn/quantized_linear/storage.hpp:85-88) straight from HBM,
+ * with no mirror -- what the CUDA backend obtains from managed memory
+ * (src/core/backend/nn/quantized_linear/cuda/storage.cu:22-43). */
+rthip_status rthip_device_memory_host_visible(int32_t* visible);
+
 /* ---- memory ----------------------------------------------------------- */
 
 /* Device (HBM) allocation; *pointer is 256-byte aligned.  bytes == 0 yields

@@ -1,0 +1,606 @@
+// Implementation of the `hip` backend adapter.
+//
+// Device work goes through the kernel C ABI only (hip_runtime.hpp); nothing in
+// this file includes a HIP header, so it builds with any C++20 host compiler.
+//
+// Storage model
+//   HipTensorStorage     fp32 tensor in HBM plus a lazily synchronised host
+//                        mirror, because TensorStorage::data() must hand out
+//                        host spans (src/core/backend/storage.hpp:21-24) that
+//                        callers may also write through.  A tensor that is
+//                        only ever produced and consumed by kernels never
+//                        allocates or touches the mirror.
+//   HipNf4WeightStorage  immutable packed codes and scales in HBM.  On servers
+//                        that map all of HBM through a large PCIe BAR the host
+//                        spans of QuantizedWeightStorage point straight at that
+//                        memory: one allocation, resident bytes == logical
+//                        bytes, as the reference's accelerator test demands
+//                        (tests/core/backend/test_quantized_linear_backend.cpp:424-430).
+//                        Otherwise a host copy is kept and counted.
+//
+// Both operations are synchronous: they return after the stream has drained
+// (docs/BACKENDS_AND_PYTHON.md:168).
+
+#include "hip_adapter.hpp"
+
+#include "hip_runtime.hpp"
+
+#if defined(RIFTCO_TRANSFORMER_IN_TREE)
+#include "core/backend/attention/reference/flash_causal.hpp"
+#include "core/backend/attention/reference/materialized_causal.hpp"
+#include "core/backend/attention/reference/paged_decode.hpp"
+#include "core/backend/nn/reference/operations.hpp"
+#include "core/backend/optim/adam/reference/update.hpp"
+#endif
+
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <stdexcept>
+#include <string>
+#include <utility>
+
+namespace riftco_transformer::backend_detail {
+namespace {
+
+[[noreturn]] void throw_unavailable(const HipRuntime& runtime) {
+    std::string message = "hip execution backend is unavailable";
+    if (!runtime.reason.empty()) {
+        message += ": ";
+        message += runtime.reason;
+    }
+    throw std::runtime_error(message);
+}
+
+const HipRuntime& require_runtime() {
+    const HipRuntime& runtime = hip_runtime();
+    if (!runtime.available) {
+        throw_unavailable(runtime);
+    }
+    return runtime;
+}
+
+// Maps an rthip_status to the exception type the reference uses for the same
+// condition (src/core/backend/adapters/cuda/adapter.cu:25-32 for bad_alloc).
+void check(const HipRuntime& runtime, rthip_status status,
+           std::string_view operation) {
+    if (status == RTHIP_OK) {
+        return;
+    }
+    std::string message = "hip " + std::string(operation) + ": " +
+                          runtime.last_error();
+    switch (status) {
+    case RTHIP_INVALID_ARGUMENT:
+        throw std::invalid_argument(message);
+    case RTHIP_OUT_OF_MEMORY:
+        throw std::bad_alloc();
+    case RTHIP_UNAVAILABLE:
+        throw_unavailable(runtime);
+    default:
+        throw std::runtime_error(message);
+    }
+}
+
+// Owning handle of one HBM allocation.
+class DeviceBuffer final {
+public:
+    DeviceBuffer() = default;
+    explicit DeviceBuffer(std::size_t bytes) : bytes_(bytes) {
+        if (bytes_ != 0) {
+            const HipRuntime& runtime = require_runtime();
+            check(runtime, runtime.malloc(&pointer_, bytes_),
+                  "device allocation");
+        }
+    }
+    DeviceBuffer(const void* host, std::size_t bytes) : DeviceBuffer(bytes) {
+        if (bytes_ != 0) {
+            const HipRuntime& runtime = require_runtime();
+            check(runtime, runtime.copy_to_device(pointer_, host, bytes_),
+                  "host-to-device copy");
+        }
+    }
+    DeviceBuffer(const DeviceBuffer&) = delete;
+    DeviceBuffer& operator=(const DeviceBuffer&) = delete;
+    DeviceBuffer(DeviceBuffer&& other) noexcept
+        : pointer_(std::exchange(other.pointer_, nullptr)),
+          bytes_(std::exchange(other.bytes_, 0)) {}
+    DeviceBuffer& operator=(DeviceBuffer&& other) noexcept {
+        if (this != &other) {
+            release();
+            pointer_ = std::exchange(other.pointer_, nullptr);
+            bytes_ = std::exchange(other.bytes_, 0);
+        }
+        return *this;
+    }
+    ~DeviceBuffer() { release(); }
+
+    [[nodiscard]] void* get() const noexcept { return pointer_; }
+    [[nodiscard]] std::size_t bytes() const noexcept { return bytes_; }
+
+private:
+    void release() noexcept {
+        if (pointer_ != nullptr) {
+            static_cast<void>(hip_runtime().free(pointer_));
+            pointer_ = nullptr;
+        }
+    }
+
+    void* pointer_ = nullptr;
+    std::size_t bytes_ = 0;
+};
+
+class HipTensorStorage final : public TensorStorage {
+public:
+    HipTensorStorage(std::size_t element_count, float fill_value)
+        : count_(element_count),
+          device_(checked_bytes(element_count)),
+          freshest_(Freshest::Device) {
+        const HipRuntime& runtime = require_runtime();
+        check(runtime,
+              runtime.fill_f32(static_cast<float*>(device_.get()), fill_value,
+                               count_, nullptr),
+              "tensor fill");
+        check(runtime, runtime.stream_synchronize(nullptr),
+              "tensor fill synchronisation");
+    }
+
+    explicit HipTensorStorage(std::vector<float> values)
+        : count_(values.size()),
+          device_(values.data(), checked_bytes(values.size())),
+          host_(std::move(values)),
+          freshest_(Freshest::Both) {}
+
+    [[nodiscard]] ExecutionBackend backend() const noexcept override {
+        return kHipBackend;
+    }
+    [[nodiscard]] std::size_t size() const noexcept override {
+        return count_;
+    }
+
+    // A writable span: from here on the host copy may be newer than HBM.
+    [[nodiscard]] std::span<float> data() noexcept override {
+        refresh_host();
+        freshest_ = Freshest::Host;
+        return host_;
+    }
+    [[nodiscard]] std::span<const float> data() const noexcept override {
+        refresh_host();
+        return host_;
+    }
+
+    // The persistent HBM allocation; identifies the tensor for the
+    // dispatcher's aliasing checks and triggers no transfer.
+    [[nodiscard]] void* native_handle() noexcept override {
+        return device_.get();
+    }
+    [[nodiscard]] const void* native_handle() const noexcept override {
+        return device_.get();
+    }
+
+    [[nodiscard]] std::unique_ptr<TensorStorage> clone() const override {
+        const auto values = data();
+        return std::make_unique<HipTensorStorage>(
+            std::vector<float>(values.begin(), values.end()));
+    }
+
+    // HBM pointer with the tensor's current contents.
+    [[nodiscard]] const float* device_for_read() const {
+        if (freshest_ == Freshest::Host) {
+            const HipRuntime& runtime = require_runtime();
+            check(runtime,
+                  runtime.copy_to_device(device_.get(), host_.data(),
+                                         count_ * sizeof(float)),
+                  "tensor upload");
+            freshest_ = Freshest::Both;
+        }
+        return static_cast<const float*>(device_.get());
+    }
+
+    // HBM pointer that a kernel is about to overwrite completely.
+    [[nodiscard]] float* device_for_overwrite() noexcept {
+        freshest_ = Freshest::Device;
+        return static_cast<float*>(device_.get());
+    }
+
+private:
+    enum class Freshest { Host, Device, Both };
+
+    static std::size_t checked_bytes(std::size_t element_count) {
+        if (element_count >
+            std::numeric_limits<std::size_t>::max() / sizeof(float)) {
+            throw std::overflow_error(
+                "hip tensor allocation size overflow");
+        }
+        return element_count * sizeof(float);
+    }
+
+    // noexcept by contract: a failing device read-back ends the process, as a
+    // failing access to a managed CUDA allocation would.
+    void refresh_host() const noexcept {
+        if (freshest_ != Freshest::Device) {
+            return;
+        }
+        host_.resize(count_);
+        const HipRuntime& runtime = hip_runtime();
+        if (count_ != 0 &&
+            runtime.copy_to_host(host_.data(), device_.get(),
+                                 count_ * sizeof(float)) != RTHIP_OK) {
+            std::abort();
+        }
+        freshest_ = Freshest::Both;
+    }
+
+    std::size_t count_;
+    DeviceBuffer device_;
+    mutable std::vector<float> host_;
+    mutable Freshest freshest_;
+};
+
+// One payload array of a packed weight: HBM allocation plus, only where HBM
+// is not host-visible (or a mirror was asked for), a host copy.
+template <typename Element>
+class WeightArray final {
+public:
+    WeightArray() = default;
+    WeightArray(std::vector<Element> values, bool keep_host_copy)
+        : count_(values.size()),
+          device_(values.data(), values.size() * sizeof(Element)) {
+        if (keep_host_copy) {
+            host_ = std::move(values);
+        }
+    }
+
+    [[nodiscard]] std::span<const Element> values() const noexcept {
+        if (!host_.empty()) {
+            return host_;
+        }
+        return {static_cast<const Element*>(device_.get()), count_};
+    }
+    [[nodiscard]] const Element* device() const noexcept {
+        return static_cast<const Element*>(device_.get());
+    }
+    [[nodiscard]] std::size_t resident_bytes() const noexcept {
+        return count_ * sizeof(Element) + host_.size() * sizeof(Element);
+    }
+
+private:
+    std::size_t count_ = 0;
+    DeviceBuffer device_;
+    std::vector<Element> host_;
+};
+
+bool scale_mirror_requested() noexcept {
+    const char* value = std::getenv("RIFTCO_TRANSFORMER_HIP_SCALE_MIRROR");
+    return value != nullptr && std::strcmp(value, "1") == 0;
+}
+
+class HipNf4WeightStorage final : public QuantizedWeightStorage,
+                                  public ScaleValidationMemo {
+public:
+    HipNf4WeightStorage(std::vector<std::uint8_t> packed_codes,
+                        Nf4ScaleStorageData scales, bool host_visible)
+        : encoding_(scales.encoding),
+          packed_codes_(std::move(packed_codes), !host_visible),
+          fp32_scales_(std::move(scales.fp32_scales),
+                       !host_visible || scale_mirror_requested()),
+          quantized_scales_(std::move(scales.quantized_scales),
+                            !host_visible || scale_mirror_requested()),
+          second_level_scales_(std::move(scales.second_level_scales),
+                               !host_visible || scale_mirror_requested()),
+          second_level_block_size_(scales.second_level_block_size),
+          offset_(scales.offset) {}
+
+    [[nodiscard]] ExecutionBackend backend() const noexcept override {
+        return kHipBackend;
+    }
+    [[nodiscard]] std::span<const std::uint8_t> packed_codes()
+        const noexcept override {
+        return packed_codes_.values();
+    }
+    [[nodiscard]] Nf4ScaleStorageView scale_storage() const noexcept override {
+        return {encoding_,
+                fp32_scales_.values(),
+                quantized_scales_.values(),
+                second_level_scales_.values(),
+                second_level_block_size_,
+                offset_};
+    }
+    [[nodiscard]] const void* packed_codes_native_handle()
+        const noexcept override {
+        return packed_codes_.device();
+    }
+    [[nodiscard]] const void* primary_scales_native_handle()
+        const noexcept override {
+        return encoding_ == Nf4ScaleEncoding::Float32
+            ? static_cast<const void*>(fp32_scales_.device())
+            : static_cast<const void*>(quantized_scales_.device());
+    }
+    [[nodiscard]] const void* secondary_scales_native_handle()
+        const noexcept override {
+        return encoding_ == Nf4ScaleEncoding::DoubleQuantizedUInt8
+            ? static_cast<const void*>(second_level_scales_.device())
+            : nullptr;
+    }
+    // Every persistent byte: HBM plus any host copy; the 4-byte offset of the
+    // double-quantised encoding lives in this object and counts once.
+    [[nodiscard]] std::size_t resident_payload_bytes()
+        const noexcept override {
+        return packed_codes_.resident_bytes() + fp32_scales_.resident_bytes() +
+               quantized_scales_.resident_bytes() +
+               second_level_scales_.resident_bytes() +
+               (encoding_ == Nf4ScaleEncoding::DoubleQuantizedUInt8
+                    ? sizeof(float)
+                    : 0);
+    }
+
+    [[nodiscard]] bool scales_validated() const noexcept override {
+        return scales_validated_;
+    }
+    void mark_scales_validated() const noexcept override {
+        scales_validated_ = true;
+    }
+
+    [[nodiscard]] Nf4ScaleEncoding encoding() const noexcept {
+        return encoding_;
+    }
+    [[nodiscard]] std::size_t second_level_block_size() const noexcept {
+        return second_level_block_size_;
+    }
+    [[nodiscard]] float offset() const noexcept { return offset_; }
+
+private:
+    Nf4ScaleEncoding encoding_;
+    WeightArray<std::uint8_t> packed_codes_;
+    WeightArray<float> fp32_scales_;
+    WeightArray<std::uint8_t> quantized_scales_;
+    WeightArray<float> second_level_scales_;
+    std::size_t second_level_block_size_;
+    float offset_;
+    mutable bool scales_validated_ = false;
+};
+
+const HipTensorStorage& require_hip_tensor(const TensorStorage& storage,
+                                           std::string_view operation) {
+    const auto* tensor = dynamic_cast<const HipTensorStorage*>(&storage);
+    if (tensor == nullptr) {
+        throw std::invalid_argument("hip " + std::string(operation) +
+                                    " requires hip tensor storage");
+    }
+    return *tensor;
+}
+
+HipTensorStorage& require_hip_tensor(TensorStorage& storage,
+                                     std::string_view operation) {
+    auto* tensor = dynamic_cast<HipTensorStorage*>(&storage);
+    if (tensor == nullptr) {
+        throw std::invalid_argument("hip " + std::string(operation) +
+                                    " requires hip tensor storage");
+    }
+    return *tensor;
+}
+
+const HipNf4WeightStorage& require_hip_weight(
+    const QuantizedWeightStorage& storage, std::string_view operation
+) {
+    const auto* weight = dynamic_cast<const HipNf4WeightStorage*>(&storage);
+    if (weight == nullptr) {
+        throw std::invalid_argument("hip " + std::string(operation) +
+                                    " requires hip quantized-weight storage");
+    }
+    if (weight->packed_codes_native_handle() == nullptr ||
+        weight->primary_scales_native_handle() == nullptr) {
+        throw std::logic_error("hip " + std::string(operation) +
+                               " received packed storage without a native "
+                               "allocation");
+    }
+    return *weight;
+}
+
+class HipBackendAdapter final : public BackendAdapter {
+public:
+    [[nodiscard]] std::string_view name() const noexcept override {
+        return "hip";
+    }
+    [[nodiscard]] bool is_available() const noexcept override {
+        return hip_runtime().available;
+    }
+    [[nodiscard]] std::string_view unavailability_reason()
+        const noexcept override {
+        return hip_runtime().reason;
+    }
+
+    [[nodiscard]] std::unique_ptr<TensorStorage> make_storage(
+        std::size_t element_count, float fill_value
+    ) const override {
+        return std::make_unique<HipTensorStorage>(element_count, fill_value);
+    }
+    [[nodiscard]] std::unique_ptr<TensorStorage> make_storage(
+        std::vector<float> values
+    ) const override {
+        return std::make_unique<HipTensorStorage>(std::move(values));
+    }
+
+    [[nodiscard]] std::unique_ptr<QuantizedWeightStorage>
+    make_nf4_weight_storage(std::vector<std::uint8_t> packed_codes,
+                            Nf4ScaleStorageData scales) const override {
+        const HipRuntime& runtime = require_runtime();
+        return std::make_unique<HipNf4WeightStorage>(
+            std::move(packed_codes), std::move(scales),
+            runtime.host_visible_memory);
+    }
+
+    void quantized_linear_forward(
+        const QuantizedLinearForwardRequest& request
+    ) const override {
+        constexpr std::string_view operation = "quantized-linear forward";
+        const HipRuntime& runtime = require_runtime();
+        const auto& input = require_hip_tensor(request.input, operation);
+        const auto& weight = require_hip_weight(request.weight, operation);
+        auto& output = require_hip_tensor(request.output, operation);
+        const float* source = input.device_for_read();
+        check(runtime,
+              runtime.nf4_linear_forward(
+                  source,
+                  static_cast<const std::uint8_t*>(
+                      weight.packed_codes_native_handle()),
+                  weight.primary_scales_native_handle(),
+                  static_cast<const float*>(
+                      weight.secondary_scales_native_handle()),
+                  static_cast<int32_t>(weight.encoding()),
+                  weight.second_level_block_size(), weight.offset(), nullptr,
+                  output.device_for_overwrite(), request.dimensions.rows,
+                  request.dimensions.input_width,
+                  request.dimensions.output_width,
+                  request.dimensions.block_size, nullptr),
+              operation);
+        check(runtime, runtime.stream_synchronize(nullptr),
+              "quantized-linear forward synchronisation");
+    }
+
+    void quantized_linear_input_backward(
+        const QuantizedLinearInputBackwardRequest& request
+    ) const override {
+        constexpr std::string_view operation =
+            "quantized-linear input backward";
+        const HipRuntime& runtime = require_runtime();
+        const auto& upstream = require_hip_tensor(request.upstream, operation);
+        const auto& weight = require_hip_weight(request.weight, operation);
+        auto& gradient = require_hip_tensor(request.input_gradient, operation);
+        const float* source = upstream.device_for_read();
+        check(runtime,
+              runtime.nf4_linear_input_backward(
+                  source,
+                  static_cast<const std::uint8_t*>(
+                      weight.packed_codes_native_handle()),
+                  weight.primary_scales_native_handle(),
+                  static_cast<const float*>(
+                      weight.secondary_scales_native_handle()),
+                  static_cast<int32_t>(weight.encoding()),
+                  weight.second_level_block_size(), weight.offset(),
+                  gradient.device_for_overwrite(), request.dimensions.rows,
+                  request.dimensions.input_width,
+                  request.dimensions.output_width,
+                  request.dimensions.block_size, nullptr),
+              operation);
+        check(runtime, runtime.stream_synchronize(nullptr),
+              "quantized-linear input-backward synchronisation");
+    }
+
+#if defined(RIFTCO_TRANSFORMER_IN_TREE)
+    // Inside the reference tree BackendAdapter has 27 more pure virtuals.  As
+    // the TPU adapter does (src/core/backend/adapters/tpu/adapter.cpp:114-200),
+    // capabilities without a native kernel run the reference host loops on
+    // the storage's host spans; the mirror of HipTensorStorage keeps those
+    // coherent with HBM.
+    void matmul(const MatmulRequest& request) const override {
+        cpu_backend_adapter().matmul(request);
+    }
+    void unary_elementwise(
+        const UnaryElementwiseRequest& request) const override {
+        nn_reference_unary_elementwise(request);
+    }
+    void binary_elementwise(
+        const BinaryElementwiseRequest& request) const override {
+        nn_reference_binary_elementwise(request);
+    }
+    void scale(const ScaleRequest& request) const override {
+        nn_reference_scale(request);
+    }
+    void gelu_forward(const GeluForwardRequest& request) const override {
+        nn_reference_gelu_forward(request);
+    }
+    void gelu_backward(const GeluBackwardRequest& request) const override {
+        nn_reference_gelu_backward(request);
+    }
+    void reduce(const ReductionRequest& request) const override {
+        nn_reference_reduce(request);
+    }
+    void copy(const CopyRequest& request) const override {
+        nn_reference_copy(request);
+    }
+    void permute(const PermuteRequest& request) const override {
+        nn_reference_permute(request);
+    }
+    void broadcast(const BroadcastRequest& request) const override {
+        nn_reference_broadcast(request);
+    }
+    void sum_to_shape(const SumToShapeRequest& request) const override {
+        nn_reference_sum_to_shape(request);
+    }
+    void softmax_forward(
+        const SoftmaxForwardRequest& request) const override {
+        nn_reference_softmax_forward(request);
+    }
+    void softmax_backward(
+        const SoftmaxBackwardRequest& request) const override {
+        nn_reference_softmax_backward(request);
+    }
+    void causal_softmax_forward(
+        const CausalSoftmaxForwardRequest& request) const override {
+        nn_reference_causal_softmax_forward(request);
+    }
+    void causal_softmax_backward(
+        const CausalSoftmaxBackwardRequest& request) const override {
+        nn_reference_causal_softmax_backward(request);
+    }
+    void gather_rows(const GatherRowsRequest& request) const override {
+        nn_reference_gather_rows(request);
+    }
+    void scatter_add_rows(
+        const ScatterAddRowsRequest& request) const override {
+        nn_reference_scatter_add_rows(request);
+    }
+    void layer_norm_forward(
+        const LayerNormForwardRequest& request) const override {
+        nn_reference_layer_norm_forward(request);
+    }
+    void layer_norm_backward(
+        const LayerNormBackwardRequest& request) const override {
+        nn_reference_layer_norm_backward(request);
+    }
+    void cross_entropy_forward(
+        const CrossEntropyForwardRequest& request) const override {
+        nn_reference_cross_entropy_forward(request);
+    }
+    void materialized_causal_attention_forward(
+        const MaterializedCausalAttentionForwardRequest& request)
+        const override {
+        reference_materialized_causal_attention_forward(request);
+    }
+    void materialized_causal_attention_context_backward(
+        const MaterializedCausalAttentionContextBackwardRequest& request)
+        const override {
+        reference_materialized_causal_attention_context_backward(request);
+    }
+    void materialized_causal_attention_probabilities_backward(
+        const MaterializedCausalAttentionProbabilitiesBackwardRequest&
+            request) const override {
+        reference_materialized_causal_attention_probabilities_backward(
+            request);
+    }
+    void flash_causal_attention_forward(
+        const FlashCausalAttentionForwardRequest& request) const override {
+        reference_flash_causal_attention_forward(request);
+    }
+    void flash_causal_attention_backward(
+        const FlashCausalAttentionBackwardRequest& request) const override {
+        reference_flash_causal_attention_backward(request);
+    }
+    void paged_decode_attention_forward(
+        const PagedDecodeAttentionForwardRequest& request) const override {
+        reference_paged_decode_attention_forward(request);
+    }
+    void adam_update(const AdamUpdateRequest& request) const override {
+        adam_reference_update(request);
+    }
+#endif
+};
+
+}  // namespace
+
+const BackendAdapter& hip_backend_adapter() noexcept {
+    static const HipBackendAdapter adapter;
+    return adapter;
+}
+
+}  // namespace riftco_transformer::backend_detail

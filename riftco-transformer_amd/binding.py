@@ -78,6 +78,7 @@ _PROTOTYPES = {
     "rthip_last_error": (ctypes.c_char_p, []),
     "rthip_device_count": (_i32, [ctypes.POINTER(_i32)]),
     "rthip_device_description": (_i32, [ctypes.c_char_p, _size]),
+    "rthip_device_memory_host_visible": (_i32, [ctypes.POINTER(_i32)]),
     "rthip_malloc": (_i32, [ctypes.POINTER(_ptr), _size]),
     "rthip_free": (_i32, [_ptr]),
     "rthip_copy_to_device": (_i32, [_ptr, _ptr, _size]),
@@ -183,6 +184,12 @@ class Library:
         buffer = ctypes.create_string_buffer(256)
         self._check(self._lib.rthip_device_description(buffer, 256))
         return buffer.value.decode()
+
+    def device_memory_host_visible(self) -> bool:
+        visible = _i32(0)
+        self._check(self._lib.rthip_device_memory_host_visible(
+            ctypes.byref(visible)))
+        return bool(visible.value)
 
     # -- memory ------------------------------------------------------------
     def malloc(self, size: int) -> int:

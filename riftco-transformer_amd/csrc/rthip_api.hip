@@ -45,6 +45,7 @@ rthip_status from_hip(hipError_t error, const char* what) {
 struct DeviceState {
     rthip_status status = RTHIP_UNAVAILABLE;
     int count = 0;
+    bool large_bar = false;
     char description[256] = "";
     char reason[256] = "";
 };
@@ -80,6 +81,7 @@ const DeviceState& device_state() {
         }
         state.status = RTHIP_OK;
         state.count = count;
+        state.large_bar = properties.isLargeBar != 0;
         std::snprintf(state.description, sizeof(state.description),
                       "%s (%s), %d CUs, %.0f GiB", properties.name,
                       properties.gcnArchName, properties.multiProcessorCount,
@@ -220,6 +222,18 @@ rthip_status rthip_device_description(char* buffer, size_t capacity) {
         return status;
     }
     std::snprintf(buffer, capacity, "%s", device_state().description);
+    return ok();
+}
+
+rthip_status rthip_device_memory_host_visible(int32_t* visible) {
+    if (visible == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "visible must not be null");
+    }
+    *visible = 0;
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    *visible = device_state().large_bar ? 1 : 0;
     return ok();
 }
 

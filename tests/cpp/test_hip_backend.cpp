@@ -1,0 +1,645 @@
+// Tests of the `hip` backend adapter through the same entry points the
+// reference's own backend test uses (make_nf4_weight_storage,
+// dispatch_quantized_linear_forward / _input_backward), against the CPU oracle.
+// Counterparts (paths under /root/reference):
+//   accelerator oracle loop, memory accounting, edge layout
+//       tests/core/backend/test_quantized_linear_backend.cpp:382-453
+//   unavailable backend must reject packed transfer   :472-499
+//   backend identity / unknown ids
+//       tests/core/backend/test_backend.cpp:172-240
+//   byte-preserving transfer   tests/core/test_quantization.cpp:400-435
+//
+// Plain main(), as the reference's tests are.  Modes:
+//   test_hip_backend                 run against whatever runtime the adapter
+//                                    loads (RIFTCO_TRANSFORMER_HIP_LIBRARY)
+//   test_hip_backend --expect-unavailable
+//                                    the runtime must be unavailable and the
+//                                    adapter must fail the documented way
+// RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP=1 turns "unavailable" into a failure.
+
+#include "../../riftco-transformer_amd/backend/dispatch.hpp"
+
+extern "C" {
+#include "../../oracle/nf4_oracle.h"
+}
+
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <iostream>
+#include <new>
+#include <stdexcept>
+#include <string>
+#include <string_view>
+#include <vector>
+
+namespace {
+
+using riftco_transformer::ExecutionBackend;
+namespace backend = riftco_transformer::backend_detail;
+
+constexpr ExecutionBackend kHip = backend::kHipBackend;
+constexpr std::size_t kEdgeWidth = 33;
+
+void require(bool condition, const std::string& message) {
+    if (!condition) {
+        throw std::runtime_error(message);
+    }
+}
+
+template <typename Exception, typename Function>
+void require_throws(Function&& function, const std::string& message,
+                    std::string_view fragment = {}) {
+    try {
+        function();
+    } catch (const Exception& error) {
+        if (!fragment.empty() &&
+            std::string(error.what()).find(fragment) == std::string::npos) {
+            throw std::runtime_error(message + ": wrong message: " +
+                                     error.what());
+        }
+        return;
+    } catch (const std::exception& error) {
+        throw std::runtime_error(message + ": wrong exception: " +
+                                 error.what());
+    }
+    throw std::runtime_error(message + ": nothing was thrown");
+}
+
+// |a - e| <= 3e-5 * max(1, |a|, |e|): the reference's tolerance
+// (test_quantized_linear_backend.cpp:46-70).
+void require_close(std::span<const float> actual,
+                   const std::vector<float>& expected,
+                   const std::string& message, float tolerance = 3.0e-5F) {
+    require(actual.size() == expected.size(), message + ": size mismatch");
+    for (std::size_t index = 0; index < expected.size(); ++index) {
+        const float scale = std::max(
+            {1.0F, std::fabs(actual[index]), std::fabs(expected[index])});
+        if (!std::isfinite(actual[index]) ||
+            std::fabs(actual[index] - expected[index]) > tolerance * scale) {
+            throw std::runtime_error(
+                message + " at flat index " + std::to_string(index) +
+                ": expected " + std::to_string(expected[index]) + ", got " +
+                std::to_string(actual[index]));
+        }
+    }
+}
+
+// ---- fixtures: the integer-formula tensors of the reference test ---------
+
+std::vector<float> aligned_weight() {  // :89-100
+    std::vector<float> values(3 * 32);
+    for (std::size_t i = 0; i < values.size(); ++i) {
+        values[i] = static_cast<float>(static_cast<int>(i % 19) - 9) * 0.1375F;
+    }
+    values[0] = -2.0F;
+    values[31] = 1.75F;
+    values[32] = 3.0F;
+    values.back() = -4.0F;
+    return values;
+}
+
+std::vector<float> aligned_input() {  // :102-109
+    std::vector<float> values(2 * 32);
+    for (std::size_t i = 0; i < values.size(); ++i) {
+        values[i] = static_cast<float>(static_cast<int>(i % 11) - 5) * 0.2F;
+    }
+    return values;
+}
+
+std::vector<float> aligned_upstream() {  // :111-124
+    return {0.25F, -0.75F, 1.5F, -1.0F, 0.5F, 0.125F};
+}
+
+std::vector<float> edge_weight() {  // :126-142
+    std::vector<float> values(kEdgeWidth * kEdgeWidth);
+    for (std::size_t i = 0; i < values.size(); ++i) {
+        values[i] = static_cast<float>(static_cast<int>(i % 37) - 18) * 0.0625F;
+    }
+    values[0] = -3.0F;
+    values[31] = 2.5F;
+    values[32] = -2.75F;
+    values[1023] = 4.0F;
+    values[1024] = -4.5F;
+    values.back() = 5.0F;
+    return values;
+}
+
+std::vector<float> edge_input() {  // :144-155
+    std::vector<float> values(2 * kEdgeWidth);
+    for (std::size_t i = 0; i < values.size(); ++i) {
+        values[i] = static_cast<float>(static_cast<int>(i % 17) - 8) * 0.125F;
+    }
+    return values;
+}
+
+std::vector<float> edge_upstream() {  // :157-168
+    std::vector<float> values(2 * kEdgeWidth);
+    for (std::size_t i = 0; i < values.size(); ++i) {
+        values[i] = static_cast<float>(static_cast<int>(i % 13) - 6) * 0.075F;
+    }
+    return values;
+}
+
+// A deterministic pseudo-normal filler for the larger layer.
+std::vector<float> pseudo_normal(std::size_t count, float sigma,
+                                 std::uint32_t seed) {
+    std::vector<float> values(count);
+    std::uint32_t state = seed * 2654435761U + 12345U;
+    for (float& value : values) {
+        float sum = 0.0F;
+        for (int k = 0; k < 4; ++k) {
+            state = state * 1664525U + 1013904223U;
+            sum += static_cast<float>(state >> 8) / 16777216.0F - 0.5F;
+        }
+        value = sum * 1.7320508F * sigma;
+    }
+    return values;
+}
+
+// ---- a packed weight on the host, quantised by the oracle ----------------
+
+struct HostWeight {
+    std::size_t output_width;
+    std::size_t input_width;
+    std::size_t block_size;
+    std::vector<std::uint8_t> codes;
+    backend::Nf4ScaleStorageData scales;
+
+    [[nodiscard]] nf4o_scales view() const {
+        nf4o_scales result{};
+        result.encoding = static_cast<int32_t>(scales.encoding);
+        result.fp32_scales = scales.fp32_scales.data();
+        result.fp32_count = scales.fp32_scales.size();
+        result.quantized_scales = scales.quantized_scales.data();
+        result.quantized_count = scales.quantized_scales.size();
+        result.second_level = scales.second_level_scales.data();
+        result.second_level_count = scales.second_level_scales.size();
+        result.second_level_block = scales.second_level_block_size;
+        result.offset = scales.offset;
+        return result;
+    }
+    [[nodiscard]] std::size_t logical_bytes() const {
+        const nf4o_scales v = view();
+        return codes.size() + nf4o_scale_payload_bytes(&v);
+    }
+};
+
+HostWeight quantize(const std::vector<float>& dense, std::size_t output_width,
+                    std::size_t input_width, std::size_t block_size,
+                    bool double_quantized, std::size_t second_level_block) {
+    HostWeight weight{output_width, input_width, block_size, {}, {}};
+    const std::size_t count = dense.size();
+    weight.codes.resize(nf4o_packed_byte_count(count));
+    std::vector<float> block_scales(nf4o_block_count(count, block_size));
+    require(nf4o_quantize(dense.data(), count, block_size, weight.codes.data(),
+                          block_scales.data()) == NF4O_OK,
+            "oracle quantizer failed");
+    if (!double_quantized) {
+        weight.scales.fp32_scales = std::move(block_scales);
+        return weight;
+    }
+    weight.scales.encoding = backend::Nf4ScaleEncoding::DoubleQuantizedUInt8;
+    weight.scales.quantized_scales.resize(block_scales.size());
+    weight.scales.second_level_scales.resize(
+        nf4o_block_count(block_scales.size(), second_level_block));
+    weight.scales.second_level_block_size = second_level_block;
+    require(nf4o_double_quantize_scales(
+                block_scales.data(), block_scales.size(), second_level_block,
+                weight.scales.quantized_scales.data(),
+                weight.scales.second_level_scales.data(),
+                &weight.scales.offset) == NF4O_OK,
+            "oracle double quantizer failed");
+    return weight;
+}
+
+std::unique_ptr<backend::QuantizedWeightStorage> to_hip(
+    const HostWeight& weight
+) {
+    return backend::make_nf4_weight_storage(kHip, weight.codes, weight.scales);
+}
+
+std::vector<float> hip_forward(const std::vector<float>& input,
+                               const backend::QuantizedWeightStorage& storage,
+                               const HostWeight& weight) {
+    const std::size_t rows = input.size() / weight.input_width;
+    auto source = backend::make_tensor_storage(kHip, input);
+    auto target =
+        backend::make_tensor_storage(kHip, rows * weight.output_width, 0.0F);
+    backend::dispatch_quantized_linear_forward(
+        kHip, {*source, storage, *target,
+               {rows, weight.input_width, weight.output_width,
+                weight.block_size}});
+    const auto data = std::as_const(*target).data();
+    return {data.begin(), data.end()};
+}
+
+std::vector<float> hip_input_backward(
+    const std::vector<float>& upstream,
+    const backend::QuantizedWeightStorage& storage, const HostWeight& weight
+) {
+    const std::size_t rows = upstream.size() / weight.output_width;
+    auto source = backend::make_tensor_storage(kHip, upstream);
+    auto target =
+        backend::make_tensor_storage(kHip, rows * weight.input_width, 0.0F);
+    backend::dispatch_quantized_linear_input_backward(
+        kHip, {*source, storage, *target,
+               {rows, weight.input_width, weight.output_width,
+                weight.block_size}});
+    const auto data = std::as_const(*target).data();
+    return {data.begin(), data.end()};
+}
+
+std::vector<float> oracle_forward(const std::vector<float>& input,
+                                  const HostWeight& weight) {
+    const std::size_t rows = input.size() / weight.input_width;
+    std::vector<float> output(rows * weight.output_width);
+    const nf4o_scales scales = weight.view();
+    nf4o_linear_forward(input.data(), weight.codes.data(), &scales,
+                        output.data(), rows, weight.input_width,
+                        weight.output_width, weight.block_size);
+    return output;
+}
+
+std::vector<float> oracle_input_backward(const std::vector<float>& upstream,
+                                         const HostWeight& weight) {
+    const std::size_t rows = upstream.size() / weight.output_width;
+    std::vector<float> gradient(rows * weight.input_width);
+    const nf4o_scales scales = weight.view();
+    nf4o_linear_input_backward(upstream.data(), weight.codes.data(), &scales,
+                               gradient.data(), rows, weight.input_width,
+                               weight.output_width, weight.block_size);
+    return gradient;
+}
+
+// ---- tests ---------------------------------------------------------------
+
+void test_identity() {
+    using riftco_transformer::execution_backend_name;
+    require(static_cast<int>(ExecutionBackend::Cpu) == 0 &&
+                static_cast<int>(ExecutionBackend::Metal) == 1 &&
+                static_cast<int>(ExecutionBackend::Cuda) == 2 &&
+                static_cast<int>(ExecutionBackend::Tpu) == 3 &&
+                static_cast<int>(ExecutionBackend::Hip) == 4,
+            "backend identities must keep their numeric values");
+    require(execution_backend_name(ExecutionBackend::Cpu) == "cpu" &&
+                execution_backend_name(ExecutionBackend::Metal) == "metal" &&
+                execution_backend_name(ExecutionBackend::Cuda) == "cuda" &&
+                execution_backend_name(ExecutionBackend::Tpu) == "tpu" &&
+                execution_backend_name(kHip) == "hip",
+            "backend names");
+    const auto unknown = static_cast<ExecutionBackend>(0xFF);
+    require(!riftco_transformer::execution_backend_available(unknown),
+            "an unknown backend is not available");
+    require(riftco_transformer::execution_backend_unavailability_reason(unknown)
+                .empty(),
+            "an unknown backend has no diagnostic");
+    require_throws<std::invalid_argument>(
+        [&] { static_cast<void>(execution_backend_name(unknown)); },
+        "naming an unknown backend must throw", "unknown execution backend");
+    require(backend::find_backend_adapter(unknown) == nullptr,
+            "the registry must not invent adapters");
+    require(&backend::hip_backend_adapter() ==
+                backend::find_backend_adapter(kHip),
+            "the registry serves the process-lifetime hip adapter");
+    require(backend::hip_backend_adapter().name() == "hip", "adapter name");
+}
+
+void test_unavailable() {
+    require(!riftco_transformer::execution_backend_available(kHip),
+            "the hip backend should be unavailable in this mode");
+    require(!riftco_transformer::execution_backend_unavailability_reason(kHip)
+                 .empty(),
+            "an unavailable hip backend must say why");
+    for (const bool double_quantized : {false, true}) {
+        const HostWeight weight =
+            quantize(aligned_weight(), 3, 32, 32, double_quantized, 32);
+        require_throws<std::runtime_error>(
+            [&] { static_cast<void>(to_hip(weight)); },
+            "an unavailable backend must reject packed weight transfer",
+            "unavailable");
+    }
+    require_throws<std::runtime_error>(
+        [&] {
+            static_cast<void>(backend::make_tensor_storage(kHip, 4, 0.0F));
+        },
+        "an unavailable backend must reject tensor storage", "unavailable");
+}
+
+void require_memory_accounting(const backend::QuantizedWeightStorage& storage,
+                               const HostWeight& weight,
+                               const std::string& description) {
+    const std::size_t logical = weight.logical_bytes();
+    const std::size_t fp32_equivalent =
+        weight.output_width * weight.input_width * sizeof(float);
+    const bool mirrored = std::getenv("FAKE_RTHIP_NO_BAR") != nullptr;
+    require(storage.resident_payload_bytes() ==
+                (mirrored ? 2 * logical - (weight.scales.encoding ==
+                                                   backend::Nf4ScaleEncoding::
+                                                       DoubleQuantizedUInt8
+                                               ? sizeof(float)
+                                               : 0)
+                          : logical),
+            description + ": resident bytes must equal the logical payload "
+                          "when HBM is host-visible");
+    require(logical < fp32_equivalent,
+            description + ": packed storage must stay below fp32 size");
+    const auto scales = storage.scale_storage();
+    if (weight.scales.encoding == backend::Nf4ScaleEncoding::Float32) {
+        require(!scales.fp32_scales.empty() &&
+                    scales.quantized_scales.empty() &&
+                    scales.second_level_scales.empty() &&
+                    scales.offset == 0.0F,
+                description + ": legacy NF4 keeps only fp32 block scales");
+    } else {
+        require(scales.fp32_scales.empty() &&
+                    !scales.quantized_scales.empty() &&
+                    !scales.second_level_scales.empty(),
+                description + ": double quantisation keeps encoded scales");
+    }
+}
+
+void require_byte_preserving(const backend::QuantizedWeightStorage& storage,
+                             const HostWeight& weight,
+                             const std::string& description) {
+    const auto codes = storage.packed_codes();
+    require(codes.size() == weight.codes.size() &&
+                std::equal(codes.begin(), codes.end(), weight.codes.begin()),
+            description + ": packed codes must survive the transfer");
+    const auto scales = storage.scale_storage();
+    const auto same_floats = [](std::span<const float> a,
+                                const std::vector<float>& b) {
+        return a.size() == b.size() &&
+               std::memcmp(a.data(), b.data(), b.size() * sizeof(float)) == 0;
+    };
+    require(same_floats(scales.fp32_scales, weight.scales.fp32_scales) &&
+                same_floats(scales.second_level_scales,
+                            weight.scales.second_level_scales) &&
+                scales.quantized_scales.size() ==
+                    weight.scales.quantized_scales.size() &&
+                std::equal(scales.quantized_scales.begin(),
+                           scales.quantized_scales.end(),
+                           weight.scales.quantized_scales.begin()) &&
+                scales.second_level_block_size ==
+                    weight.scales.second_level_block_size &&
+                scales.offset == weight.scales.offset &&
+                scales.encoding == weight.scales.encoding,
+            description + ": scales must survive the transfer bit for bit");
+    require(storage.backend() == kHip, description + ": backend identity");
+    require(storage.packed_codes_native_handle() != nullptr &&
+                storage.primary_scales_native_handle() != nullptr &&
+                (storage.secondary_scales_native_handle() != nullptr) ==
+                    (weight.scales.encoding ==
+                     backend::Nf4ScaleEncoding::DoubleQuantizedUInt8),
+            description + ": native handles");
+}
+
+void run_accelerator_oracle(const std::vector<float>& dense,
+                            std::size_t output_width, std::size_t input_width,
+                            const std::vector<float>& input,
+                            const std::vector<float>& upstream,
+                            bool double_quantized, bool edge_layout) {
+    const std::string description =
+        std::string("hip") + (double_quantized ? " double-quantized" : "") +
+        " NF4 " + (edge_layout ? "edge" : "aligned") + " fixture";
+    const HostWeight weight = quantize(dense, output_width, input_width, 32,
+                                       double_quantized, 32);
+    if (edge_layout) {
+        // odd element count, partial last block, two second-level groups
+        require(weight.codes.size() == (kEdgeWidth * kEdgeWidth + 1) / 2 &&
+                    (weight.codes.back() & 0xF0U) == 0,
+                description + ": canonical odd packed-code tail");
+        require(nf4o_block_count(kEdgeWidth * kEdgeWidth, 32) == 35,
+                description + ": partial last block");
+        if (double_quantized) {
+            require(weight.scales.second_level_scales.size() == 2,
+                    description + ": two second-level groups");
+        }
+    }
+    const auto storage = to_hip(weight);
+    require_byte_preserving(*storage, weight, description);
+    require_memory_accounting(*storage, weight, description);
+    require_close(hip_forward(input, *storage, weight),
+                  oracle_forward(input, weight),
+                  description + " forward must match the CPU oracle");
+    require_close(hip_input_backward(upstream, *storage, weight),
+                  oracle_input_backward(upstream, weight),
+                  description + " input backward must match the CPU oracle");
+    // the frozen weight is untouched by execution
+    require_byte_preserving(*storage, weight, description + " after use");
+}
+
+void test_accelerator_oracle() {
+    for (const bool double_quantized : {false, true}) {
+        run_accelerator_oracle(aligned_weight(), 3, 32, aligned_input(),
+                               aligned_upstream(), double_quantized, false);
+        run_accelerator_oracle(edge_weight(), kEdgeWidth, kEdgeWidth,
+                               edge_input(), edge_upstream(), double_quantized,
+                               true);
+    }
+}
+
+void test_transformer_sized_layer() {
+    // [768 x 256], block 64: rows 1 (decode kernel) and 16 (tiled kernel).
+    const std::vector<float> dense = pseudo_normal(768 * 256, 0.02F, 1);
+    for (const bool double_quantized : {false, true}) {
+        const HostWeight weight =
+            quantize(dense, 768, 256, 64, double_quantized, 256);
+        const auto storage = to_hip(weight);
+        require_memory_accounting(*storage, weight, "layer");
+        for (const std::size_t rows : {std::size_t{1}, std::size_t{16}}) {
+            const auto input = pseudo_normal(rows * 256, 1.0F, 2);
+            const auto upstream = pseudo_normal(rows * 768, 0.01F, 3);
+            require_close(hip_forward(input, *storage, weight),
+                          oracle_forward(input, weight), "layer forward");
+            require_close(hip_input_backward(upstream, *storage, weight),
+                          oracle_input_backward(upstream, weight),
+                          "layer input backward");
+        }
+    }
+}
+
+void test_tensor_storage() {
+    auto filled = backend::make_tensor_storage(kHip, 5, 1.5F);
+    require(filled->backend() == kHip && filled->size() == 5 &&
+                filled->native_handle() != nullptr,
+            "filled tensor storage identity");
+    for (const float value : std::as_const(*filled).data()) {
+        require(value == 1.5F, "fill value must reach the host view");
+    }
+    auto copy = filled->clone();
+    filled->data()[2] = -7.0F;  // a host write through the mutable span
+    require(std::as_const(*copy).data()[2] == 1.5F &&
+                copy->native_handle() != filled->native_handle(),
+            "a clone owns separate storage");
+
+    // a host write must be seen by the next kernel that reads the tensor
+    const HostWeight weight = quantize(aligned_weight(), 3, 32, 32, false, 32);
+    const auto storage = to_hip(weight);
+    std::vector<float> input = aligned_input();
+    auto source = backend::make_tensor_storage(kHip, input);
+    auto target = backend::make_tensor_storage(kHip, 2 * 3, 0.0F);
+    source->data()[5] = 3.25F;
+    input[5] = 3.25F;
+    backend::dispatch_quantized_linear_forward(
+        kHip, {*source, *storage, *target, {2, 32, 3, 32}});
+    require_close(std::as_const(*target).data(), oracle_forward(input, weight),
+                  "kernels must see host writes made through data()");
+}
+
+void test_dispatch_validation() {
+    const HostWeight weight = quantize(aligned_weight(), 3, 32, 32, false, 32);
+    const auto storage = to_hip(weight);
+    auto input = backend::make_tensor_storage(kHip, aligned_input());
+    auto output = backend::make_tensor_storage(kHip, 2 * 3, 0.0F);
+    const backend::QuantizedLinearDimensions good{2, 32, 3, 32};
+
+    {
+        // a square weight, so that one tensor fits both roles
+        const HostWeight square = quantize(pseudo_normal(32 * 32, 0.02F, 9),
+                                           32, 32, 32, false, 32);
+        const auto square_storage = to_hip(square);
+        require_throws<std::invalid_argument>(
+            [&] {
+                backend::dispatch_quantized_linear_forward(
+                    kHip,
+                    {*input, *square_storage, *input, {2, 32, 32, 32}});
+            },
+            "input and output must not alias", "must not alias");
+        require_throws<std::invalid_argument>(
+            [&] {
+                backend::dispatch_quantized_linear_input_backward(
+                    kHip,
+                    {*input, *square_storage, *input, {2, 32, 32, 32}});
+            },
+            "upstream and gradient must not alias", "must not alias");
+    }
+    require_throws<std::invalid_argument>(
+        [&] {
+            backend::dispatch_quantized_linear_forward(
+                kHip, {*input, *storage, *output, {0, 32, 3, 32}});
+        },
+        "zero rows must be rejected", "positive");
+    require_throws<std::logic_error>(
+        [&] {
+            backend::dispatch_quantized_linear_forward(
+                kHip, {*input, *storage, *output, {3, 32, 3, 32}});
+        },
+        "tensor size must match the dimensions");
+    require_throws<std::logic_error>(
+        [&] {
+            backend::dispatch_quantized_linear_forward(
+                kHip, {*input, *storage, *output, {2, 16, 3, 32}});
+        },
+        "tensor/weight size must match the dimensions");
+    require_throws<std::invalid_argument>(
+        [&] {
+            backend::dispatch_quantized_linear_forward(
+                static_cast<ExecutionBackend>(0xFF),
+                {*input, *storage, *output, good});
+        },
+        "unknown backend", "unknown execution backend");
+    require_throws<std::runtime_error>(
+        [&] {
+            backend::dispatch_quantized_linear_forward(
+                ExecutionBackend::Cuda, {*input, *storage, *output, good});
+        },
+        "a backend that is not part of the build is unavailable",
+        "cuda execution backend is unavailable");
+
+    // storage construction validates the payload before anything is uploaded
+    require_throws<std::invalid_argument>(
+        [&] {
+            static_cast<void>(backend::make_nf4_weight_storage(
+                kHip, {}, weight.scales));
+        },
+        "empty codes", "must not be empty");
+    require_throws<std::invalid_argument>(
+        [&] {
+            backend::Nf4ScaleStorageData scales = weight.scales;
+            scales.fp32_scales[1] = -1.0F;
+            static_cast<void>(backend::make_nf4_weight_storage(
+                kHip, weight.codes, std::move(scales)));
+        },
+        "negative scale", "finite and non-negative");
+    require_throws<std::invalid_argument>(
+        [&] {
+            backend::Nf4ScaleStorageData scales = weight.scales;
+            scales.offset = 1.0F;
+            static_cast<void>(backend::make_nf4_weight_storage(
+                kHip, weight.codes, std::move(scales)));
+        },
+        "legacy representation with an offset", "invalid representation");
+    require_throws<std::invalid_argument>(
+        [&] {
+            backend::Nf4ScaleStorageData scales;
+            scales.encoding = backend::Nf4ScaleEncoding::DoubleQuantizedUInt8;
+            scales.quantized_scales = {128, 128, 128};
+            scales.second_level_scales = {0.0F};
+            scales.second_level_block_size = 48;
+            static_cast<void>(backend::make_nf4_weight_storage(
+                kHip, weight.codes, std::move(scales)));
+        },
+        "unsupported second-level block", "invalid representation");
+}
+
+void test_out_of_memory_maps_to_bad_alloc() {
+    // Only the fake runtime can be told to fail an allocation.
+    if (std::getenv("FAKE_RTHIP_CAN_FAIL") == nullptr) {
+        return;
+    }
+    setenv("FAKE_RTHIP_OUT_OF_MEMORY", "1", 1);
+    require_throws<std::bad_alloc>(
+        [&] {
+            static_cast<void>(backend::make_tensor_storage(kHip, 16, 0.0F));
+        },
+        "device out-of-memory must surface as std::bad_alloc");
+    unsetenv("FAKE_RTHIP_OUT_OF_MEMORY");
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+    try {
+        const bool expect_unavailable =
+            argc == 2 && std::string_view(argv[1]) == "--expect-unavailable";
+        if (argc > 2 || (argc == 2 && !expect_unavailable)) {
+            throw std::invalid_argument(
+                "usage: test_hip_backend [--expect-unavailable]");
+        }
+        test_identity();
+        const bool available =
+            riftco_transformer::execution_backend_available(kHip);
+        if (expect_unavailable) {
+            test_unavailable();
+            std::cout << "hip backend tests passed (unavailable path: "
+                      << riftco_transformer::
+                             execution_backend_unavailability_reason(kHip)
+                      << ")\n";
+            return 0;
+        }
+        if (!available) {
+            const char* required =
+                std::getenv("RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP");
+            require(required == nullptr || std::string_view(required) != "1",
+                    "hip backend tests require an available backend: " +
+                        std::string(riftco_transformer::
+                                        execution_backend_unavailability_reason(
+                                            kHip)));
+            test_unavailable();
+            std::cout << "hip backend tests passed (backend unavailable)\n";
+            return 0;
+        }
+        test_accelerator_oracle();
+        test_transformer_sized_layer();
+        test_tensor_storage();
+        test_dispatch_validation();
+        test_out_of_memory_maps_to_bad_alloc();
+        std::cout << "hip backend tests passed\n";
+        return 0;
+    } catch (const std::exception& error) {
+        std::cerr << "hip backend test failure: " << error.what() << '\n';
+        return 1;
+    }
+}

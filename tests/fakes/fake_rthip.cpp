@@ -1,0 +1,268 @@
+// TEST INFRASTRUCTURE ONLY: a host-only implementation of the kernel C ABI
+// (include/rthip.h) so that the `hip` adapter, the dispatcher's validation,
+// storage accounting and error mapping can be exercised on a machine without a
+// GPU.  "Device memory" is host memory and the two products are computed by the
+// CPU oracle.  It plays the role tests/fakes/fake_pjrt_tpu.cpp plays for the
+// reference's TPU adapter.  The product never loads this library by itself: a
+// test selects it with RIFTCO_TRANSFORMER_HIP_LIBRARY, and
+// RIFTCO_TRANSFORMER_HIP_REJECT_TEST_PLUGIN=1 makes the adapter refuse it (it
+// is recognised by the marker symbol below).
+
+#include "../../include/rthip.h"
+#include "../../oracle/nf4_oracle.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+extern "C" void nf4o_linear_forward_rowcached(
+    const float*, const uint8_t*, const nf4o_scales*, float*, size_t, size_t,
+    size_t, size_t);
+extern "C" void nf4o_linear_input_backward_rowcached(
+    const float*, const uint8_t*, const nf4o_scales*, float*, size_t, size_t,
+    size_t, size_t);
+
+namespace {
+
+thread_local char g_error[256] = "";
+
+rthip_status fail(rthip_status status, const char* message) {
+    std::snprintf(g_error, sizeof(g_error), "%s", message);
+    return status;
+}
+
+bool supported_block(uint64_t block) {
+    for (uint64_t candidate = 32; candidate <= 4096; candidate *= 2) {
+        if (block == candidate) {
+            return true;
+        }
+    }
+    return false;
+}
+
+// Rebuilds the oracle's scale view from the six ABI values.
+rthip_status make_scales(const void* primary, const float* secondary,
+                         int32_t encoding, uint64_t second_level_block,
+                         float offset, size_t block_count,
+                         nf4o_scales* scales) {
+    std::memset(scales, 0, sizeof(*scales));
+    scales->encoding = encoding;
+    if (primary == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "primary scales must not be null");
+    }
+    if (encoding == RTHIP_NF4_SCALE_FLOAT32) {
+        scales->fp32_scales = static_cast<const float*>(primary);
+        scales->fp32_count = block_count;
+        return RTHIP_OK;
+    }
+    if (encoding != RTHIP_NF4_SCALE_DOUBLE_QUANTIZED_UINT8) {
+        return fail(RTHIP_INVALID_ARGUMENT, "unknown NF4 scale encoding");
+    }
+    if (!supported_block(second_level_block) || secondary == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "invalid double-quantized scale description");
+    }
+    scales->quantized_scales = static_cast<const uint8_t*>(primary);
+    scales->quantized_count = block_count;
+    scales->second_level = secondary;
+    scales->second_level_count =
+        (block_count + second_level_block - 1) / second_level_block;
+    scales->second_level_block = second_level_block;
+    scales->offset = offset;
+    return RTHIP_OK;
+}
+
+rthip_status check_dimensions(uint64_t rows, uint64_t input_width,
+                              uint64_t output_width, uint64_t block_size) {
+    if (rows == 0 || input_width == 0 || output_width == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "quantized linear dimensions must be positive");
+    }
+    if (!supported_block(block_size)) {
+        return fail(RTHIP_INVALID_ARGUMENT, "unsupported NF4 block size");
+    }
+    return RTHIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+// Recognised by the adapter's test-plugin gate.
+int rthip_test_plugin_marker = 1;
+
+uint32_t rthip_abi_version(void) {
+    return (RTHIP_ABI_VERSION_MAJOR << 16) | RTHIP_ABI_VERSION_MINOR;
+}
+const char* rthip_last_error(void) { return g_error; }
+
+rthip_status rthip_device_count(int32_t* count) {
+    if (std::getenv("FAKE_RTHIP_NO_DEVICE") != nullptr) {
+        *count = 0;
+        return fail(RTHIP_UNAVAILABLE, "no HIP device is visible (fake)");
+    }
+    *count = 1;
+    return RTHIP_OK;
+}
+rthip_status rthip_device_description(char* buffer, size_t capacity) {
+    std::snprintf(buffer, capacity, "host-only test runtime");
+    return RTHIP_OK;
+}
+rthip_status rthip_device_memory_host_visible(int32_t* visible) {
+    *visible = std::getenv("FAKE_RTHIP_NO_BAR") != nullptr ? 0 : 1;
+    return RTHIP_OK;
+}
+
+rthip_status rthip_malloc(void** pointer, size_t bytes) {
+    *pointer = nullptr;
+    if (bytes == 0) {
+        return RTHIP_OK;
+    }
+    if (std::getenv("FAKE_RTHIP_OUT_OF_MEMORY") != nullptr) {
+        return fail(RTHIP_OUT_OF_MEMORY, "device allocation: out of memory");
+    }
+    *pointer = std::aligned_alloc(256, (bytes + 255) / 256 * 256);
+    return *pointer != nullptr ? RTHIP_OK
+                               : fail(RTHIP_OUT_OF_MEMORY, "out of memory");
+}
+rthip_status rthip_free(void* pointer) {
+    std::free(pointer);
+    return RTHIP_OK;
+}
+rthip_status rthip_copy_to_device(void* device, const void* host,
+                                  size_t bytes) {
+    std::memcpy(device, host, bytes);
+    return RTHIP_OK;
+}
+rthip_status rthip_copy_to_host(void* host, const void* device, size_t bytes) {
+    std::memcpy(host, device, bytes);
+    return RTHIP_OK;
+}
+rthip_status rthip_fill_f32(float* device, float value, uint64_t count,
+                            void*) {
+    for (uint64_t index = 0; index < count; ++index) {
+        device[index] = value;
+    }
+    return RTHIP_OK;
+}
+rthip_status rthip_stream_synchronize(void*) { return RTHIP_OK; }
+
+rthip_status rthip_nf4_select_algorithm(int32_t, uint64_t rows,
+                                        uint64_t input_width,
+                                        uint64_t output_width,
+                                        uint64_t block_size,
+                                        int32_t* algorithm) {
+    if (const rthip_status status =
+            check_dimensions(rows, input_width, output_width, block_size);
+        status != RTHIP_OK) {
+        return status;
+    }
+    *algorithm = RTHIP_NF4_ALGORITHM_GENERIC;
+    return RTHIP_OK;
+}
+
+rthip_status rthip_nf4_linear_forward(
+    const float* x, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, const float* bias_or_null,
+    float* y, uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void*) {
+    if (x == nullptr || y == nullptr || codes == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "null tensor pointer");
+    }
+    if (const rthip_status status =
+            check_dimensions(rows, input_width, output_width, block_size);
+        status != RTHIP_OK) {
+        return status;
+    }
+    const size_t blocks =
+        (output_width * input_width + block_size - 1) / block_size;
+    nf4o_scales scales;
+    if (const rthip_status status =
+            make_scales(primary_scales, secondary_scales, encoding,
+                        second_level_block, offset, blocks, &scales);
+        status != RTHIP_OK) {
+        return status;
+    }
+    nf4o_linear_forward_rowcached(x, codes, &scales, y, rows, input_width,
+                                  output_width, block_size);
+    if (bias_or_null != nullptr) {
+        nf4o_add_bias(y, bias_or_null, rows, output_width);
+    }
+    return RTHIP_OK;
+}
+
+rthip_status rthip_nf4_linear_input_backward(
+    const float* dy, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, float* dx, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size, void*) {
+    if (dy == nullptr || dx == nullptr || codes == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "null tensor pointer");
+    }
+    if (const rthip_status status =
+            check_dimensions(rows, input_width, output_width, block_size);
+        status != RTHIP_OK) {
+        return status;
+    }
+    const size_t blocks =
+        (output_width * input_width + block_size - 1) / block_size;
+    nf4o_scales scales;
+    if (const rthip_status status =
+            make_scales(primary_scales, secondary_scales, encoding,
+                        second_level_block, offset, blocks, &scales);
+        status != RTHIP_OK) {
+        return status;
+    }
+    nf4o_linear_input_backward_rowcached(dy, codes, &scales, dx, rows,
+                                         input_width, output_width,
+                                         block_size);
+    return RTHIP_OK;
+}
+
+rthip_status rthip_nf4_linear_forward_with(
+    int32_t, const float* x, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, const float* bias_or_null,
+    float* y, uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream) {
+    return rthip_nf4_linear_forward(x, codes, primary_scales, secondary_scales,
+                                    encoding, second_level_block, offset,
+                                    bias_or_null, y, rows, input_width,
+                                    output_width, block_size, stream);
+}
+
+rthip_status rthip_nf4_linear_input_backward_with(
+    int32_t, const float* dy, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset, float* dx,
+    uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream) {
+    return rthip_nf4_linear_input_backward(
+        dy, codes, primary_scales, secondary_scales, encoding,
+        second_level_block, offset, dx, rows, input_width, output_width,
+        block_size, stream);
+}
+
+rthip_status rthip_nf4_dequantize(
+    const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, float* out,
+    uint64_t element_count, uint64_t block_size, void*) {
+    if (out == nullptr || codes == nullptr || element_count == 0 ||
+        !supported_block(block_size)) {
+        return fail(RTHIP_INVALID_ARGUMENT, "invalid dequantize arguments");
+    }
+    const size_t blocks = (element_count + block_size - 1) / block_size;
+    nf4o_scales scales;
+    if (const rthip_status status =
+            make_scales(primary_scales, secondary_scales, encoding,
+                        second_level_block, offset, blocks, &scales);
+        status != RTHIP_OK) {
+        return status;
+    }
+    nf4o_dequantize(codes, &scales, element_count, block_size, out);
+    return RTHIP_OK;
+}
+
+}  // extern "C"

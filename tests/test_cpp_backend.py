@@ -1,0 +1,97 @@
+"""Runs the C++ tests of the `hip` backend adapter (tests/cpp).
+
+Without a GPU the adapter is exercised against the host-only test runtime
+(tests/fakes/fake_rthip.cpp, a stand-in for librthip.so that computes with the
+CPU oracle): storage accounting, byte-preserving transfer, dispatcher
+validation, error mapping and the unavailable paths.  With a GPU the same
+binary runs against the real library, with test plugins refused.
+
+The binaries are built beforehand by `make -C tests/cpp` (which
+__graft_entry__.build() runs); a missing binary is a failure, not a skip.
+"""
+import os
+import subprocess
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+BUILD = os.path.join(HERE, "cpp", "build")
+BINARY = os.path.join(BUILD, "test_hip_backend")
+FAKE = os.path.join(BUILD, "librthip_fake.so")
+CONFORMANCE = os.path.join(BUILD, "test_in_tree_conformance")
+
+
+def run(arguments=(), **environment):
+    env = {k: v for k, v in os.environ.items()
+           if not k.startswith(("RIFTCO_TRANSFORMER_", "FAKE_RTHIP_"))}
+    env.update(environment)
+    assert os.path.exists(BINARY), \
+        "tests/cpp/build/test_hip_backend is not built (make -C tests/cpp)"
+    return subprocess.run([BINARY, *arguments], env=env, capture_output=True,
+                          text=True, timeout=300)
+
+
+def expect_pass(result, fragment="hip backend tests passed"):
+    assert result.returncode == 0, result.stdout + result.stderr
+    assert fragment in result.stdout
+
+
+def test_adapter_on_the_host_only_runtime():
+    expect_pass(run(RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE,
+                    RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1",
+                    FAKE_RTHIP_CAN_FAIL="1"))
+
+
+def test_adapter_keeps_a_counted_mirror_without_host_visible_memory():
+    expect_pass(run(RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE,
+                    RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1",
+                    FAKE_RTHIP_NO_BAR="1"))
+
+
+def test_unavailable_when_the_runtime_sees_no_device():
+    result = run(["--expect-unavailable"],
+                 RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE, FAKE_RTHIP_NO_DEVICE="1")
+    expect_pass(result, "no HIP device is visible")
+
+
+def test_unavailable_when_the_library_is_missing():
+    result = run(["--expect-unavailable"],
+                 RIFTCO_TRANSFORMER_HIP_LIBRARY="/nonexistent/librthip.so")
+    expect_pass(result, "cannot load the HIP runtime library")
+
+
+def test_hardware_gate_refuses_the_test_plugin():
+    result = run(["--expect-unavailable"],
+                 RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE,
+                 RIFTCO_TRANSFORMER_HIP_REJECT_TEST_PLUGIN="1")
+    expect_pass(result, "test plugins are rejected")
+
+
+def test_required_hardware_turns_unavailable_into_failure():
+    result = run(RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE, FAKE_RTHIP_NO_DEVICE="1",
+                 RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1")
+    assert result.returncode == 1
+    assert "require an available backend" in result.stderr
+
+
+def test_in_tree_conformance_against_the_reference_headers():
+    """hip_adapter.cpp compiled against the reference's own BackendAdapter and
+    linked with the reference's own objects; built only where the reference
+    tree exists."""
+    if not os.path.exists(CONFORMANCE):
+        pytest.skip("built only where /root/reference is present")
+    env = dict(os.environ, RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE)
+    result = subprocess.run([CONFORMANCE], env=env, capture_output=True,
+                            text=True, timeout=300)
+    assert result.returncode == 0, result.stdout + result.stderr
+    assert "in-tree conformance tests passed" in result.stdout
+
+
+@pytest.mark.gpu
+def test_adapter_on_the_real_library():
+    """The same binary against librthip.so on a real MI355X: kernels, device
+    storage served through the PCIe BAR, resident == logical bytes."""
+    result = run(RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1",
+                 RIFTCO_TRANSFORMER_HIP_REJECT_TEST_PLUGIN="1")
+    expect_pass(result)
+    assert "unavailable" not in result.stdout
