@@ -273,6 +273,10 @@ def main():
     parser.add_argument("--skip-extras", action="store_true",
                         help="only the headline decode workload")
     parser.add_argument("--skip-cpu", action="store_true")
+    parser.add_argument("--traffic-calibration", action="store_true",
+                        help="for rocprofv3 --pmc runs: a 1 GiB elementwise "
+                             "copy of known traffic, then one decode step "
+                             "launched kernel by kernel, nothing else")
     parser.add_argument("--no-graph", action="store_true",
                         help="launch the decode kernels one by one from "
                              "Python instead of replaying a HIP graph")
@@ -287,6 +291,20 @@ def main():
     library = package.load_library()
     if not torch.cuda.is_available() or not library.is_available():
         sys.exit("bench.py: no usable MI355X: " + library.last_error())
+
+    if arguments.traffic_calibration:
+        # torch's elementwise kernel reads 2^30 B and writes 2^30 B per call:
+        # the yardstick for FETCH_SIZE / WRITE_SIZE readings.
+        source = torch.zeros(2 ** 28, device="cuda")
+        target = torch.empty_like(source)
+        for _ in range(3):
+            torch.add(source, 1.0, out=target)
+        torch.cuda.synchronize()
+        bench_decode(package, device, torch, arguments.layers, 1, 0, False)
+        print(json.dumps({"traffic_calibration": "done",
+                          "copy_bytes_read": 2 ** 30,
+                          "copy_bytes_written": 2 ** 30}))
+        return
 
     decode = bench_decode(package, device, torch, arguments.layers,
                           arguments.steps, arguments.warmup,
