@@ -75,7 +75,10 @@ enum {
     /* wavefront-reduced streaming GEMV for small row counts (HBM-bound) */
     RTHIP_NF4_ALGORITHM_GEMV = 2,
     /* LDS-tiled fp32 MFMA GEMM with dequantisation fused into the tile load */
-    RTHIP_NF4_ALGORITHM_MFMA = 3
+    RTHIP_NF4_ALGORITHM_MFMA = 3,
+    /* small batches (forward, up to 64 rows): weights decoded straight into
+     * MFMA operands, no LDS tile */
+    RTHIP_NF4_ALGORITHM_SKINNY = 4
 };
 
 /* ---- library / device ------------------------------------------------- */

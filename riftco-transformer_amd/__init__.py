@@ -10,6 +10,7 @@ from .binding import (  # noqa: F401
     ALGORITHM_GENERIC,
     ALGORITHM_MFMA,
     ALGORITHM_NAMES,
+    ALGORITHM_SKINNY,
     EXPORTED_SYMBOLS,
     FORWARD,
     INPUT_BACKWARD,

@@ -29,7 +29,9 @@ ALGORITHM_AUTO = 0
 ALGORITHM_GENERIC = 1
 ALGORITHM_GEMV = 2
 ALGORITHM_MFMA = 3
-ALGORITHM_NAMES = {0: "auto", 1: "generic", 2: "gemv", 3: "mfma"}
+ALGORITHM_SKINNY = 4
+ALGORITHM_NAMES = {0: "auto", 1: "generic", 2: "gemv", 3: "mfma",
+                   4: "skinny"}
 
 FORWARD = 0
 INPUT_BACKWARD = 1

@@ -41,6 +41,12 @@ constexpr std::size_t kGemvMaxRows = 4;
 bool gemv_forward_supports(const LinearProblem& problem);
 void launch_gemv_forward(const LinearProblem& problem, hipStream_t stream);
 
+// nf4_skinny.hip -- forward only, up to 64 rows, decode straight into MFMA
+// operands.
+constexpr std::size_t kSkinnyMaxRows = 64;
+bool skinny_forward_supports(const LinearProblem& problem);
+void launch_skinny_forward(const LinearProblem& problem, hipStream_t stream);
+
 // nf4_mfma.hip
 bool mfma_forward_supports(const LinearProblem& problem);
 void launch_mfma_forward(const LinearProblem& problem, hipStream_t stream);

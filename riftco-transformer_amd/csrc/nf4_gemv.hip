@@ -46,6 +46,7 @@
 
 #include "kernels.hpp"
 #include "nf4_decode.hpp"
+#include "nf4_pair_table.hpp"
 
 namespace rthip {
 namespace {
@@ -53,8 +54,6 @@ namespace {
 constexpr int kWave = 64;
 constexpr int kTeamThreads = 256;  // threads that share one weight row
 constexpr int kSegment = 16;       // weights per thread per row visit
-constexpr int kReplicas = 16;      // interleaved copies of the pair table
-constexpr int kEntryStride = 256;  // bytes between table entries
 constexpr int kRowLanes = 16;      // lanes of one DPP row
 constexpr int kTeamDppRows = kTeamThreads / kRowLanes;
 constexpr unsigned kComputeUnits = 256;
@@ -65,71 +64,6 @@ constexpr unsigned kMaxIterations = 8;  // batches per team kept in LDS
 #ifndef RTHIP_GEMV_ROWS
 #define RTHIP_GEMV_ROWS 4
 #endif
-
-// codebook[n] selected with compare/select on instruction literals (no memory
-// access, so it cannot stall behind the streaming loads).
-__device__ __forceinline__ float codebook_literal(unsigned n) {
-    const float lo0 = (n & 1U) ? -0.6961928009986877F : -1.0F;
-    const float lo1 = (n & 1U) ? -0.39491748809814453F : -0.5250730514526367F;
-    const float lo2 = (n & 1U) ? -0.18477343022823334F : -0.28444138169288635F;
-    const float lo3 = (n & 1U) ? 0.0F : -0.09105003625154495F;
-    const float hi0 = (n & 1U) ? 0.16093020141124725F : 0.07958029955625534F;
-    const float hi1 = (n & 1U) ? 0.33791524171829224F : 0.24611230194568634F;
-    const float hi2 = (n & 1U) ? 0.5626170039176941F : 0.44070982933044434F;
-    const float hi3 = (n & 1U) ? 1.0F : 0.7229568362236023F;
-    const float a = (n & 2U) ? lo1 : lo0;
-    const float b = (n & 2U) ? lo3 : lo2;
-    const float c = (n & 2U) ? hi1 : hi0;
-    const float d = (n & 2U) ? hi3 : hi2;
-    const float low = (n & 4U) ? b : a;
-    const float high = (n & 4U) ? d : c;
-    return (n & 8U) ? high : low;
-}
-
-// Level of nibble 4 * quarter + i (i is a compile-time constant).
-template <int kIndex>
-__device__ __forceinline__ float level_in_quarter(unsigned quarter) {
-    constexpr float kLevels[16] = {
-        -1.0F, -0.6961928009986877F, -0.5250730514526367F,
-        -0.39491748809814453F, -0.28444138169288635F, -0.18477343022823334F,
-        -0.09105003625154495F, 0.0F, 0.07958029955625534F,
-        0.16093020141124725F, 0.24611230194568634F, 0.33791524171829224F,
-        0.44070982933044434F, 0.5626170039176941F, 0.7229568362236023F, 1.0F};
-    const float low = (quarter & 1U) ? kLevels[4 + kIndex] : kLevels[kIndex];
-    const float high =
-        (quarter & 1U) ? kLevels[12 + kIndex] : kLevels[8 + kIndex];
-    return (quarter & 2U) ? high : low;
-}
-
-// Builds the replicated pair table with all kThreads threads of the
-// workgroup.  A thread fills one replica of 4096 / kThreads consecutive
-// entries, in groups of four that share a high nibble and a low-nibble
-// quarter.
-template <int kThreads>
-__device__ __forceinline__ void build_pair_table(char* table) {
-    constexpr int kEntries = 256 * kReplicas / kThreads;  // per thread
-    static_assert(kEntries >= 4 && kEntries % 4 == 0);
-    const unsigned replica = threadIdx.x % kReplicas;
-    const unsigned first_entry = (threadIdx.x / kReplicas) * kEntries;
-    char* slot = table + replica * sizeof(float2);
-#pragma unroll
-    for (int group = 0; group < kEntries / 4; ++group) {
-        const unsigned entry = first_entry + 4 * group;
-        const float high_level = codebook_literal(entry >> 4);
-        const unsigned quarter = (entry >> 2) & 3U;
-        float2* target =
-            reinterpret_cast<float2*>(slot + entry * kEntryStride);
-        constexpr int kStep = kEntryStride / sizeof(float2);
-        target[0 * kStep] =
-            make_float2(level_in_quarter<0>(quarter), high_level);
-        target[1 * kStep] =
-            make_float2(level_in_quarter<1>(quarter), high_level);
-        target[2 * kStep] =
-            make_float2(level_in_quarter<2>(quarter), high_level);
-        target[3 * kStep] =
-            make_float2(level_in_quarter<3>(quarter), high_level);
-    }
-}
 
 // value of lane (l ^ kXor) within the 16-lane DPP row, vector ALU only.
 template <int kXor>
@@ -240,7 +174,7 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
 ) {
     constexpr int kThreads = kTeamThreads * kTeams;
     constexpr int kValues = kRows * kX;
-    __shared__ __attribute__((aligned(256))) char table[256 * kEntryStride];
+    __shared__ __attribute__((aligned(256))) char table[kPairTableBytes];
     __shared__ float partial[kTeams][kMaxIterations][kTeamDppRows][kValues];
 
     const unsigned team =
@@ -345,10 +279,7 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
     build_pair_table<kThreads>(table);
     __syncthreads();
 
-    const unsigned lane_bits = (lane % kReplicas) * sizeof(float2);  // < 128
-    // v_perm_b32 selectors: (byte b of the code word) << 8 | lane_bits.
-    constexpr unsigned kSelect[4] = {0x0C0C0400U, 0x0C0C0500U, 0x0C0C0600U,
-                                     0x0C0C0700U};
+    const unsigned lane_bits = pair_table_lane_bits(lane);
 
     // One batch: prefetch `next`, compute `current`, reduce, write.
     const auto step = [&](const RowBatch<kRows, kSegments>& current,
@@ -386,10 +317,8 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
                 for (int w = 0; w < 2; ++w) {
 #pragma unroll
                     for (int b = 0; b < 4; ++b) {
-                        const unsigned address = __builtin_amdgcn_perm(
-                            words[w], lane_bits, kSelect[b]);
                         const float2 levels =
-                            *reinterpret_cast<const float2*>(table + address);
+                            pair_table_lookup(table, words[w], b, lane_bits);
 #pragma unroll
                         for (int r = 0; r < kX; ++r) {
                             even[r] += xs[r][j][8 * w + 2 * b] * levels.x;

@@ -178,6 +178,10 @@ int32_t select_forward(const rthip::LinearProblem& problem) {
         rthip::gemv_forward_supports(problem)) {
         return RTHIP_NF4_ALGORITHM_GEMV;
     }
+    if (problem.rows <= rthip::kSkinnyMaxRows &&
+        rthip::skinny_forward_supports(problem)) {
+        return RTHIP_NF4_ALGORITHM_SKINNY;
+    }
     if (rthip::mfma_forward_supports(problem)) {
         return RTHIP_NF4_ALGORITHM_MFMA;
     }
@@ -398,6 +402,15 @@ rthip_status rthip_nf4_linear_forward_with(
         }
         rthip::launch_mfma_forward(problem, hip_stream);
         break;
+    case RTHIP_NF4_ALGORITHM_SKINNY:
+        if (!rthip::skinny_forward_supports(problem)) {
+            return fail(RTHIP_UNSUPPORTED,
+                        "the small-batch family needs rows <= %zu, a row "
+                        "width that is a multiple of 64 and aligned pointers",
+                        rthip::kSkinnyMaxRows);
+        }
+        rthip::launch_skinny_forward(problem, hip_stream);
+        break;
     default:
         return fail(RTHIP_INVALID_ARGUMENT, "unknown algorithm %d",
                     static_cast<int>(algorithm));
@@ -475,8 +488,9 @@ rthip_status rthip_nf4_linear_input_backward_with(
         rthip::launch_mfma_input_backward(problem, hip_stream);
         break;
     case RTHIP_NF4_ALGORITHM_GEMV:
+    case RTHIP_NF4_ALGORITHM_SKINNY:
         return fail(RTHIP_UNSUPPORTED,
-                    "the GEMV family implements the forward product only");
+                    "this family implements the forward product only");
     default:
         return fail(RTHIP_INVALID_ARGUMENT, "unknown algorithm %d",
                     static_cast<int>(algorithm));

@@ -41,7 +41,12 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(fwd, 1, 11008, 4096, 64) == package.ALGORITHM_GEMV
     # prefill / training -> MFMA GEMM, both directions
     assert select(fwd, 2048, 4096, 11008, 64) == package.ALGORITHM_MFMA
-    assert select(fwd, 16, 256, 768, 64) == package.ALGORITHM_MFMA
+    # small batches -> weights decoded straight into MFMA operands
+    assert select(fwd, 16, 256, 768, 64) == package.ALGORITHM_SKINNY
+    assert select(fwd, 64, 4096, 11008, 64) == package.ALGORITHM_SKINNY
+    assert select(fwd, 65, 4096, 11008, 64) == package.ALGORITHM_MFMA
+    assert select(fwd, 16, 96, 768, 32) == package.ALGORITHM_SKINNY
+    assert select(fwd, 16, 40, 768, 32) == package.ALGORITHM_GENERIC
     assert select(bwd, 2048, 4096, 11008, 64) == package.ALGORITHM_MFMA
     assert select(bwd, 2048, 11008, 4096, 64) == package.ALGORITHM_MFMA
     # the reference's edge layout -> shape-agnostic kernels

@@ -49,7 +49,7 @@ def families(package):
     """AUTO plus every pinned kernel family; a family that does not accept a
     shape answers RTHIP_UNSUPPORTED and is skipped by `run`."""
     return (None, package.ALGORITHM_GENERIC, package.ALGORITHM_GEMV,
-            package.ALGORITHM_MFMA)
+            package.ALGORITHM_MFMA, package.ALGORITHM_SKINNY)
 
 
 def run(package, function, *args, algorithm):
