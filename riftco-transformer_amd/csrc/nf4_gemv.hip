@@ -209,12 +209,6 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
             const unsigned row_block = row_start >> block_shift;
 #pragma unroll
             for (int j = 0; j < kSegments; ++j) {
-#ifdef RTHIP_GEMV_DEBUG_NOLOAD
-                batch.codes[row][j].x = thread * 2654435761u + row_start;
-                batch.codes[row][j].y = thread * 40503u + row_start;
-                batch.scales[row][j] = 1.0F;
-                continue;
-#endif
                 batch.codes[row][j] = __builtin_amdgcn_raw_buffer_load_b64(
                     code_buffer, segment_weights[j] >> 1, row_start >> 1, 0);
                 const unsigned segment_block =
@@ -290,9 +284,35 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
             load_batch(next, batch_index + stride);
         }
 
+        // Table lookups run one weight row ahead of the multiply-adds that
+        // consume them: a row's 8 * kSegments ds_read_b64 are all in flight
+        // while the previous row is accumulated, which keeps the LDS queue
+        // deep enough to stream at its full rate.
+        float2 levels[2][kSegments][8];
+        const auto look_up = [&](int row, float2 (&out)[kSegments][8]) {
+#pragma unroll
+            for (int j = 0; j < kSegments; ++j) {
+                const unsigned words[2] = {current.codes[row][j].x,
+                                           current.codes[row][j].y};
+#pragma unroll
+                for (int w = 0; w < 2; ++w) {
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        out[j][4 * w + b] =
+                            pair_table_lookup(table, words[w], b, lane_bits);
+                    }
+                }
+            }
+        };
+
         float acc[kValues];
+        look_up(0, levels[0]);
 #pragma unroll
         for (int row = 0; row < kRows; ++row) {
+            if (row + 1 < kRows) {
+                look_up(row + 1, levels[(row + 1) & 1]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
             float row_acc[kX];
 #pragma unroll
             for (int r = 0; r < kX; ++r) {
@@ -307,26 +327,15 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
                     even[r] = 0.0F;
                     odd[r] = 0.0F;
                 }
-                const unsigned words[2] = {current.codes[row][j].x,
-                                           current.codes[row][j].y};
-#ifdef RTHIP_GEMV_DEBUG_NOCOMPUTE
-                even[0] = __builtin_bit_cast(float, words[0] & 0x3FFFFFFFU);
-                odd[0] = __builtin_bit_cast(float, words[1] & 0x3FFFFFFFU);
-#else
 #pragma unroll
-                for (int w = 0; w < 2; ++w) {
+                for (int p = 0; p < 8; ++p) {
+                    const float2 pair = levels[row & 1][j][p];
 #pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        const float2 levels =
-                            pair_table_lookup(table, words[w], b, lane_bits);
-#pragma unroll
-                        for (int r = 0; r < kX; ++r) {
-                            even[r] += xs[r][j][8 * w + 2 * b] * levels.x;
-                            odd[r] += xs[r][j][8 * w + 2 * b + 1] * levels.y;
-                        }
+                    for (int r = 0; r < kX; ++r) {
+                        even[r] += xs[r][j][2 * p] * pair.x;
+                        odd[r] += xs[r][j][2 * p + 1] * pair.y;
                     }
                 }
-#endif
 #pragma unroll
                 for (int r = 0; r < kX; ++r) {
                     row_acc[r] += (even[r] + odd[r]) * current.scales[row][j];
@@ -336,6 +345,7 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
             for (int r = 0; r < kX; ++r) {
                 acc[row * kX + r] = row_acc[r];
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
 
         // Park this DPP row's totals; nobody waits here.
