@@ -42,10 +42,13 @@ bool gemv_forward_supports(const LinearProblem& problem);
 void launch_gemv_forward(const LinearProblem& problem, hipStream_t stream);
 
 // nf4_skinny.hip -- forward only, up to 64 rows, decode straight into MFMA
-// operands.
+// operands.  Shapes whose output tiles are shared between workgroups use a
+// per-stream workspace that is allocated on first use, so the launcher can
+// fail.
 constexpr std::size_t kSkinnyMaxRows = 64;
 bool skinny_forward_supports(const LinearProblem& problem);
-void launch_skinny_forward(const LinearProblem& problem, hipStream_t stream);
+hipError_t launch_skinny_forward(const LinearProblem& problem,
+                                 hipStream_t stream);
 
 // nf4_mfma.hip
 bool mfma_forward_supports(const LinearProblem& problem);

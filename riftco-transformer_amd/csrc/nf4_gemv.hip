@@ -57,12 +57,16 @@ constexpr int kSegment = 16;       // weights per thread per row visit
 constexpr int kRowLanes = 16;      // lanes of one DPP row
 constexpr int kTeamDppRows = kTeamThreads / kRowLanes;
 constexpr unsigned kComputeUnits = 256;
-constexpr unsigned kMaxIterations = 8;  // batches per team kept in LDS
+// Row totals a team may park in LDS before the final barrier, per DPP row.
+constexpr unsigned kParkedValues = 128;
 #ifndef RTHIP_GEMV_TEAMS
 #define RTHIP_GEMV_TEAMS 2
 #endif
 #ifndef RTHIP_GEMV_ROWS
 #define RTHIP_GEMV_ROWS 4
+#endif
+#ifndef RTHIP_GEMV_DEPTH
+#define RTHIP_GEMV_DEPTH 2
 #endif
 
 // value of lane (l ^ kXor) within the 16-lane DPP row, vector ALU only.
@@ -147,13 +151,6 @@ struct RowBatch {
     float scales[kRows][kSegments];
 };
 
-// Buffer descriptors of one packed weight; sizes are in bytes.
-struct GemvBuffers {
-    unsigned code_bytes;
-    unsigned primary_bytes;
-    unsigned secondary_bytes;
-};
-
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base,
                                                              unsigned bytes) {
     // Raw (untyped, stride 0) buffer with range checking on `bytes`.
@@ -165,15 +162,17 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base,
 // kX: x rows held per thread (1, 2 or 4; a 3-row call runs as 4 with a zero
 // row).  kSegments: segments per thread.  kRows: weight rows per batch.
 // kTeams: teams per workgroup.
-template <int kX, int kSegments, int kRows, int kTeams, bool kDoubleQuantized>
+template <int kX, int kSegments, int kRows, int kTeams, int kDepth,
+          bool kDoubleQuantized>
 __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
-    const float* __restrict__ x, Nf4WeightView weight, GemvBuffers sizes,
+    const float* __restrict__ x, Nf4WeightView weight, unsigned secondary_bytes,
     const float* __restrict__ bias, float* __restrict__ y, unsigned x_rows,
     unsigned input_width, unsigned output_width, unsigned block_shift,
     unsigned batch_count, unsigned iterations
 ) {
     constexpr int kThreads = kTeamThreads * kTeams;
     constexpr int kValues = kRows * kX;
+    constexpr unsigned kMaxIterations = kParkedValues / kValues;
     __shared__ __attribute__((aligned(256))) char table[kPairTableBytes];
     __shared__ float partial[kTeams][kMaxIterations][kTeamDppRows][kValues];
 
@@ -183,12 +182,18 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
     const unsigned lane = thread % kWave;
     const unsigned segment_count = input_width / kSegment;
 
-    const __amdgpu_buffer_rsrc_t code_buffer =
-        make_buffer(weight.codes, sizes.code_bytes);
-    const __amdgpu_buffer_rsrc_t primary_buffer =
-        make_buffer(weight.primary_scales, sizes.primary_bytes);
+    // The hardware range check covers the per-lane offset only, not the
+    // scalar offset, so every weight row gets descriptors of its own: base at
+    // the row's first code byte / first scale, extent one row (zero for rows
+    // past the output width).  They are built with a few scalar instructions
+    // per row; lanes past the row end then read zeros instead of memory
+    // beyond the payload.
+    const unsigned row_code_bytes = input_width / 2;
+    const unsigned row_blocks = input_width >> block_shift;
     const __amdgpu_buffer_rsrc_t secondary_buffer =
-        make_buffer(weight.secondary_scales, sizes.secondary_bytes);
+        make_buffer(weight.secondary_scales, secondary_bytes);
+    const std::uint8_t* const primary_bytes =
+        static_cast<const std::uint8_t*>(weight.primary_scales);
 
     // Per-lane constants: where this thread's segments sit inside a row.  The
     // row width is a multiple of the block size, so a row starts on a block
@@ -199,31 +204,43 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
         segment_weights[j] = (thread + kTeamThreads * j) * kSegment;
     }
 
-    // All indices fit 32 bits (the launcher checks O * I < 2^32).
     const auto load_batch = [&](RowBatch<kRows, kSegments>& batch,
                                 unsigned batch_index) {
 #pragma unroll
         for (int row = 0; row < kRows; ++row) {
             const unsigned o = batch_index * kRows + row;  // scalar
-            const unsigned row_start = o * input_width;
-            const unsigned row_block = row_start >> block_shift;
+            const bool row_valid = o < output_width;
+            const std::size_t row_start =
+                static_cast<std::size_t>(o) * input_width;
+            const std::size_t row_block = row_start >> block_shift;
+            const __amdgpu_buffer_rsrc_t code_row = make_buffer(
+                weight.codes + (row_start >> 1),
+                row_valid ? row_code_bytes : 0U);
+            constexpr unsigned kScaleBytes = kDoubleQuantized ? 1 : 4;
+            const __amdgpu_buffer_rsrc_t primary_row = make_buffer(
+                primary_bytes + row_block * kScaleBytes,
+                row_valid ? row_blocks * kScaleBytes : 0U);
 #pragma unroll
             for (int j = 0; j < kSegments; ++j) {
                 batch.codes[row][j] = __builtin_amdgcn_raw_buffer_load_b64(
-                    code_buffer, segment_weights[j] >> 1, row_start >> 1, 0);
+                    code_row, segment_weights[j] >> 1, 0, 0);
                 const unsigned segment_block =
                     segment_weights[j] >> block_shift;
                 if constexpr (!kDoubleQuantized) {
                     batch.scales[row][j] = __builtin_bit_cast(
                         float, __builtin_amdgcn_raw_buffer_load_b32(
-                                   primary_buffer, segment_block * 4,
-                                   row_block * 4, 0));
+                                   primary_row, segment_block * 4, 0, 0));
                 } else {
                     const std::uint8_t scale_code =
                         __builtin_amdgcn_raw_buffer_load_b8(
-                            primary_buffer, segment_block, row_block, 0);
-                    const unsigned group = (row_block + segment_block) >>
-                                           weight.second_level_shift;
+                            primary_row, segment_block, 0, 0);
+                    // Rows past the output width get an index past the end
+                    // of the table, which reads as zero.
+                    const unsigned group =
+                        row_valid ? static_cast<unsigned>(
+                                        (row_block + segment_block) >>
+                                        weight.second_level_shift)
+                                  : 0x3FFFFFFFU;
                     const float second = __builtin_bit_cast(
                         float, __builtin_amdgcn_raw_buffer_load_b32(
                                    secondary_buffer, group * 4, 0, 0));
@@ -239,9 +256,14 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
     const unsigned stride = gridDim.x * kTeams;
     const unsigned first_batch = blockIdx.x * kTeams + team;
 
-    RowBatch<kRows, kSegments> ping;
-    RowBatch<kRows, kSegments> pong;
-    load_batch(ping, first_batch);
+    // A ring of register batches: batch i lives in slot i % kDepth and is
+    // requested kDepth - 1 batches before it is used.  (Loads past the last
+    // batch are range-checked to zero by the buffer descriptor.)
+    RowBatch<kRows, kSegments> ring[kDepth];
+#pragma unroll
+    for (int d = 0; d < kDepth - 1; ++d) {
+        load_batch(ring[d], first_batch + d * stride);
+    }
 
     // This thread's slice of x, resident for the whole kernel.  Segments past
     // the row end and rows past x_rows read as zero.
@@ -275,13 +297,14 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
 
     const unsigned lane_bits = pair_table_lane_bits(lane);
 
-    // One batch: prefetch `next`, compute `current`, reduce, write.
+    // One batch: refill the slot freed by the previous batch, compute
+    // `current`, reduce, park.
     const auto step = [&](const RowBatch<kRows, kSegments>& current,
-                          RowBatch<kRows, kSegments>& next,
+                          RowBatch<kRows, kSegments>& refill,
                           unsigned iteration) {
         const unsigned batch_index = first_batch + iteration * stride;
-        if (iteration + 1 < iterations) {
-            load_batch(next, batch_index + stride);
+        if (iteration + kDepth - 1 < iterations) {
+            load_batch(refill, batch_index + (kDepth - 1) * stride);
         }
 
         // Table lookups run one weight row ahead of the multiply-adds that
@@ -356,11 +379,14 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
         }
     };
 
-    // Ping-pong between the two register batches (no copies).
-    for (unsigned iteration = 0; iteration < iterations; iteration += 2) {
-        step(ping, pong, iteration);
-        if (iteration + 1 < iterations) {
-            step(pong, ping, iteration + 1);
+    // Walk the ring with static slot numbers (no register copies).
+    for (unsigned iteration = 0; iteration < iterations;
+         iteration += kDepth) {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            if (iteration + d < iterations) {
+                step(ring[d], ring[(d + kDepth - 1) % kDepth], iteration + d);
+            }
         }
     }
 
@@ -400,19 +426,18 @@ void launch_instance(const LinearProblem& p, hipStream_t stream) {
     // batch so that its registers fit.
     constexpr bool kLight = kX * kSegments == 1;
     constexpr int kTeams = kLight ? RTHIP_GEMV_TEAMS : 2;
-    constexpr int kRows = kLight ? RTHIP_GEMV_ROWS : (kX * kSegments <= 4 ? 4 : 2);
+    constexpr int kRows =
+        kLight ? RTHIP_GEMV_ROWS : (kX * kSegments <= 4 ? 4 : 2);
+    constexpr int kDepth = kLight ? RTHIP_GEMV_DEPTH : 2;
+    constexpr unsigned kMaxIterations = kParkedValues / (kRows * kX);
     const std::size_t elements = p.output_width * p.input_width;
     const std::size_t block_count = elements >> p.block_shift;
-    GemvBuffers sizes;
-    sizes.code_bytes = static_cast<unsigned>(elements / 2);
-    if constexpr (!kDoubleQuantized) {
-        sizes.primary_bytes = static_cast<unsigned>(block_count * 4);
-        sizes.secondary_bytes = 0;
-    } else {
-        sizes.primary_bytes = static_cast<unsigned>(block_count);
-        sizes.secondary_bytes = static_cast<unsigned>(
-            (((block_count - 1) >> p.weight.second_level_shift) + 1) * 4);
-    }
+    // extent of the second-level scale table (double-quantised scales only)
+    const unsigned secondary_bytes =
+        kDoubleQuantized
+            ? static_cast<unsigned>(
+                  (((block_count - 1) >> p.weight.second_level_shift) + 1) * 4)
+            : 0U;
     const unsigned batch_count =
         static_cast<unsigned>((p.output_width + kRows - 1) / kRows);
     const unsigned team_groups = (batch_count + kTeams - 1) / kTeams;
@@ -423,9 +448,9 @@ void launch_instance(const LinearProblem& p, hipStream_t stream) {
         blocks = (team_groups + kMaxIterations - 1) / kMaxIterations;
     }
     const unsigned iterations = (team_groups + blocks - 1) / blocks;
-    gemv_forward_kernel<kX, kSegments, kRows, kTeams, kDoubleQuantized>
+    gemv_forward_kernel<kX, kSegments, kRows, kTeams, kDepth, kDoubleQuantized>
         <<<blocks, kTeamThreads * kTeams, 0, stream>>>(
-            p.activations, p.weight, sizes, p.bias, p.result,
+            p.activations, p.weight, secondary_bytes, p.bias, p.result,
             static_cast<unsigned>(p.rows),
             static_cast<unsigned>(p.input_width),
             static_cast<unsigned>(p.output_width), p.block_shift, batch_count,

@@ -409,7 +409,11 @@ rthip_status rthip_nf4_linear_forward_with(
                         "width that is a multiple of 64 and aligned pointers",
                         rthip::kSkinnyMaxRows);
         }
-        rthip::launch_skinny_forward(problem, hip_stream);
+        if (const hipError_t status =
+                rthip::launch_skinny_forward(problem, hip_stream);
+            status != hipSuccess) {
+            return from_hip(status, "small-batch workspace allocation");
+        }
         break;
     default:
         return fail(RTHIP_INVALID_ARGUMENT, "unknown algorithm %d",

@@ -45,7 +45,9 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(fwd, 16, 256, 768, 64) == package.ALGORITHM_SKINNY
     assert select(fwd, 64, 4096, 11008, 64) == package.ALGORITHM_SKINNY
     assert select(fwd, 65, 4096, 11008, 64) == package.ALGORITHM_MFMA
-    assert select(fwd, 16, 96, 768, 32) == package.ALGORITHM_SKINNY
+    assert select(fwd, 16, 128, 768, 32) == package.ALGORITHM_SKINNY
+    # (row width a multiple of 32 but not of 64 -> tiled GEMM)
+    assert select(fwd, 16, 96, 768, 32) == package.ALGORITHM_MFMA
     assert select(fwd, 16, 40, 768, 32) == package.ALGORITHM_GENERIC
     assert select(bwd, 2048, 4096, 11008, 64) == package.ALGORITHM_MFMA
     assert select(bwd, 2048, 11008, 4096, 64) == package.ALGORITHM_MFMA

@@ -246,6 +246,29 @@ def test_ragged_shapes_and_block_sizes(gpu, package, library, oracle, out_w,
         check_layer(gpu, package, library, oracle, weight, x, dy)
 
 
+@pytest.mark.parametrize("out_w,in_w,block,double_quantized", [
+    (33000, 64, 32, False),    # >= 256 output tiles: one workgroup per tile
+    (300, 1280, 64, True),     # fewer (tile, round) units than compute units
+    (2000, 1600, 64, False),   # last round and last tile partly empty
+    (5000, 2048, 64, True),    # runs of one and two units, tiles shared
+    (1000, 16384, 128, False),  # many workgroups per output tile
+    (30000, 512, 32, True),    # runs that cross from one tile into the next
+])
+def test_small_batch_work_split(gpu, package, library, oracle, out_w, in_w,
+                                block, double_quantized):
+    """Shapes chosen for how the small-batch family deals (tile, round) units
+    to workgroups: whole tiles written directly, partial tiles added by the
+    second kernel, with bias."""
+    dense = helpers.normal(65, (out_w, in_w), 0.02)
+    weight = oracle.quantize(dense, block, double_quantized, 64)
+    bias = helpers.normal(66, (out_w,), 0.01)
+    for rows in (5, 17, 64):
+        x = helpers.normal(67 + rows, (rows, in_w), 1.0)
+        dy = helpers.normal(68 + rows, (rows, out_w), 1.0e-2)
+        check_layer(gpu, package, library, oracle, weight, x, dy, bias=bias,
+                    oracle_rows=min(rows, 5))
+
+
 def test_zero_scale_blocks_and_saturated_scales(gpu, package, library,
                                                 oracle):
     dense = helpers.normal(70, (64, 128), 0.02)
