@@ -148,12 +148,24 @@ def bench_decode(package, device, torch, layers, steps, warmup, use_graph):
         "launches_per_step": launches_per_step,
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
-            "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            "traffic": DOMINANT_KERNEL_HBM_BYTES,
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+                              "scaled by a copy of known size "
+                              "(profiles/decode_gemv_hbm_traffic_pmc.txt)",
             "kernel": "gemv_forward_kernel<rows=1, K=4096>",
             "bytes_per_launch": dominant_bytes / len(dominant),
             "avg_launch_us": average_us,
         },
     }
+
+
+# HBM bytes per launch of the dominant kernel (average over its 4:2 mix of
+# 4096x4096 and 11008x4096 weights), measured with rocprofv3 counters in runs
+# of their own -- a counter run cannot be nested inside this timing run:
+# FETCH_SIZE 7303.0 x 2.00 KiB (the factor a copy kernel of known size gives)
+# plus WRITE_SIZE 25.0 x 1.00 KiB.  Algorithmic bytes: 14 745 600.
+DOMINANT_KERNEL_HBM_BYTES = int((7303.0 * 2.00 + 25.0) * 1024)
 
 
 def bench_gemm(package, device, torch, steps):
