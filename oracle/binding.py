@@ -147,6 +147,13 @@ class Oracle:
             fn.argtypes = [vp, vp, sp, vp, sz, sz, sz, sz]
         lib.nf4o_add_bias.restype = None
         lib.nf4o_add_bias.argtypes = [vp, vp, sz, sz]
+        for name in ("nf4o_matmul", "nf4o_matmul_nt"):
+            fn = getattr(lib, name)
+            fn.restype = None
+            fn.argtypes = [vp, vp, vp, sz, sz, sz]
+        lib.nf4o_lora_linear_forward.restype = None
+        lib.nf4o_lora_linear_forward.argtypes = [
+            vp, vp, sp, vp, vp, vp, sz, ctypes.c_float, vp, sz, sz, sz, sz]
         lib.nf4o_validate_payload.restype = i32
         lib.nf4o_validate_payload.argtypes = [
             sz, sz, vp, sz, sp, ctypes.POINTER(ctypes.c_char_p)]
@@ -245,6 +252,38 @@ class Oracle:
         return self._linear(name, dy, weight, weight.output_width,
                             weight.input_width)
 
+    def matmul(self, left, right) -> np.ndarray:
+        """left [rows, shared] x right [shared, columns]."""
+        left, right = _f32(left), _f32(right)
+        out = np.empty((left.shape[0], right.shape[1]), dtype=np.float32)
+        self._lib.nf4o_matmul(left.ctypes.data, right.ctypes.data,
+                              out.ctypes.data, left.shape[0], left.shape[1],
+                              right.shape[1])
+        return out
+
+    def matmul_nt(self, left, right_t) -> np.ndarray:
+        """left [rows, shared] x right_t[columns, shared]^T."""
+        left, right_t = _f32(left), _f32(right_t)
+        out = np.empty((left.shape[0], right_t.shape[0]), dtype=np.float32)
+        self._lib.nf4o_matmul_nt(left.ctypes.data, right_t.ctypes.data,
+                                 out.ctypes.data, left.shape[0],
+                                 left.shape[1], right_t.shape[0])
+        return out
+
+    def lora_forward(self, x, weight: Nf4Weight, lora_a, lora_b,
+                     lora_scale: float, bias=None) -> np.ndarray:
+        x = _f32(x).reshape(-1, weight.input_width)
+        lora_a, lora_b = _f32(lora_a), _f32(lora_b)
+        bias = None if bias is None else _f32(bias)
+        out = np.empty((x.shape[0], weight.output_width), dtype=np.float32)
+        view = _scales_struct(weight)
+        self._lib.nf4o_lora_linear_forward(
+            x.ctypes.data, weight.codes.ctypes.data, ctypes.byref(view),
+            _ptr(bias), lora_a.ctypes.data, lora_b.ctypes.data,
+            lora_a.shape[0], lora_scale, out.ctypes.data, x.shape[0],
+            weight.input_width, weight.output_width, weight.block_size)
+        return out
+
     # -- validation ------------------------------------------------------
     def validate_payload(self, weight: Nf4Weight) -> None:
         view = _scales_struct(weight)
@@ -301,6 +340,11 @@ class Reference:
         lib.nf4ref_run.argtypes = [i32, vp, vp, sz, sz, sz, sz] + payload
         lib.nf4ref_memory_usage.restype = i32
         lib.nf4ref_memory_usage.argtypes = [sz, sz, sz] + payload + [vp]
+        lib.nf4ref_matmul.restype = i32
+        lib.nf4ref_matmul.argtypes = [vp, vp, vp, sz, sz, sz]
+        lib.nf4ref_lora_linear_forward.restype = i32
+        lib.nf4ref_lora_linear_forward.argtypes = [
+            vp, vp, vp, vp, sz, f32, vp, sz, sz, sz, sz] + payload
 
     def _check(self, status: int) -> None:
         if status != 0:
@@ -383,6 +427,28 @@ class Reference:
         dy = _f32(dy).reshape(-1, weight.output_width)
         return self._run(2, dy, weight, dy.shape[0],
                          (dy.shape[0], weight.input_width))
+
+    def matmul(self, left, right) -> np.ndarray:
+        left, right = _f32(left), _f32(right)
+        out = np.empty((left.shape[0], right.shape[1]), dtype=np.float32)
+        self._check(self._lib.nf4ref_matmul(
+            left.ctypes.data, right.ctypes.data, out.ctypes.data,
+            left.shape[0], left.shape[1], right.shape[1]))
+        return out
+
+    def lora_forward(self, x, weight: Nf4Weight, lora_a, lora_b,
+                     lora_scale: float, bias=None) -> np.ndarray:
+        x = _f32(x).reshape(-1, weight.input_width)
+        lora_a, lora_b = _f32(lora_a), _f32(lora_b)
+        bias = None if bias is None else _f32(bias)
+        out = np.empty((x.shape[0], weight.output_width), dtype=np.float32)
+        self._check(self._lib.nf4ref_lora_linear_forward(
+            x.ctypes.data, _ptr(bias), lora_a.ctypes.data,
+            lora_b.ctypes.data, lora_a.shape[0], lora_scale,
+            out.ctypes.data, x.shape[0], weight.input_width,
+            weight.output_width, weight.block_size,
+            *self._payload_args(weight)))
+        return out
 
     def memory_usage(self, weight: Nf4Weight) -> dict:
         out = np.zeros(9, dtype=np.uintp)

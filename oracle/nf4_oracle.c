@@ -331,6 +331,64 @@ void nf4o_add_bias(float* y, const float* bias, size_t rows,
     }
 }
 
+void nf4o_matmul(const float* left, const float* right, float* out,
+                 size_t rows, size_t shared, size_t columns) {
+    size_t row;
+    size_t column;
+    size_t inner;
+    for (row = 0; row < rows; ++row) {
+        for (column = 0; column < columns; ++column) {
+            float total = 0.0F;
+            for (inner = 0; inner < shared; ++inner) {
+                total += left[row * shared + inner] *
+                         right[inner * columns + column];
+            }
+            out[row * columns + column] = total;
+        }
+    }
+}
+
+void nf4o_matmul_nt(const float* left, const float* right_t, float* out,
+                    size_t rows, size_t shared, size_t columns) {
+    size_t row;
+    size_t column;
+    size_t inner;
+    for (row = 0; row < rows; ++row) {
+        for (column = 0; column < columns; ++column) {
+            float total = 0.0F;
+            for (inner = 0; inner < shared; ++inner) {
+                total += left[row * shared + inner] *
+                         right_t[column * shared + inner];
+            }
+            out[row * columns + column] = total;
+        }
+    }
+}
+
+void nf4o_lora_linear_forward(const float* x, const uint8_t* codes,
+                              const nf4o_scales* scales, const float* bias,
+                              const float* lora_a, const float* lora_b,
+                              size_t rank, float lora_scale, float* y,
+                              size_t rows, size_t input_width,
+                              size_t output_width, size_t block_size) {
+    float* reduced = (float*)malloc(sizeof(float) * rows * rank);
+    float* expanded = (float*)malloc(sizeof(float) * rows * output_width);
+    size_t index;
+    nf4o_linear_forward_rowcached(x, codes, scales, y, rows, input_width,
+                                  output_width, block_size);
+    if (bias != NULL) {
+        nf4o_add_bias(y, bias, rows, output_width);
+    }
+    nf4o_matmul_nt(x, lora_a, reduced, rows, input_width, rank);
+    nf4o_matmul_nt(reduced, lora_b, expanded, rows, rank, output_width);
+    for (index = 0; index < rows * output_width; ++index) {
+        const float scaled = expanded[index] * lora_scale;
+        y[index] = y[index] + scaled;
+    }
+    free(reduced);
+    free(expanded);
+}
+
 size_t nf4o_scale_payload_bytes(const nf4o_scales* scales) {
     if (scales->encoding == NF4O_SCALE_FLOAT32) {
         return scales->fp32_count * sizeof(float);

@@ -135,6 +135,34 @@ void nf4o_linear_input_backward_rowcached(const float* dy,
 void nf4o_add_bias(float* y, const float* bias, size_t rows,
                    size_t output_width);
 
+/* CpuBackendAdapter::matmul, src/core/backend/adapters/cpu/adapter.cpp:158-203,
+ * one batch: out[r,c] = sum_k left[r,k] * right[k,c]; fp32 accumulator,
+ * ascending k; left is [rows, shared], right [shared, columns], row-major. */
+void nf4o_matmul(const float* left, const float* right, float* out,
+                 size_t rows, size_t shared, size_t columns);
+
+/* The same sums with the right operand given transposed ([columns, shared]
+ * row-major): out[r,c] = sum_k left[r,k] * right_t[c,k].  This is what
+ * matmul(x, transpose_2d(W)) computes once the transpose is materialised
+ * (src/nn/linear.cpp:158-163, src/nn/low_rank_adapter.cpp:140-147). */
+void nf4o_matmul_nt(const float* left, const float* right_t, float* out,
+                    size_t rows, size_t shared, size_t columns);
+
+/* Linear::forward with a packed weight, optional bias and an attached
+ * low-rank adapter, src/nn/linear.cpp:147-172 and
+ * src/nn/low_rank_adapter.cpp:126-151:
+ *   base = x.deq(W)^T (+ bias, a separate broadcast add)
+ *   reduced  = matmul(x, transpose(A))        A: [rank, input_width]
+ *   expanded = matmul(reduced, transpose(B))  B: [output_width, rank]
+ *   y = base + expanded * lora_scale
+ * every step rounded to fp32 on its own.  bias may be NULL. */
+void nf4o_lora_linear_forward(const float* x, const uint8_t* codes,
+                              const nf4o_scales* scales, const float* bias,
+                              const float* lora_a, const float* lora_b,
+                              size_t rank, float lora_scale, float* y,
+                              size_t rows, size_t input_width,
+                              size_t output_width, size_t block_size);
+
 /* require_canonical_payload, src/core/quantization/quantized_weight.cpp:102-174.
  * Returns NF4O_OK or the status of the exception the reference throws;
  * *message (may be NULL) receives a static description. */

@@ -12,11 +12,14 @@
 //       include/riftco_transformer/core/quantized_weight.hpp:69-111
 //   dispatch_quantized_linear_forward / _input_backward
 //       src/core/backend/nn/quantized_linear/dispatch.hpp:19-27
+//   tensor_ops::matmul / transpose_2d / scale / add / broadcast_to
+//       include/riftco_transformer/core/tensor_ops.hpp:12-36
 
 #include "core/backend/nn/quantized_linear/dispatch.hpp"
 #include "riftco_transformer/core/backend.hpp"
 #include "riftco_transformer/core/quantized_weight.hpp"
 #include "riftco_transformer/core/tensor.hpp"
+#include "riftco_transformer/core/tensor_ops.hpp"
 
 #include <algorithm>
 #include <cstddef>
@@ -216,6 +219,85 @@ int nf4ref_memory_usage(
         out[6] = usage.scale_code_bytes;
         out[7] = usage.second_level_scale_bytes;
         out[8] = usage.scale_offset_bytes;
+    });
+}
+
+// out[rows, columns] = left[rows, shared] x right[shared, columns] through
+// tensor_ops::matmul on the CPU backend.
+int nf4ref_matmul(
+    const float* left, const float* right, float* out, std::size_t rows,
+    std::size_t shared, std::size_t columns
+) {
+    return guarded([&] {
+        const Tensor a({rows, shared},
+                       std::vector<float>(left, left + rows * shared),
+                       ExecutionBackend::Cpu);
+        const Tensor b({shared, columns},
+                       std::vector<float>(right, right + shared * columns),
+                       ExecutionBackend::Cpu);
+        const Tensor c = riftco_transformer::tensor_ops::matmul(a, b);
+        const auto data = c.data();
+        std::copy(data.begin(), data.end(), out);
+    });
+}
+
+// The forward of a Linear that holds a packed weight, an optional bias and a
+// low-rank adapter, composed from the reference's own tensor operations in
+// the order of src/nn/linear.cpp:147-172 and
+// src/nn/low_rank_adapter.cpp:126-151 (the autograd wrappers those files use
+// call exactly these operations for their forward values).
+int nf4ref_lora_linear_forward(
+    const float* x, const float* bias_or_null, const float* lora_a,
+    const float* lora_b, std::size_t rank, float lora_scale, float* y,
+    std::size_t rows, std::size_t input_width, std::size_t output_width,
+    std::size_t block_size, const std::uint8_t* codes, std::size_t code_bytes,
+    int encoding, const float* fp32_scales, std::size_t fp32_count,
+    const std::uint8_t* scale_codes, std::size_t scale_code_count,
+    const float* second_level, std::size_t second_level_count,
+    std::size_t second_level_block, float offset
+) {
+    namespace ops = riftco_transformer::tensor_ops;
+    return guarded([&] {
+        const QuantizedWeight weight = QuantizedWeight::from_packed_nf4(
+            {output_width, input_width}, block_size,
+            make_payload(codes, code_bytes, encoding, fp32_scales, fp32_count,
+                         scale_codes, scale_code_count, second_level,
+                         second_level_count, second_level_block, offset),
+            ExecutionBackend::Cpu
+        );
+        const Tensor input({rows, input_width},
+                           std::vector<float>(x, x + rows * input_width),
+                           ExecutionBackend::Cpu);
+        Tensor projected({rows, output_width}, ExecutionBackend::Cpu);
+        backend::dispatch_quantized_linear_forward(
+            ExecutionBackend::Cpu,
+            {backend::tensor_storage(input),
+             backend::quantized_weight_storage(weight),
+             backend::tensor_storage(projected),
+             backend::QuantizedLinearDimensions{rows, input_width,
+                                                output_width, block_size}});
+        Tensor base = projected;
+        if (bias_or_null != nullptr) {
+            const Tensor bias(
+                {output_width},
+                std::vector<float>(bias_or_null, bias_or_null + output_width),
+                ExecutionBackend::Cpu);
+            base = ops::add(projected,
+                            ops::broadcast_to(bias, {rows, output_width}));
+        }
+        const Tensor a({rank, input_width},
+                       std::vector<float>(lora_a, lora_a + rank * input_width),
+                       ExecutionBackend::Cpu);
+        const Tensor b({output_width, rank},
+                       std::vector<float>(lora_b,
+                                          lora_b + output_width * rank),
+                       ExecutionBackend::Cpu);
+        const Tensor reduced = ops::matmul(input, ops::transpose_2d(a));
+        const Tensor expanded = ops::matmul(reduced, ops::transpose_2d(b));
+        const Tensor result =
+            ops::add(base, ops::scale(expanded, lora_scale));
+        const auto data = result.data();
+        std::copy(data.begin(), data.end(), y);
     });
 }
 

@@ -156,3 +156,28 @@ def test_block_sizes_and_nonfinite_sources(oracle):
     values[0] = np.nan
     with pytest.raises(ValueError):
         oracle.quantize(values, 32)
+
+
+def test_lora_composes_its_scaled_low_rank_delta(oracle):
+    """tests/nn/test_lora.cpp:208-243: A = [[1,0,0],[0,1,0]], B = [[1,2],[-1,3]],
+    alpha 4 at rank 2 (scale 2), x = [1,2,3]; the dense base of that test
+    contributes [14.5, 4.5] (W x + b), supplied here as the bias of an all-zero
+    packed weight.  Expected output [24.5, 14.5]."""
+    weight = oracle.quantize(np.zeros((2, 32), dtype=np.float32), 32)
+    x = np.zeros((1, 32), dtype=np.float32)
+    x[0, :3] = [1.0, 2.0, 3.0]
+    lora_a = np.zeros((2, 32), dtype=np.float32)
+    lora_a[0, 0] = 1.0
+    lora_a[1, 1] = 1.0
+    lora_b = np.array([[1.0, 2.0], [-1.0, 3.0]], dtype=np.float32)
+    bias = np.array([14.5, 4.5], dtype=np.float32)
+    y = oracle.lora_forward(x, weight, lora_a, lora_b, 4.0 / 2.0, bias)
+    assert y.tolist() == [[24.5, 14.5]]
+
+
+def test_matmul_small_integer_case(oracle):
+    left = np.array([[1, 2, 3], [4, 5, 6]], dtype=np.float32)
+    right = np.array([[1, 0], [0, 1], [2, -1]], dtype=np.float32)
+    assert oracle.matmul(left, right).tolist() == [[7.0, -1.0], [16.0, -1.0]]
+    assert oracle.matmul_nt(left, np.ascontiguousarray(right.T)).tolist() == \
+        [[7.0, -1.0], [16.0, -1.0]]

@@ -158,3 +158,31 @@ def test_bias_is_a_separate_add(oracle):
     bias = helpers.normal(32, (8,), 0.01)
     helpers.assert_bit_equal(oracle.forward(x, weight, bias),
                              oracle.forward(x, weight) + bias[None, :])
+
+
+def test_lora_with_zero_b_is_the_plain_layer(oracle):
+    """A freshly attached adapter has B = 0 (tests/nn/test_lora.cpp:150-157):
+    the layer's output is then exactly the base output."""
+    dense = helpers.normal(30, (48, 128), 0.02)
+    weight = oracle.quantize(dense, 64)
+    x = helpers.normal(31, (4, 128), 1.0)
+    bias = helpers.normal(32, (48,), 0.01)
+    lora_a = helpers.normal(33, (8, 128), 0.05)
+    lora_b = np.zeros((48, 8), dtype=np.float32)
+    helpers.assert_bit_equal(
+        oracle.lora_forward(x, weight, lora_a, lora_b, 2.0, bias),
+        oracle.forward(x, weight, bias))
+
+
+def test_lora_matches_float64_composition(oracle):
+    dense = helpers.normal(34, (96, 256), 0.02)
+    weight = oracle.quantize(dense, 64, True, 32)
+    x = helpers.normal(35, (6, 256), 1.0)
+    lora_a = helpers.normal(36, (16, 256), 0.05)
+    lora_b = helpers.normal(37, (96, 16), 0.05)
+    deq = oracle.dequantize(weight).astype(np.float64)
+    exact = x.astype(np.float64) @ deq.T + 0.5 * (
+        (x.astype(np.float64) @ lora_a.astype(np.float64).T)
+        @ lora_b.astype(np.float64).T)
+    got = oracle.lora_forward(x, weight, lora_a, lora_b, 0.5)
+    assert np.max(np.abs(got - exact)) <= 1e-5 * np.max(np.abs(exact))

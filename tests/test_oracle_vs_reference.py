@@ -105,3 +105,34 @@ def test_memory_usage_known_answers(oracle, reference):
         "scale_offset_bytes": 4}
     assert oracle.scale_payload_bytes(weight) == usage["scale_bytes"]
     assert weight.payload_bytes == usage["logical_payload_bytes"]
+
+
+@pytest.mark.parametrize("rows,shared,columns", [
+    (1, 1, 1), (3, 33, 5), (16, 256, 8), (7, 1000, 64)])
+def test_matmul_bitwise(oracle, reference, rows, shared, columns):
+    left = helpers.normal(44, (rows, shared), 1.0)
+    right = helpers.normal(45, (shared, columns), 0.05)
+    theirs = reference.matmul(left, right)
+    helpers.assert_bit_equal(oracle.matmul(left, right), theirs)
+    # the transposed-operand form is the same sum
+    helpers.assert_bit_equal(
+        oracle.matmul_nt(left, np.ascontiguousarray(right.T)), theirs)
+
+
+@pytest.mark.parametrize("shape,block,rank", [
+    ((768, 256), 64, 8), ((33, 33), 32, 2), ((64, 1000), 128, 16),
+    ((40, 96), 32, 64)])
+@pytest.mark.parametrize("double_quantized", [False, True])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_lora_linear_forward_bitwise(oracle, reference, shape, block, rank,
+                                     double_quantized, with_bias):
+    out_w, in_w = shape
+    dense = helpers.normal(46, shape, 0.02)
+    weight = oracle.quantize(dense, block, double_quantized, 32)
+    x = helpers.normal(47, (5, in_w), 1.0)
+    lora_a = helpers.normal(48, (rank, in_w), 0.05)
+    lora_b = helpers.normal(49, (out_w, rank), 0.05)
+    bias = helpers.normal(50, (out_w,), 0.01) if with_bias else None
+    helpers.assert_bit_equal(
+        oracle.lora_forward(x, weight, lora_a, lora_b, 16.0 / rank, bias),
+        reference.lora_forward(x, weight, lora_a, lora_b, 16.0 / rank, bias))
