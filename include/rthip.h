@@ -162,6 +162,33 @@ rthip_status rthip_nf4_linear_input_backward(
     uint64_t input_width, uint64_t output_width, uint64_t block_size,
     void* stream);
 
+/*
+ * y = x.deq(W)^T + bias + lora_scale * ((x.A^T).B^T)
+ *
+ * Linear::forward of a layer that holds a packed weight, an optional bias and
+ * an attached low-rank adapter (src/nn/linear.cpp:147-172 with
+ * LowRankAdapter::forward, src/nn/low_rank_adapter.cpp:126-151), which the
+ * reference evaluates as six separate operations (packed product, broadcast,
+ * add, two dense matmuls over materialised transposes, scale, add).  Here it
+ * is two launches: reduced = x.A^T, then the packed product with bias and the
+ * rank-sized sum in its epilogue.
+ *   lora_a   [lora_rank, input_width]    (LowRankAdapter::a, "lora_a.weight")
+ *   lora_b   [output_width, lora_rank]   (LowRankAdapter::b, "lora_b.weight")
+ *   lora_scale = alpha / rank            (LowRankAdapter::scale)
+ *   reduced  [rows, lora_rank]  caller-provided device buffer that receives
+ *            x.A^T (the saved activation the adapter's backward needs)
+ * Rounding follows the reference: the rank sum in fp32 in ascending order,
+ * times lora_scale, added to (product + bias).
+ */
+rthip_status rthip_nf4_lora_linear_forward(
+    const float* x, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, const float* bias_or_null,
+    const float* lora_a, const float* lora_b, uint64_t lora_rank,
+    float lora_scale, float* reduced, float* y, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream);
+
 /* The same two operations with the kernel family pinned (tests, measurement).
  * RTHIP_UNSUPPORTED when `algorithm` cannot handle the shape. */
 rthip_status rthip_nf4_linear_forward_with(
@@ -171,6 +198,14 @@ rthip_status rthip_nf4_linear_forward_with(
     const float* bias_or_null, float* y, uint64_t rows, uint64_t input_width,
     uint64_t output_width, uint64_t block_size, void* stream);
 
+rthip_status rthip_nf4_lora_linear_forward_with(
+    int32_t algorithm, const float* x, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset,
+    const float* bias_or_null, const float* lora_a, const float* lora_b,
+    uint64_t lora_rank, float lora_scale, float* reduced, float* y,
+    uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream);
 rthip_status rthip_nf4_linear_input_backward_with(
     int32_t algorithm, const float* dy, const uint8_t* codes,
     const void* primary_scales, const float* secondary_scales,

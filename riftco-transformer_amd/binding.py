@@ -96,6 +96,14 @@ _PROTOTYPES = {
         [_i32, _ptr] + _WEIGHT + [_ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
     "rthip_nf4_linear_input_backward_with": (
         _i32, [_i32, _ptr] + _WEIGHT + [_ptr, _u64, _u64, _u64, _u64, _ptr]),
+    "rthip_nf4_lora_linear_forward": (
+        _i32,
+        [_ptr] + _WEIGHT + [_ptr, _ptr, _ptr, _u64, _f32, _ptr, _ptr, _u64,
+                            _u64, _u64, _u64, _ptr]),
+    "rthip_nf4_lora_linear_forward_with": (
+        _i32,
+        [_i32, _ptr] + _WEIGHT + [_ptr, _ptr, _ptr, _u64, _f32, _ptr, _ptr,
+                                  _u64, _u64, _u64, _u64, _ptr]),
     "rthip_nf4_select_algorithm": (
         _i32, [_i32, _u64, _u64, _u64, _u64, ctypes.POINTER(_i32)]),
     "rthip_nf4_dequantize": (_i32, _WEIGHT + [_ptr, _u64, _u64, _ptr]),
@@ -235,6 +243,23 @@ class Library:
                 x_ptr, *weight.abi_arguments(), *tail)
         else:
             status = self._lib.rthip_nf4_linear_forward_with(
+                algorithm, x_ptr, *weight.abi_arguments(), *tail)
+        self._check(status)
+
+    def lora_linear_forward(self, x_ptr: int, weight: DeviceWeight,
+                            bias_ptr: Optional[int], lora_a_ptr: int,
+                            lora_b_ptr: int, rank: int, lora_scale: float,
+                            reduced_ptr: int, y_ptr: int, rows: int,
+                            stream: int = 0,
+                            algorithm: Optional[int] = None) -> None:
+        tail = [bias_ptr, lora_a_ptr, lora_b_ptr, rank, lora_scale,
+                reduced_ptr, y_ptr, rows, weight.input_width,
+                weight.output_width, weight.block_size, stream]
+        if algorithm is None:
+            status = self._lib.rthip_nf4_lora_linear_forward(
+                x_ptr, *weight.abi_arguments(), *tail)
+        else:
+            status = self._lib.rthip_nf4_lora_linear_forward_with(
                 algorithm, x_ptr, *weight.abi_arguments(), *tail)
         self._check(status)
 

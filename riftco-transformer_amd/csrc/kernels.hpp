@@ -3,6 +3,7 @@
 // matching *_supports() predicate, which the C ABI consults before launching.
 #pragma once
 
+#include "lora_epilogue.hpp"
 #include "nf4_decode.hpp"
 
 #include <hip/hip_runtime.h>
@@ -24,6 +25,9 @@ struct LinearProblem {
     std::size_t input_width;
     std::size_t output_width;
     unsigned block_shift;  // log2(block_size)
+    // forward only: low-rank adapter term added in the epilogue
+    // (lora.reduced == nullptr: none)
+    LoraEpilogue lora{nullptr, nullptr, 0U, 0.0F};
 };
 
 // nf4_generic.hip
@@ -49,6 +53,11 @@ constexpr std::size_t kSkinnyMaxRows = 64;
 bool skinny_forward_supports(const LinearProblem& problem);
 hipError_t launch_skinny_forward(const LinearProblem& problem,
                                  hipStream_t stream);
+
+// lora.hip -- reduced[rows, rank] = x A^T, the input of the adapter epilogue.
+void launch_lora_reduce(const float* x, const float* a, float* reduced,
+                        std::size_t rows, std::size_t input_width,
+                        std::size_t rank, hipStream_t stream);
 
 // nf4_mfma.hip
 bool mfma_forward_supports(const LinearProblem& problem);

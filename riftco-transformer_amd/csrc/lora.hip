@@ -1,0 +1,210 @@
+// reduced[m, j] = sum_k x[m, k] * A[j, k]: the first product of a low-rank
+// adapter, matmul(x, transpose(A)) in LowRankAdapter::forward
+// (src/nn/low_rank_adapter.cpp:140-143 under /root/reference).  A is
+// [rank, input_width]; the result is tiny ([rows, rank]) and is consumed by
+// the epilogue of the packed-weight kernels (lora_epilogue.hpp).
+//
+// x is read exactly once.  A workgroup of sixteen wavefronts owns 16 rows of x
+// and up to 64 adapter rows; the contraction axis is cut into sixteen spans,
+// one per wavefront, which each run v_mfma_f32_16x16x4_f32 over their span
+// (A operand: x[16 rows][4 k]; B operand: A^T[4 k][16 adapter rows]) from
+// 16-byte loads, and the sixteen partial tiles are added through LDS in
+// wavefront order.  With one token (rows = 1) this is a single workgroup whose
+// wavefronts each see 1/16 of the row, which keeps the latency of the whole
+// product near one memory round trip.
+//
+// Loads are raw buffer loads; lanes past the last row, the last adapter row or
+// the row end get an offset the range check rejects and read zeros.
+
+#include "kernels.hpp"
+
+namespace rthip {
+namespace {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWaves = 16;
+constexpr int kThreads = 64 * kWaves;
+constexpr unsigned kRejectedOffset = 0x80000000U;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_buffer(const void* base,
+                                                            std::size_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+// kBlocks: 16-row blocks of A handled by one workgroup (1, 2 or 4).
+template <int kBlocks>
+__global__ __launch_bounds__(kThreads) void lora_reduce_kernel(
+    const float* __restrict__ x, const float* __restrict__ a,
+    float* __restrict__ reduced, unsigned rows, unsigned input_width,
+    unsigned rank
+) {
+    __shared__ float partial[kWaves][kBlocks][4][64];
+
+    const unsigned lane = threadIdx.x % 64;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const unsigned quarter = lane / 16;
+    const unsigned row = blockIdx.x * 16 + lane % 16;         // of x
+    const unsigned first_adapter_row = blockIdx.y * 16 * kBlocks;
+
+    const __amdgpu_buffer_rsrc_t x_buffer = raw_buffer(
+        x, static_cast<std::size_t>(rows) * input_width * sizeof(float));
+    const __amdgpu_buffer_rsrc_t a_buffer = raw_buffer(
+        a, static_cast<std::size_t>(rank) * input_width * sizeof(float));
+
+    // Spans are multiples of 16 contraction values.
+    const unsigned span = ((input_width + 16 * kWaves - 1) / (16 * kWaves)) * 16;
+    const unsigned span_begin = wave * span;
+    const unsigned span_end = min(span_begin + span, input_width);
+
+    const bool row_valid = row < rows;
+    const unsigned x_row_bytes = row * input_width * 4U;
+    bool adapter_valid[kBlocks];
+    unsigned a_row_bytes[kBlocks];
+#pragma unroll
+    for (int b = 0; b < kBlocks; ++b) {
+        const unsigned j = first_adapter_row + 16 * b + lane % 16;
+        adapter_valid[b] = j < rank;
+        a_row_bytes[b] = j * input_width * 4U;
+    }
+
+    floatx4 acc[kBlocks];
+#pragma unroll
+    for (int b = 0; b < kBlocks; ++b) {
+        acc[b] = floatx4{0.0F, 0.0F, 0.0F, 0.0F};
+    }
+    // Four steps of 16 contraction values per trip, so that their loads are
+    // in flight together; steps past the span read zeros.
+    constexpr int kUnroll = 4;
+    for (unsigned k0 = span_begin; k0 < span_end; k0 += 16 * kUnroll) {
+        floatx4 xv[kUnroll];
+        floatx4 av[kUnroll][kBlocks];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const unsigned k = k0 + 16 * u + 4 * quarter;
+            // spans and the row width are multiples of 4, so a float4 lies
+            // inside or outside as a whole
+            const bool column_valid = k < span_end;
+            xv[u] = __builtin_bit_cast(
+                floatx4, __builtin_amdgcn_raw_buffer_load_b128(
+                             x_buffer,
+                             row_valid && column_valid ? x_row_bytes + k * 4U
+                                                       : kRejectedOffset,
+                             0, 0));
+#pragma unroll
+            for (int b = 0; b < kBlocks; ++b) {
+                av[u][b] = __builtin_bit_cast(
+                    floatx4, __builtin_amdgcn_raw_buffer_load_b128(
+                                 a_buffer,
+                                 adapter_valid[b] && column_valid
+                                     ? a_row_bytes[b] + k * 4U
+                                     : kRejectedOffset,
+                                 0, 0));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+            for (int b = 0; b < kBlocks; ++b) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                        xv[u][e], av[u][b][e], acc[b], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int b = 0; b < kBlocks; ++b) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            partial[wave][b][r][lane] = acc[b][r];
+        }
+    }
+    __syncthreads();
+    // Accumulator element r of lane l is x row 4 * (l / 16) + r, adapter row
+    // l % 16 of its block.  Thread t adds up element t of the tile.
+    for (unsigned index = threadIdx.x; index < kBlocks * 256U;
+         index += kThreads) {
+        const unsigned b = index / 256;
+        const unsigned r = (index / 64) % 4;
+        const unsigned l = index % 64;
+        float sum = 0.0F;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            sum += partial[w][b][r][l];
+        }
+        const unsigned m = blockIdx.x * 16 + 4 * (l / 16) + r;
+        const unsigned j = first_adapter_row + 16 * b + l % 16;
+        if (m < rows && j < rank) {
+            reduced[static_cast<std::size_t>(m) * rank + j] = sum;
+        }
+    }
+}
+
+// Any shape and alignment: one wavefront per output.
+__global__ __launch_bounds__(256) void lora_reduce_generic_kernel(
+    const float* __restrict__ x, const float* __restrict__ a,
+    float* __restrict__ reduced, std::size_t rows, std::size_t input_width,
+    std::size_t rank
+) {
+    const std::size_t output =
+        (static_cast<std::size_t>(blockIdx.x) * blockDim.x + threadIdx.x) / 64;
+    const unsigned lane = threadIdx.x % 64;
+    if (output >= rows * rank) {
+        return;
+    }
+    const float* x_row = x + (output / rank) * input_width;
+    const float* a_row = a + (output % rank) * input_width;
+    float sum = 0.0F;
+    for (std::size_t k = lane; k < input_width; k += 64) {
+        sum += x_row[k] * a_row[k];
+    }
+#pragma unroll
+    for (int offset = 32; offset >= 1; offset /= 2) {
+        sum += __shfl_xor(sum, offset, 64);
+    }
+    if (lane == 0) {
+        reduced[output] = sum;
+    }
+}
+
+}  // namespace
+
+void launch_lora_reduce(const float* x, const float* a, float* reduced,
+                        std::size_t rows, std::size_t input_width,
+                        std::size_t rank, hipStream_t stream) {
+    const bool tiled =
+        input_width % 4 == 0 &&
+        rows * input_width * sizeof(float) < kRejectedOffset &&
+        rank * input_width * sizeof(float) < kRejectedOffset &&
+        (rows + 15) / 16 < (1ULL << 31) && (rank + 63) / 64 <= 65535 &&
+        reinterpret_cast<std::uintptr_t>(x) % 16 == 0 &&
+        reinterpret_cast<std::uintptr_t>(a) % 16 == 0;
+    if (!tiled) {
+        const std::size_t waves = rows * rank;
+        const unsigned blocks = static_cast<unsigned>((waves + 3) / 4);
+        lora_reduce_generic_kernel<<<blocks, 256, 0, stream>>>(
+            x, a, reduced, rows, input_width, rank);
+        return;
+    }
+    const unsigned row_tiles = static_cast<unsigned>((rows + 15) / 16);
+    const auto r = static_cast<unsigned>(rows);
+    const auto i = static_cast<unsigned>(input_width);
+    const auto k = static_cast<unsigned>(rank);
+    if (rank <= 16) {
+        lora_reduce_kernel<1><<<dim3(row_tiles, 1), kThreads, 0, stream>>>(
+            x, a, reduced, r, i, k);
+    } else if (rank <= 32) {
+        lora_reduce_kernel<2><<<dim3(row_tiles, 1), kThreads, 0, stream>>>(
+            x, a, reduced, r, i, k);
+    } else {
+        const unsigned chunks = static_cast<unsigned>((rank + 63) / 64);
+        lora_reduce_kernel<4><<<dim3(row_tiles, chunks), kThreads, 0, stream>>>(
+            x, a, reduced, r, i, k);
+    }
+}
+
+}  // namespace rthip

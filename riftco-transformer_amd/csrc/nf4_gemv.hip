@@ -168,7 +168,7 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
     const float* __restrict__ x, Nf4WeightView weight, unsigned secondary_bytes,
     const float* __restrict__ bias, float* __restrict__ y, unsigned x_rows,
     unsigned input_width, unsigned output_width, unsigned block_shift,
-    unsigned batch_count, unsigned iterations
+    unsigned batch_count, unsigned iterations, LoraEpilogue lora
 ) {
     constexpr int kThreads = kTeamThreads * kTeams;
     constexpr int kValues = kRows * kX;
@@ -410,6 +410,9 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
             if (bias != nullptr) {
                 sum += bias[o];
             }
+            if (lora.reduced != nullptr) {
+                sum += lora_term(lora, r, o);
+            }
             y[r * output_width + o] = sum;
         }
     }
@@ -454,7 +457,7 @@ void launch_instance(const LinearProblem& p, hipStream_t stream) {
             static_cast<unsigned>(p.rows),
             static_cast<unsigned>(p.input_width),
             static_cast<unsigned>(p.output_width), p.block_shift, batch_count,
-            iterations);
+            iterations, p.lora);
 }
 
 template <int kX, bool kDoubleQuantized>

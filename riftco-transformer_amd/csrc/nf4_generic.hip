@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void generic_forward_kernel(
     const float* __restrict__ x, Nf4WeightView weight,
     const float* __restrict__ bias, float* __restrict__ y,
     std::size_t rows, std::size_t input_width, std::size_t output_width,
-    unsigned block_shift
+    unsigned block_shift, LoraEpilogue lora
 ) {
     const std::size_t waves_per_block = blockDim.x / kWave;
     const std::size_t wave =
@@ -61,7 +61,12 @@ __global__ __launch_bounds__(256) void generic_forward_kernel(
         }
         total = wave_sum(total);
         if (lane == 0) {
-            y[output_index] = bias != nullptr ? total + bias[column] : total;
+            float value = bias != nullptr ? total + bias[column] : total;
+            if (lora.reduced != nullptr) {
+                value += lora_term(lora, static_cast<unsigned>(row),
+                                   static_cast<unsigned>(column));
+            }
+            y[output_index] = value;
         }
     }
 }
@@ -153,7 +158,7 @@ void launch_generic_forward(const LinearProblem& p, hipStream_t stream) {
     const std::size_t outputs = p.rows * p.output_width;
     generic_forward_kernel<<<grid_for(outputs, 4), 256, 0, stream>>>(
         p.activations, p.weight, p.bias, p.result, p.rows, p.input_width,
-        p.output_width, p.block_shift);
+        p.output_width, p.block_shift, p.lora);
 }
 
 void launch_generic_input_backward(const LinearProblem& p,

@@ -182,7 +182,7 @@ template <bool kDoubleQuantized, bool kBackward>
 __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
     const float* __restrict__ activations, Nf4WeightView weight,
     const float* __restrict__ bias, float* __restrict__ result,
-    GemmShape shape, unsigned block_shift
+    GemmShape shape, unsigned block_shift, LoraEpilogue lora
 ) {
     __shared__ __attribute__((aligned(16))) float a_tile[kTileM * kStride];
     __shared__ __attribute__((aligned(16))) float b_tile[kTileN * kStride];
@@ -321,13 +321,37 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
                     addend = bias[column];
                 }
             }
+            float term[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                term[e] = 0.0F;
+            }
+            if constexpr (!kBackward) {
+                if (lora.reduced != nullptr) {  // uniform
+                    const float* reduced_rows[16];
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const unsigned row =
+                            min(row0 + wave_m * 64 + i * 32 + 8 * (e / 4) +
+                                    4 * (lane / 32) + e % 4,
+                                shape.rows - 1);
+                        reduced_rows[e] =
+                            lora.reduced +
+                            static_cast<std::size_t>(row) * lora.rank;
+                    }
+                    lora_terms<16>(
+                        term,
+                        lora.b + static_cast<std::size_t>(column) * lora.rank,
+                        reduced_rows, lora.rank, lora.scale);
+                }
+            }
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const unsigned row = row0 + wave_m * 64 + i * 32 +
                                      8 * (e / 4) + 4 * (lane / 32) + e % 4;
                 if (row < shape.rows) {
                     result[static_cast<std::size_t>(row) * shape.columns +
-                           column] = total[i][j][e] + addend;
+                           column] = (total[i][j][e] + addend) + term[e];
                 }
             }
         }
@@ -350,10 +374,12 @@ void launch(const LinearProblem& p, hipStream_t stream) {
                     (shape.rows + kTileM - 1) / kTileM);
     if (p.weight.encoding == 0) {
         mfma_gemm_kernel<false, kBackward><<<grid, kThreads, 0, stream>>>(
-            p.activations, p.weight, p.bias, p.result, shape, p.block_shift);
+            p.activations, p.weight, p.bias, p.result, shape, p.block_shift,
+            p.lora);
     } else {
         mfma_gemm_kernel<true, kBackward><<<grid, kThreads, 0, stream>>>(
-            p.activations, p.weight, p.bias, p.result, shape, p.block_shift);
+            p.activations, p.weight, p.bias, p.result, shape, p.block_shift,
+            p.lora);
     }
 }
 

@@ -94,7 +94,8 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
     const float* __restrict__ x, Nf4WeightView weight,
     const float* __restrict__ bias, float* __restrict__ y,
     float* __restrict__ workspace, unsigned rows, unsigned input_width,
-    unsigned output_width, unsigned block_shift, UnitSplit split
+    unsigned output_width, unsigned block_shift, UnitSplit split,
+    LoraEpilogue lora
 ) {
     constexpr int kRows = 16 * kBlocks;
     // float4 copies per thread to move one x tile
@@ -256,12 +257,28 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
                 const float addend = bias != nullptr ? bias[n] : 0.0F;
 #pragma unroll
                 for (int b = 0; b < kBlocks; ++b) {
+                    float term[4] = {0.0F, 0.0F, 0.0F, 0.0F};
+                    if (lora.reduced != nullptr) {  // uniform
+                        const float* reduced_rows[4];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const unsigned m =
+                                min(16U * b + 4 * quarter + r, rows - 1);
+                            reduced_rows[r] =
+                                lora.reduced +
+                                static_cast<std::size_t>(m) * lora.rank;
+                        }
+                        lora_terms<4>(
+                            term,
+                            lora.b + static_cast<std::size_t>(n) * lora.rank,
+                            reduced_rows, lora.rank, lora.scale);
+                    }
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const unsigned m = 16 * b + 4 * quarter + r;
                         if (m < rows) {
                             y[static_cast<std::size_t>(m) * output_width + n] =
-                                acc[b][r] + addend;
+                                (acc[b][r] + addend) + term[r];
                         }
                     }
                 }
@@ -410,7 +427,7 @@ template <int kBlocks>
 __global__ __launch_bounds__(256) void skinny_reduce_kernel(
     const float* __restrict__ workspace, const float* __restrict__ bias,
     float* __restrict__ y, unsigned rows, unsigned output_width,
-    UnitSplit split
+    UnitSplit split, LoraEpilogue lora
 ) {
     constexpr int kRows = 16 * kBlocks;
     constexpr int kBatch = 8;  // partial tiles fetched together
@@ -451,6 +468,9 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(
     }
     if (bias != nullptr) {
         sum += bias[n];
+    }
+    if (lora.reduced != nullptr) {
+        sum += lora_term(lora, m, n);
     }
     y[static_cast<std::size_t>(m) * output_width + n] = sum;
 }
@@ -539,13 +559,13 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     kernel<<<groups, kThreads, kSharedBytes, stream>>>(
         p.activations, p.weight, p.bias, p.result, workspace,
         static_cast<unsigned>(p.rows), static_cast<unsigned>(p.input_width),
-        static_cast<unsigned>(p.output_width), p.block_shift, split);
+        static_cast<unsigned>(p.output_width), p.block_shift, split, p.lora);
     if (partial_tiles) {
         const dim3 reduce_grid(
             tiles, static_cast<unsigned>((p.rows * kTileN + 255) / 256));
         skinny_reduce_kernel<kBlocks><<<reduce_grid, 256, 0, stream>>>(
             workspace, p.bias, p.result, static_cast<unsigned>(p.rows),
-            static_cast<unsigned>(p.output_width), split);
+            static_cast<unsigned>(p.output_width), split, p.lora);
     }
     return hipSuccess;
 }

@@ -7,7 +7,9 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cmath>
 #include <cstdarg>
+#include <cstdint>
 #include <cstdio>
 #include <cstring>
 #include <limits>
@@ -338,12 +340,24 @@ rthip_status rthip_nf4_select_algorithm(
     return ok();
 }
 
-rthip_status rthip_nf4_linear_forward_with(
+namespace {
+
+// The adapter arguments of the *_lora_* entry points; a == nullptr: none.
+struct LoraArguments {
+    const float* a;
+    const float* b;
+    uint64_t rank;
+    float scale;
+    float* reduced;
+};
+
+rthip_status linear_forward_common(
     int32_t algorithm, const float* x, const uint8_t* codes,
     const void* primary_scales, const float* secondary_scales,
     int32_t encoding, uint64_t second_level_block, float offset,
-    const float* bias_or_null, float* y, uint64_t rows, uint64_t input_width,
-    uint64_t output_width, uint64_t block_size, void* stream
+    const float* bias_or_null, const LoraArguments& lora, float* y,
+    uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream
 ) {
     if (x == nullptr || y == nullptr) {
         return fail(RTHIP_INVALID_ARGUMENT,
@@ -376,6 +390,16 @@ rthip_status rthip_nf4_linear_forward_with(
     problem.input_width = input_width;
     problem.output_width = output_width;
     const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+
+    if (lora.a != nullptr) {
+        // reduced = x A^T first; the main kernel's epilogue consumes it.
+        rthip::launch_lora_reduce(x, lora.a, lora.reduced, rows, input_width,
+                                  lora.rank, hip_stream);
+        problem.lora.reduced = lora.reduced;
+        problem.lora.b = lora.b;
+        problem.lora.rank = static_cast<unsigned>(lora.rank);
+        problem.lora.scale = lora.scale;
+    }
 
     if (algorithm == RTHIP_NF4_ALGORITHM_AUTO) {
         algorithm = select_forward(problem);
@@ -420,6 +444,95 @@ rthip_status rthip_nf4_linear_forward_with(
                     static_cast<int>(algorithm));
     }
     return finish_launch("NF4 linear forward launch");
+}
+
+rthip_status check_lora_arguments(const LoraArguments& lora, const float* x,
+                                  const float* y, uint64_t rows,
+                                  uint64_t input_width,
+                                  uint64_t output_width) {
+    if (lora.a == nullptr || lora.b == nullptr || lora.reduced == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "adapter matrices and the reduced buffer must not be "
+                    "null");
+    }
+    if (lora.rank == 0 || lora.rank > (1ULL << 20)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "LoRA rank must be greater than zero (and at most 2^20)");
+    }
+    if (!std::isfinite(lora.scale)) {
+        return fail(RTHIP_INVALID_ARGUMENT, "LoRA scale must be finite");
+    }
+    if (lora.rank > UINT64_MAX / sizeof(float) / rows ||
+        lora.rank > UINT64_MAX / sizeof(float) / input_width ||
+        lora.rank > UINT64_MAX / sizeof(float) / output_width) {
+        return fail(RTHIP_INVALID_ARGUMENT, "LoRA dimensions overflow");
+    }
+    const void* const reduced = lora.reduced;
+    if (reduced == static_cast<const void*>(x) ||
+        reduced == static_cast<const void*>(y) ||
+        reduced == static_cast<const void*>(lora.a) ||
+        reduced == static_cast<const void*>(lora.b)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "the reduced buffer must not alias another operand");
+    }
+    return RTHIP_OK;
+}
+
+}  // namespace
+
+rthip_status rthip_nf4_linear_forward_with(
+    int32_t algorithm, const float* x, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset,
+    const float* bias_or_null, float* y, uint64_t rows, uint64_t input_width,
+    uint64_t output_width, uint64_t block_size, void* stream
+) {
+    return linear_forward_common(
+        algorithm, x, codes, primary_scales, secondary_scales, encoding,
+        second_level_block, offset, bias_or_null,
+        LoraArguments{nullptr, nullptr, 0, 0.0F, nullptr}, y, rows,
+        input_width, output_width, block_size, stream);
+}
+
+rthip_status rthip_nf4_lora_linear_forward_with(
+    int32_t algorithm, const float* x, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset,
+    const float* bias_or_null, const float* lora_a, const float* lora_b,
+    uint64_t lora_rank, float lora_scale, float* reduced, float* y,
+    uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream
+) {
+    const LoraArguments lora{lora_a, lora_b, lora_rank, lora_scale, reduced};
+    if (rows == 0 || input_width == 0 || output_width == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "quantized linear dimensions must be greater than zero");
+    }
+    if (const rthip_status status = check_lora_arguments(
+            lora, x, y, rows, input_width, output_width);
+        status != RTHIP_OK) {
+        return status;
+    }
+    return linear_forward_common(
+        algorithm, x, codes, primary_scales, secondary_scales, encoding,
+        second_level_block, offset, bias_or_null, lora, y, rows, input_width,
+        output_width, block_size, stream);
+}
+
+rthip_status rthip_nf4_lora_linear_forward(
+    const float* x, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, const float* bias_or_null,
+    const float* lora_a, const float* lora_b, uint64_t lora_rank,
+    float lora_scale, float* reduced, float* y, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream
+) {
+    return rthip_nf4_lora_linear_forward_with(
+        RTHIP_NF4_ALGORITHM_AUTO, x, codes, primary_scales, secondary_scales,
+        encoding, second_level_block, offset, bias_or_null, lora_a, lora_b,
+        lora_rank, lora_scale, reduced, y, rows, input_width, output_width,
+        block_size, stream);
 }
 
 rthip_status rthip_nf4_linear_forward(

@@ -57,6 +57,36 @@ def linear_forward(x: torch.Tensor, weight: DeviceWeight,
     return out
 
 
+def lora_linear_forward(x: torch.Tensor, weight: DeviceWeight,
+                        lora_a: torch.Tensor, lora_b: torch.Tensor,
+                        lora_scale: float,
+                        bias: Optional[torch.Tensor] = None,
+                        out: Optional[torch.Tensor] = None,
+                        reduced: Optional[torch.Tensor] = None,
+                        algorithm: Optional[int] = None):
+    """y = x . deq(W)^T (+ bias) + lora_scale * (x . A^T) . B^T through
+    rthip_nf4_lora_linear_forward.  Returns (y, reduced) where reduced is
+    x . A^T, [rows, rank]."""
+    for tensor in (x, lora_a, lora_b):
+        assert tensor.is_cuda and tensor.dtype == torch.float32 and \
+            tensor.is_contiguous()
+    rows = x.numel() // weight.input_width
+    rank = lora_a.shape[0]
+    assert tuple(lora_a.shape) == (rank, weight.input_width)
+    assert tuple(lora_b.shape) == (weight.output_width, rank)
+    if out is None:
+        out = torch.empty((rows, weight.output_width), dtype=torch.float32,
+                          device=x.device)
+    if reduced is None:
+        reduced = torch.empty((rows, rank), dtype=torch.float32,
+                              device=x.device)
+    load_library().lora_linear_forward(
+        x.data_ptr(), weight, None if bias is None else bias.data_ptr(),
+        lora_a.data_ptr(), lora_b.data_ptr(), rank, float(lora_scale),
+        reduced.data_ptr(), out.data_ptr(), rows, _stream(), algorithm)
+    return out, reduced
+
+
 def linear_input_backward(dy: torch.Tensor, weight: DeviceWeight,
                           out: Optional[torch.Tensor] = None,
                           algorithm: Optional[int] = None) -> torch.Tensor:

@@ -81,6 +81,23 @@ def test_reports_unavailable_without_a_device(package, library):
         library.linear_forward(0x3000, weight, None, 0x4000, 1)
 
 
+def test_lora_arguments_are_checked_before_any_device_work(package, library):
+    weight = package.DeviceWeight(
+        64, 64, 64, package.SCALE_FLOAT32, _Fake(0x1000), _Fake(0x2000), None)
+    call = library.lora_linear_forward
+    # (x, weight, bias, A, B, rank, scale, reduced, y, rows)
+    with pytest.raises(package.InvalidArgument):
+        call(0x3000, weight, None, 0, 0x6000, 8, 1.0, 0x7000, 0x4000, 1)
+    with pytest.raises(package.InvalidArgument):
+        call(0x3000, weight, None, 0x5000, 0x6000, 0, 1.0, 0x7000, 0x4000, 1)
+    with pytest.raises(package.InvalidArgument):
+        call(0x3000, weight, None, 0x5000, 0x6000, 8, float("inf"), 0x7000,
+             0x4000, 1)
+    with pytest.raises(package.InvalidArgument):  # reduced aliases x
+        call(0x3000, weight, None, 0x5000, 0x6000, 8, 1.0, 0x3000, 0x4000, 1)
+    assert "alias" in library.last_error()
+
+
 class _Fake:
     """Stands in for a tensor: only its address is ever passed on."""
 

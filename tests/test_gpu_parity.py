@@ -352,6 +352,81 @@ def test_decode_shapes_small_batches(gpu, package, library, oracle):
                         oracle_rows=min(rows, 4))
 
 
+# ---- the fused bias + low-rank adapter epilogue ---------------------------
+
+@pytest.mark.parametrize("out_w,in_w,block,rank,row_counts", [
+    (768, 256, 64, 8, (1, 16)),         # the tiny parity layer
+    (33, 33, 32, 1, (2,)),              # shape-agnostic kernels, rank one
+    (1000, 1600, 64, 2, (1, 5, 70)),    # rank that is not a multiple of 4
+    (4096, 4096, 64, 16, (1, 4, 64, 300)),
+    (512, 2048, 128, 100, (3, 40)),     # more than one 64-row adapter chunk
+])
+@pytest.mark.parametrize("double_quantized", [False, True])
+def test_lora_linear_forward(gpu, package, library, oracle, out_w, in_w,
+                             block, rank, row_counts, double_quantized):
+    """y = x.deq(W)^T + b + s.(x.A^T).B^T against the oracle's restatement of
+    the reference's composition and against fp64; every kernel family.
+    Tolerance: 1e-5 of an output's standard deviation (and the oracle's own
+    distance from fp64 on top, for the comparison with the oracle)."""
+    dense = helpers.normal(100, (out_w, in_w), 0.02)
+    weight = oracle.quantize(dense, block, double_quantized, 64)
+    device_weight = upload(gpu, weight)
+    deq = oracle.dequantize(weight).astype(np.float64)
+    lora_a = helpers.normal(101, (rank, in_w), 0.05)
+    lora_b = helpers.normal(102, (out_w, rank), 0.05)
+    bias = helpers.normal(103, (out_w,), 0.01)
+    lora_scale = 16.0 / rank
+    for rows in row_counts:
+        x = helpers.normal(104 + rows, (rows, in_w), 1.0)
+        x64 = x.astype(np.float64)
+        exact_reduced = x64 @ lora_a.astype(np.float64).T
+        exact = (x64 @ deq.T + bias.astype(np.float64)[None, :] +
+                 lora_scale * (exact_reduced @ lora_b.astype(np.float64).T))
+        unit = helpers.rms(exact)
+        sample = slice(0, min(rows, 5))
+        cpu = oracle.lora_forward(x[sample], weight, lora_a, lora_b,
+                                  lora_scale, bias)
+        cpu_error = np.abs(cpu - exact[sample]).max() / unit
+        for family in families(package):
+            try:
+                y, reduced = gpu.lora_linear_forward(
+                    to_device(x), device_weight, to_device(lora_a),
+                    to_device(lora_b), lora_scale, bias=to_device(bias),
+                    algorithm=family)
+            except package.Unsupported:
+                assert family is not None
+                continue
+            y, reduced = host(y), host(reduced)
+            name = package.ALGORITHM_NAMES[family or 0]
+            reduced_error = np.abs(reduced - exact_reduced).max() / \
+                helpers.rms(exact_reduced)
+            assert reduced_error <= TOLERANCE, \
+                f"x.A^T/{name} rows={rows}: {reduced_error:.3g}"
+            error = np.abs(y - exact).max() / unit
+            assert error <= TOLERANCE, \
+                f"lora forward/{name} rows={rows} vs fp64: {error:.3g}"
+            drift = np.abs(y[sample] - cpu).max() / unit
+            assert drift <= TOLERANCE + cpu_error, \
+                f"lora forward/{name} rows={rows} vs oracle: {drift:.3g}"
+
+
+def test_lora_with_zero_b_equals_the_plain_forward(gpu, package, library,
+                                                   oracle):
+    """A freshly attached adapter (B = 0) leaves the output bit-identical to
+    the plain kernel's."""
+    dense = helpers.normal(110, (4096, 4096), 0.02)
+    weight = oracle.quantize(dense, 64)
+    device_weight = upload(gpu, weight)
+    lora_a = to_device(helpers.normal(111, (16, 4096), 0.05))
+    lora_b = to_device(np.zeros((4096, 16), dtype=np.float32))
+    for rows in (1, 16, 200):
+        x = to_device(helpers.normal(112 + rows, (rows, 4096), 1.0))
+        plain = host(gpu.linear_forward(x, device_weight))
+        fused, _ = gpu.lora_linear_forward(x, device_weight, lora_a, lora_b,
+                                           1.0)
+        helpers.assert_bit_equal(host(fused), plain)
+
+
 # ---- the ABI's error behaviour on a live device --------------------------
 
 def test_abi_rejects_bad_arguments(gpu, package, library, oracle):
