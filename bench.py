@@ -17,6 +17,7 @@ The same JSON line carries
   gemm          M = 2048 forward and input-backward GEMMs of BASELINE configs 4
                 and 5 with their fp32-MFMA rooflines
   small_batch   M in {4, 16, 64} on the three distinct shapes (config 3)
+  lora          the fused bias + rank-16 adapter forward beside the plain one
   cpu_baseline  the reference CPU backend (oracle/_ref, else the C
                 restatement) timed on this host, single thread, on one layer
 
@@ -240,6 +241,50 @@ def bench_small_batch(package, device, torch, steps):
     return results
 
 
+def bench_lora(package, device, torch, steps):
+    """The fused bias + low-rank adapter forward (rank 16) beside the plain
+    forward on the same weights: what the adapter costs per call."""
+    results = []
+    rank = 16
+    for name, out_w, in_w in (LAYER_SHAPES[0], LAYER_SHAPES[4]):
+        copies = 36 if out_w * in_w < 2 ** 25 else 12
+        weights = [synthetic_weight(package, torch, out_w, in_w, False, 700 + i)
+                   for i in range(copies)]
+        lora_a = torch.randn(rank, in_w, device="cuda") * 0.05
+        lora_b = torch.randn(out_w, rank, device="cuda") * 0.05
+        bias = torch.randn(out_w, device="cuda") * 0.01
+        for rows in (1, 16, 2048):
+            used = weights if rows < 2048 else weights[:2]
+            source = torch.randn(rows, in_w, device="cuda")
+            target = torch.empty(rows, out_w, device="cuda")
+            reduced = torch.empty(rows, rank, device="cuda")
+
+            def plain():
+                for weight in used:
+                    device.linear_forward(source, weight, bias, out=target)
+
+            def fused():
+                for weight in used:
+                    device.lora_linear_forward(
+                        source, weight, lora_a, lora_b, 1.0, bias=bias,
+                        out=target, reduced=reduced)
+
+            timings = {}
+            for label, body in (("plain", plain), ("fused", fused)):
+                body()
+                torch.cuda.synchronize()
+                body = capture(torch, body)
+                body()
+                timings[label] = time_region(torch, body, steps) / (
+                    steps * len(used)) * 1e3
+            results.append({
+                "shape": name, "rows": rows, "rank": rank,
+                "plain_us": timings["plain"], "with_adapter_us": timings["fused"],
+            })
+        del weights
+    return results
+
+
 def cpu_baseline(budget_seconds=12.0):
     """The reference CPU backend (oracle/_ref when built, else the C
     restatement) on this host, single thread: whole Llama-7B layers (7
@@ -347,6 +392,8 @@ def main():
                                   max(3, arguments.steps // 4))
         line["small_batch"] = bench_small_batch(package, device, torch,
                                                 max(3, arguments.steps // 4))
+        line["lora"] = bench_lora(package, device, torch,
+                                  max(3, arguments.steps // 4))
     if not arguments.skip_cpu:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))

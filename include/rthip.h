@@ -177,6 +177,9 @@ rthip_status rthip_nf4_linear_input_backward(
  *   lora_scale = alpha / rank            (LowRankAdapter::scale)
  *   reduced  [rows, lora_rank]  caller-provided device buffer that receives
  *            x.A^T (the saved activation the adapter's backward needs)
+ * lora_a may be NULL: `reduced` then already holds x.A^T (from
+ * rthip_lora_reduce, for example one launch over the stacked A matrices of
+ * several projections that share x) and only the second launch is made.
  * Rounding follows the reference: the rank sum in fp32 in ascending order,
  * times lora_scale, added to (product + bias).
  */
@@ -188,6 +191,17 @@ rthip_status rthip_nf4_lora_linear_forward(
     float lora_scale, float* reduced, float* y, uint64_t rows,
     uint64_t input_width, uint64_t output_width, uint64_t block_size,
     void* stream);
+
+/*
+ * reduced[r,j] = sum_k x[r,k] * A[j,k]: matmul(x, transpose(A)), the first
+ * product of LowRankAdapter::forward (src/nn/low_rank_adapter.cpp:140-143).
+ * x is [rows, input_width], lora_a [lora_rank, input_width], reduced
+ * [rows, lora_rank].
+ */
+rthip_status rthip_lora_reduce(const float* x, const float* lora_a,
+                               float* reduced, uint64_t rows,
+                               uint64_t input_width, uint64_t lora_rank,
+                               void* stream);
 
 /* The same two operations with the kernel family pinned (tests, measurement).
  * RTHIP_UNSUPPORTED when `algorithm` cannot handle the shape. */

@@ -96,6 +96,7 @@ _PROTOTYPES = {
         [_i32, _ptr] + _WEIGHT + [_ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
     "rthip_nf4_linear_input_backward_with": (
         _i32, [_i32, _ptr] + _WEIGHT + [_ptr, _u64, _u64, _u64, _u64, _ptr]),
+    "rthip_lora_reduce": (_i32, [_ptr, _ptr, _ptr, _u64, _u64, _u64, _ptr]),
     "rthip_nf4_lora_linear_forward": (
         _i32,
         [_ptr] + _WEIGHT + [_ptr, _ptr, _ptr, _u64, _f32, _ptr, _ptr, _u64,
@@ -246,8 +247,15 @@ class Library:
                 algorithm, x_ptr, *weight.abi_arguments(), *tail)
         self._check(status)
 
+    def lora_reduce(self, x_ptr: int, lora_a_ptr: int, reduced_ptr: int,
+                    rows: int, input_width: int, rank: int,
+                    stream: int = 0) -> None:
+        self._check(self._lib.rthip_lora_reduce(
+            x_ptr, lora_a_ptr, reduced_ptr, rows, input_width, rank, stream))
+
     def lora_linear_forward(self, x_ptr: int, weight: DeviceWeight,
-                            bias_ptr: Optional[int], lora_a_ptr: int,
+                            bias_ptr: Optional[int],
+                            lora_a_ptr: Optional[int],
                             lora_b_ptr: int, rank: int, lora_scale: float,
                             reduced_ptr: int, y_ptr: int, rows: int,
                             stream: int = 0,

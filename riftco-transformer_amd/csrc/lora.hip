@@ -4,14 +4,14 @@
 // [rank, input_width]; the result is tiny ([rows, rank]) and is consumed by
 // the epilogue of the packed-weight kernels (lora_epilogue.hpp).
 //
-// x is read exactly once.  A workgroup of sixteen wavefronts owns 16 rows of x
-// and up to 64 adapter rows; the contraction axis is cut into sixteen spans,
+// Up to 64 rows: one workgroup per output element (lora_reduce_rows_kernel).
+// Beyond that x is read exactly once: a workgroup of sixteen wavefronts owns
+// 16 rows of x and up to 64 adapter rows; the contraction axis is cut into
+// sixteen spans,
 // one per wavefront, which each run v_mfma_f32_16x16x4_f32 over their span
 // (A operand: x[16 rows][4 k]; B operand: A^T[4 k][16 adapter rows]) from
 // 16-byte loads, and the sixteen partial tiles are added through LDS in
-// wavefront order.  With one token (rows = 1) this is a single workgroup whose
-// wavefronts each see 1/16 of the row, which keeps the latency of the whole
-// product near one memory round trip.
+// wavefront order.
 //
 // Loads are raw buffer loads; lanes past the last row, the last adapter row or
 // the row end get an offset the range check rejects and read zeros.
@@ -144,6 +144,63 @@ __global__ __launch_bounds__(kThreads) void lora_reduce_kernel(
     }
 }
 
+// Few rows (decode and small batches): one workgroup per output element, so
+// that the product takes one memory round trip however small it is.  Thread t
+// takes float4 chunks t, t + 256, ...; the 256 partial sums are added with
+// DPP-free shuffles inside each wavefront and then in wavefront order.
+constexpr int kDotThreads = 256;
+
+__global__ __launch_bounds__(kDotThreads) void lora_reduce_rows_kernel(
+    const float* __restrict__ x, const float* __restrict__ a,
+    float* __restrict__ reduced, unsigned input_width, unsigned rank
+) {
+    __shared__ float wave_sums[kDotThreads / 64];
+    const unsigned j = blockIdx.x;
+    const unsigned m = blockIdx.y;
+    const float4* x_row = reinterpret_cast<const float4*>(
+        x + static_cast<std::size_t>(m) * input_width);
+    const float4* a_row = reinterpret_cast<const float4*>(
+        a + static_cast<std::size_t>(j) * input_width);
+    const unsigned chunks = input_width / 4;
+    float sum = 0.0F;
+    constexpr int kUnroll = 4;
+    for (unsigned c0 = threadIdx.x; c0 < chunks; c0 += kDotThreads * kUnroll) {
+        float4 xv[kUnroll];
+        float4 av[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const unsigned c = c0 + kDotThreads * u;
+            const bool valid = c < chunks;
+            const unsigned clamped = valid ? c : 0;
+            xv[u] = x_row[clamped];
+            av[u] = valid ? a_row[clamped] : make_float4(0.0F, 0.0F, 0.0F, 0.0F);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            sum += xv[u].x * av[u].x;
+            sum += xv[u].y * av[u].y;
+            sum += xv[u].z * av[u].z;
+            sum += xv[u].w * av[u].w;
+        }
+    }
+#pragma unroll
+    for (int offset = 32; offset >= 1; offset /= 2) {
+        sum += __shfl_xor(sum, offset, 64);
+    }
+    if (threadIdx.x % 64 == 0) {
+        wave_sums[threadIdx.x / 64] = sum;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float total = 0.0F;
+#pragma unroll
+        for (int w = 0; w < kDotThreads / 64; ++w) {
+            total += wave_sums[w];
+        }
+        reduced[static_cast<std::size_t>(m) * rank + j] = total;
+    }
+}
+
 // Any shape and alignment: one wavefront per output.
 __global__ __launch_bounds__(256) void lora_reduce_generic_kernel(
     const float* __restrict__ x, const float* __restrict__ a,
@@ -188,6 +245,14 @@ void launch_lora_reduce(const float* x, const float* a, float* reduced,
         const unsigned blocks = static_cast<unsigned>((waves + 3) / 4);
         lora_reduce_generic_kernel<<<blocks, 256, 0, stream>>>(
             x, a, reduced, rows, input_width, rank);
+        return;
+    }
+    if (rows <= 64 && rank <= 65535) {
+        lora_reduce_rows_kernel<<<dim3(static_cast<unsigned>(rank),
+                                       static_cast<unsigned>(rows)),
+                                  kDotThreads, 0, stream>>>(
+            x, a, reduced, static_cast<unsigned>(input_width),
+            static_cast<unsigned>(rank));
         return;
     }
     const unsigned row_tiles = static_cast<unsigned>((rows + 15) / 16);

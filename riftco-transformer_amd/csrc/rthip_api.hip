@@ -391,10 +391,12 @@ rthip_status linear_forward_common(
     problem.output_width = output_width;
     const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
 
-    if (lora.a != nullptr) {
-        // reduced = x A^T first; the main kernel's epilogue consumes it.
-        rthip::launch_lora_reduce(x, lora.a, lora.reduced, rows, input_width,
-                                  lora.rank, hip_stream);
+    if (lora.reduced != nullptr) {
+        if (lora.a != nullptr) {
+            // reduced = x A^T first; the main kernel's epilogue consumes it.
+            rthip::launch_lora_reduce(x, lora.a, lora.reduced, rows,
+                                      input_width, lora.rank, hip_stream);
+        }
         problem.lora.reduced = lora.reduced;
         problem.lora.b = lora.b;
         problem.lora.rank = static_cast<unsigned>(lora.rank);
@@ -450,10 +452,10 @@ rthip_status check_lora_arguments(const LoraArguments& lora, const float* x,
                                   const float* y, uint64_t rows,
                                   uint64_t input_width,
                                   uint64_t output_width) {
-    if (lora.a == nullptr || lora.b == nullptr || lora.reduced == nullptr) {
+    if (lora.b == nullptr || lora.reduced == nullptr) {
         return fail(RTHIP_INVALID_ARGUMENT,
-                    "adapter matrices and the reduced buffer must not be "
-                    "null");
+                    "the adapter's B matrix and the reduced buffer must not "
+                    "be null");
     }
     if (lora.rank == 0 || lora.rank > (1ULL << 20)) {
         return fail(RTHIP_INVALID_ARGUMENT,
@@ -517,6 +519,39 @@ rthip_status rthip_nf4_lora_linear_forward_with(
         algorithm, x, codes, primary_scales, secondary_scales, encoding,
         second_level_block, offset, bias_or_null, lora, y, rows, input_width,
         output_width, block_size, stream);
+}
+
+rthip_status rthip_lora_reduce(const float* x, const float* lora_a,
+                               float* reduced, uint64_t rows,
+                               uint64_t input_width, uint64_t lora_rank,
+                               void* stream) {
+    if (x == nullptr || lora_a == nullptr || reduced == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "x, the adapter's A matrix and the reduced buffer must "
+                    "not be null");
+    }
+    if (rows == 0 || input_width == 0 || lora_rank == 0 ||
+        lora_rank > (1ULL << 20)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "rows, input width and LoRA rank must be greater than "
+                    "zero (rank at most 2^20)");
+    }
+    if (input_width > UINT64_MAX / sizeof(float) / rows ||
+        input_width > UINT64_MAX / sizeof(float) / lora_rank) {
+        return fail(RTHIP_INVALID_ARGUMENT, "LoRA dimensions overflow");
+    }
+    if (static_cast<const void*>(reduced) == static_cast<const void*>(x) ||
+        static_cast<const void*>(reduced) ==
+            static_cast<const void*>(lora_a)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "the reduced buffer must not alias another operand");
+    }
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    rthip::launch_lora_reduce(x, lora_a, reduced, rows, input_width,
+                              lora_rank, static_cast<hipStream_t>(stream));
+    return finish_launch("LoRA reduce launch");
 }
 
 rthip_status rthip_nf4_lora_linear_forward(

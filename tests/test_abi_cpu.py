@@ -86,8 +86,10 @@ def test_lora_arguments_are_checked_before_any_device_work(package, library):
         64, 64, 64, package.SCALE_FLOAT32, _Fake(0x1000), _Fake(0x2000), None)
     call = library.lora_linear_forward
     # (x, weight, bias, A, B, rank, scale, reduced, y, rows)
-    with pytest.raises(package.InvalidArgument):
-        call(0x3000, weight, None, 0, 0x6000, 8, 1.0, 0x7000, 0x4000, 1)
+    with pytest.raises(package.InvalidArgument):  # B missing
+        call(0x3000, weight, None, 0x5000, 0, 8, 1.0, 0x7000, 0x4000, 1)
+    with pytest.raises(package.InvalidArgument):  # reduced missing
+        call(0x3000, weight, None, 0x5000, 0x6000, 8, 1.0, 0, 0x4000, 1)
     with pytest.raises(package.InvalidArgument):
         call(0x3000, weight, None, 0x5000, 0x6000, 0, 1.0, 0x7000, 0x4000, 1)
     with pytest.raises(package.InvalidArgument):
@@ -96,6 +98,10 @@ def test_lora_arguments_are_checked_before_any_device_work(package, library):
     with pytest.raises(package.InvalidArgument):  # reduced aliases x
         call(0x3000, weight, None, 0x5000, 0x6000, 8, 1.0, 0x3000, 0x4000, 1)
     assert "alias" in library.last_error()
+    with pytest.raises(package.InvalidArgument):
+        library.lora_reduce(0x3000, 0, 0x7000, 1, 64, 8)
+    with pytest.raises(package.InvalidArgument):
+        library.lora_reduce(0x3000, 0x5000, 0x7000, 1, 64, 0)
 
 
 class _Fake:

@@ -410,6 +410,37 @@ def test_lora_linear_forward(gpu, package, library, oracle, out_w, in_w,
                 f"lora forward/{name} rows={rows} vs oracle: {drift:.3g}"
 
 
+def test_lora_forward_with_a_precomputed_first_product(gpu, package, library,
+                                                       oracle):
+    """One rthip_lora_reduce over the stacked A matrices of two projections
+    that share x, then two forwards that take their slice of the result."""
+    import torch
+    rows, in_w, rank = 3, 1024, 8
+    x = to_device(helpers.normal(120, (rows, in_w), 1.0))
+    stacked_a = to_device(helpers.normal(121, (2 * rank, in_w), 0.05))
+    reduced = torch.empty((rows, 2 * rank), dtype=torch.float32,
+                          device="cuda")
+    library.lora_reduce(x.data_ptr(), stacked_a.data_ptr(),
+                        reduced.data_ptr(), rows, in_w, 2 * rank,
+                        torch.cuda.current_stream().cuda_stream)
+    for index, out_w in enumerate((256, 640)):
+        dense = helpers.normal(122 + index, (out_w, in_w), 0.02)
+        weight = oracle.quantize(dense, 64)
+        device_weight = upload(gpu, weight)
+        lora_a = stacked_a[index * rank:(index + 1) * rank].contiguous()
+        lora_b = to_device(helpers.normal(124 + index, (out_w, rank), 0.05))
+        mine = reduced[:, index * rank:(index + 1) * rank].contiguous()
+        want, want_reduced = gpu.lora_linear_forward(
+            x, device_weight, lora_a, lora_b, 2.0)
+        helpers.assert_bit_equal(host(mine), host(want_reduced))
+        got = torch.empty_like(want)
+        library.lora_linear_forward(
+            x.data_ptr(), device_weight, None, None, lora_b.data_ptr(), rank,
+            2.0, mine.data_ptr(), got.data_ptr(), rows,
+            torch.cuda.current_stream().cuda_stream)
+        helpers.assert_bit_equal(host(got), host(want))
+
+
 def test_lora_with_zero_b_equals_the_plain_forward(gpu, package, library,
                                                    oracle):
     """A freshly attached adapter (B = 0) leaves the output bit-identical to
