@@ -18,6 +18,7 @@ The same JSON line carries
                 and 5 with their fp32-MFMA rooflines
   small_batch   M in {4, 16, 64} on the three distinct shapes (config 3)
   lora          the fused bias + rank-16 adapter forward beside the plain one
+  matmul        dense fp32 matmul at layer and adapter shapes
   cpu_baseline  the reference CPU backend (oracle/_ref, else the C
                 restatement) timed on this host, single thread, on one layer
 
@@ -285,6 +286,31 @@ def bench_lora(package, device, torch, steps):
     return results
 
 
+def bench_matmul(package, device, torch, steps):
+    """Dense fp32 matmul at the layer's shapes and at adapter shapes."""
+    results = []
+    for rows, shared, columns in ((2048, 4096, 4096), (2048, 4096, 11008),
+                                  (2048, 16, 4096), (2048, 4096, 16)):
+        left = torch.randn(rows, shared, device="cuda")
+        right = torch.randn(shared, columns, device="cuda") * 0.02
+        out = torch.empty(rows, columns, device="cuda")
+        body = lambda: device.matmul(left, right, out=out)
+        body()
+        body()
+        milliseconds = time_region(torch, body, steps) / steps
+        tflops = 2.0 * rows * shared * columns / (milliseconds / 1e3) / 1e12
+        results.append({
+            "rows": rows, "shared": shared, "columns": columns,
+            "ms": milliseconds,
+            "roofline": {"bound": "mfma", "achieved": tflops,
+                         "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
+                         "traffic": None},
+        })
+        del left, right, out
+    return results
+
+
 def cpu_baseline(budget_seconds=12.0):
     """The reference CPU backend (oracle/_ref when built, else the C
     restatement) on this host, single thread: whole Llama-7B layers (7
@@ -394,6 +420,8 @@ def main():
                                                 max(3, arguments.steps // 4))
         line["lora"] = bench_lora(package, device, torch,
                                   max(3, arguments.steps // 4))
+        line["matmul"] = bench_matmul(package, device, torch,
+                                      max(3, arguments.steps // 4))
     if not arguments.skip_cpu:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))

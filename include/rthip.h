@@ -193,6 +193,18 @@ rthip_status rthip_nf4_lora_linear_forward(
     void* stream);
 
 /*
+ * out[b][r,c] = sum_k left[b][r,k] * right[b][k,c]
+ *
+ * Replaces BackendAdapter::matmul (src/core/backend/adapter.hpp:46-52; CPU form
+ * src/core/backend/adapters/cpu/adapter.cpp:158-203) with MatmulDimensions
+ * {batch_count, rows, shared, columns}: contiguous row-major operands, no
+ * batch broadcasting, output overwritten.
+ */
+rthip_status rthip_matmul(const float* left, const float* right, float* out,
+                          uint64_t batch_count, uint64_t rows,
+                          uint64_t shared, uint64_t columns, void* stream);
+
+/*
  * reduced[r,j] = sum_k x[r,k] * A[j,k]: matmul(x, transpose(A)), the first
  * product of LowRankAdapter::forward (src/nn/low_rank_adapter.cpp:140-143).
  * x is [rows, input_width], lora_a [lora_rank, input_width], reduced

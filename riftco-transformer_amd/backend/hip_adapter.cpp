@@ -492,8 +492,26 @@ public:
     // capabilities without a native kernel run the reference host loops on
     // the storage's host spans; the mirror of HipTensorStorage keeps those
     // coherent with HBM.
+    // Dense matmul runs on the device (BackendAdapter::matmul,
+    // src/core/backend/adapter.hpp:46-52).
     void matmul(const MatmulRequest& request) const override {
-        cpu_backend_adapter().matmul(request);
+        constexpr std::string_view operation = "matmul";
+        const HipRuntime& runtime = require_runtime();
+        const auto& left = require_hip_tensor(request.left, operation);
+        const auto& right = require_hip_tensor(request.right, operation);
+        auto& output = require_hip_tensor(request.output, operation);
+        const float* left_device = left.device_for_read();
+        const float* right_device = right.device_for_read();
+        check(runtime,
+              runtime.matmul(left_device, right_device,
+                             output.device_for_overwrite(),
+                             request.dimensions.batch_count,
+                             request.dimensions.rows,
+                             request.dimensions.shared,
+                             request.dimensions.columns, nullptr),
+              operation);
+        check(runtime, runtime.stream_synchronize(nullptr),
+              "matmul synchronisation");
     }
     void unary_elementwise(
         const UnaryElementwiseRequest& request) const override {

@@ -83,7 +83,8 @@ void load(HipRuntime& runtime) {
         !bind(library, "rthip_nf4_linear_input_backward",
               runtime.nf4_linear_input_backward, reason) ||
         !bind(library, "rthip_nf4_dequantize", runtime.nf4_dequantize,
-              reason)) {
+              reason) ||
+        !bind(library, "rthip_matmul", runtime.matmul, reason)) {
         return;
     }
     if ((abi_version() >> 16) != RTHIP_ABI_VERSION_MAJOR) {

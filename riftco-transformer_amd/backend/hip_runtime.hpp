@@ -38,6 +38,7 @@ struct HipRuntime {
     decltype(&rthip_nf4_linear_input_backward) nf4_linear_input_backward =
         nullptr;
     decltype(&rthip_nf4_dequantize) nf4_dequantize = nullptr;
+    decltype(&rthip_matmul) matmul = nullptr;
 };
 
 // Process-lifetime runtime; loading happens once, on the first call.

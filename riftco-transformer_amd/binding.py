@@ -96,6 +96,8 @@ _PROTOTYPES = {
         [_i32, _ptr] + _WEIGHT + [_ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
     "rthip_nf4_linear_input_backward_with": (
         _i32, [_i32, _ptr] + _WEIGHT + [_ptr, _u64, _u64, _u64, _u64, _ptr]),
+    "rthip_matmul": (
+        _i32, [_ptr, _ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
     "rthip_lora_reduce": (_i32, [_ptr, _ptr, _ptr, _u64, _u64, _u64, _ptr]),
     "rthip_nf4_lora_linear_forward": (
         _i32,
@@ -246,6 +248,13 @@ class Library:
             status = self._lib.rthip_nf4_linear_forward_with(
                 algorithm, x_ptr, *weight.abi_arguments(), *tail)
         self._check(status)
+
+    def matmul(self, left_ptr: int, right_ptr: int, out_ptr: int,
+               batch_count: int, rows: int, shared: int, columns: int,
+               stream: int = 0) -> None:
+        self._check(self._lib.rthip_matmul(
+            left_ptr, right_ptr, out_ptr, batch_count, rows, shared, columns,
+            stream))
 
     def lora_reduce(self, x_ptr: int, lora_a_ptr: int, reduced_ptr: int,
                     rows: int, input_width: int, rank: int,

@@ -1,0 +1,300 @@
+// Dense fp32 matmul  out[b] [M, N] = left[b] [M, K] * right[b] [K, N]
+// (row-major, batched), restating BackendAdapter::matmul as the CPU adapter
+// computes it (src/core/backend/adapters/cpu/adapter.cpp:158-203 under
+// /root/reference).  In a QLoRA layer this is every product that is not the
+// packed one: the adapter's x A^T, (.) B^T and their gradients.
+//
+// Tiling is the one of the packed GEMM (nf4_mfma.hip): a workgroup of four
+// wavefronts computes a 128 x 128 output tile in steps of 32 along K, each
+// wavefront owns a 64 x 64 quadrant as 2 x 2 blocks of v_mfma_f32_32x32x2_f32,
+// both LDS tiles are [row-or-column][k] with a padded stride of 36 floats and
+// are read with one ds_read_b128 per lane per four MFMAs, global loads of step
+// t + 1 are issued before the MFMAs of step t, and accumulation is two-level
+// (chains of 256 contraction values folded into a second accumulator).
+// The right operand is [K, N]: a step reads 32 of its rows x 128 contiguous
+// columns and transposes while writing LDS.  All edges (M, N, K not multiples
+// of the tile) are handled by zero-filling; only K % 4 == 0, N % 4 == 0 and
+// 16-byte aligned pointers are required -- other shapes take the plain kernel
+// below, which is also the exact restatement of the reference loop (one fp32
+// accumulator per output, ascending k).
+
+#include "kernels.hpp"
+
+namespace rthip {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int kTileM = 128;
+constexpr int kTileN = 128;
+constexpr int kTileK = 32;
+constexpr int kStride = 36;
+constexpr unsigned kFlushSteps = 8;
+
+struct MatmulShape {
+    unsigned rows;     // M
+    unsigned shared;   // K
+    unsigned columns;  // N
+};
+
+struct Staged {
+    float4 left[4];
+    float4 right[4];
+};
+
+__device__ __forceinline__ float4 zero4() {
+    return make_float4(0.0F, 0.0F, 0.0F, 0.0F);
+}
+
+// left tile: rows row0..row0+127, 32 contraction values from k0.  Thread t
+// takes float4 column t % 8 of rows t / 8 + 32 * pass.
+__device__ __forceinline__ void load_left(Staged& staged,
+                                          const float* __restrict__ left,
+                                          const MatmulShape& shape,
+                                          unsigned row0, unsigned k0) {
+    const unsigned thread = threadIdx.x;
+    const unsigned k = k0 + (thread % 8) * 4;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const unsigned row = row0 + thread / 8 + 32 * pass;
+        staged.left[pass] =
+            row < shape.rows && k < shape.shared
+                ? *reinterpret_cast<const float4*>(
+                      left + static_cast<std::size_t>(row) * shape.shared + k)
+                : zero4();
+    }
+}
+
+// right tile: contraction rows k0..k0+31, columns col0..col0+127.  Thread t
+// takes 16 consecutive columns (t / 32) * 16 of row k0 + t % 32.
+__device__ __forceinline__ void load_right(Staged& staged,
+                                           const float* __restrict__ right,
+                                           const MatmulShape& shape,
+                                           unsigned col0, unsigned k0) {
+    const unsigned thread = threadIdx.x;
+    const unsigned k = k0 + thread % 32;
+    const unsigned column = col0 + (thread / 32) * 16;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        staged.right[q] =
+            k < shape.shared && column + 4 * q < shape.columns
+                ? *reinterpret_cast<const float4*>(
+                      right + static_cast<std::size_t>(k) * shape.columns +
+                      column + 4 * q)
+                : zero4();
+    }
+}
+
+__device__ __forceinline__ void store_tiles(const Staged& staged,
+                                            float* __restrict__ left_tile,
+                                            float* __restrict__ right_tile) {
+    const unsigned thread = threadIdx.x;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        *reinterpret_cast<float4*>(left_tile +
+                                   (thread / 8 + 32 * pass) * kStride +
+                                   (thread % 8) * 4) = staged.left[pass];
+    }
+    // tile[column][k]: transpose while writing.
+    float* destination =
+        right_tile + ((thread / 32) * 16) * kStride + thread % 32;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        destination[(4 * q + 0) * kStride] = staged.right[q].x;
+        destination[(4 * q + 1) * kStride] = staged.right[q].y;
+        destination[(4 * q + 2) * kStride] = staged.right[q].z;
+        destination[(4 * q + 3) * kStride] = staged.right[q].w;
+    }
+}
+
+__global__ __launch_bounds__(kThreads, 2) void dense_matmul_kernel(
+    const float* __restrict__ left, const float* __restrict__ right,
+    float* __restrict__ out, MatmulShape shape
+) {
+    __shared__ __attribute__((aligned(16))) float left_tile[kTileM * kStride];
+    __shared__ __attribute__((aligned(16))) float right_tile[kTileN * kStride];
+
+    const unsigned lane = threadIdx.x % 64;
+    const unsigned wave = threadIdx.x / 64;
+    const unsigned wave_m = wave / 2;
+    const unsigned wave_n = wave % 2;
+    const unsigned row0 = blockIdx.y * kTileM;
+    const unsigned col0 = blockIdx.x * kTileN;
+    const std::size_t batch = blockIdx.z;
+    left += batch * shape.rows * shape.shared;
+    right += batch * shape.shared * shape.columns;
+    out += batch * shape.rows * shape.columns;
+
+    floatx16 acc[2][2];
+    floatx16 total[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                acc[i][j][e] = 0.0F;
+                total[i][j][e] = 0.0F;
+            }
+        }
+    }
+    unsigned steps_since_flush = 0;
+
+    Staged staged;
+    load_left(staged, left, shape, row0, 0);
+    load_right(staged, right, shape, col0, 0);
+
+    const float* left_fragment =
+        left_tile + (wave_m * 64 + lane % 32) * kStride + 4 * (lane / 32);
+    const float* right_fragment =
+        right_tile + (wave_n * 64 + lane % 32) * kStride + 4 * (lane / 32);
+
+    for (unsigned k0 = 0; k0 < shape.shared; k0 += kTileK) {
+        __syncthreads();  // previous step's fragment reads are done
+        store_tiles(staged, left_tile, right_tile);
+        __syncthreads();
+
+        const unsigned next = k0 + kTileK;
+        if (next < shape.shared) {
+            load_left(staged, left, shape, row0, next);
+            load_right(staged, right, shape, col0, next);
+        }
+
+#pragma unroll
+        for (int kk = 0; kk < kTileK; kk += 8) {
+            float4 a[2];
+            float4 b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                a[i] = *reinterpret_cast<const float4*>(
+                    left_fragment + i * 32 * kStride + kk);
+                b[i] = *reinterpret_cast<const float4*>(
+                    right_fragment + i * 32 * kStride + kk);
+            }
+            const float a_values[2][4] = {{a[0].x, a[0].y, a[0].z, a[0].w},
+                                          {a[1].x, a[1].y, a[1].z, a[1].w}};
+            const float b_values[2][4] = {{b[0].x, b[0].y, b[0].z, b[0].w},
+                                          {b[1].x, b[1].y, b[1].z, b[1].w}};
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                            a_values[i][s], b_values[j][s], acc[i][j], 0, 0,
+                            0);
+                    }
+                }
+            }
+        }
+
+        if (++steps_since_flush == kFlushSteps) {
+            steps_since_flush = 0;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        total[i][j][e] += acc[i][j][e];
+                        acc[i][j][e] = 0.0F;
+                    }
+                }
+            }
+        }
+    }
+
+    // Accumulator element e of lane l is output row 8*(e/4) + 4*(l/32) + e%4,
+    // column l%32 of its 32 x 32 block.
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const unsigned column = col0 + wave_n * 64 + j * 32 + lane % 32;
+            if (column >= shape.columns) {
+                continue;
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const unsigned row = row0 + wave_m * 64 + i * 32 +
+                                     8 * (e / 4) + 4 * (lane / 32) + e % 4;
+                if (row < shape.rows) {
+                    out[static_cast<std::size_t>(row) * shape.columns +
+                        column] = total[i][j][e] + acc[i][j][e];
+                }
+            }
+        }
+    }
+}
+
+// Any shape: one thread per output, one fp32 accumulator, ascending k --
+// the reference loop itself.  Neighbouring threads take neighbouring columns.
+__global__ __launch_bounds__(256) void plain_matmul_kernel(
+    const float* __restrict__ left, const float* __restrict__ right,
+    float* __restrict__ out, std::size_t batch_count, std::size_t rows,
+    std::size_t shared, std::size_t columns
+) {
+    const std::size_t per_batch = rows * columns;
+    const std::size_t count = batch_count * per_batch;
+    const std::size_t stride =
+        static_cast<std::size_t>(gridDim.x) * blockDim.x;
+    for (std::size_t index =
+             static_cast<std::size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+         index < count; index += stride) {
+        const std::size_t batch = index / per_batch;
+        const std::size_t row = (index % per_batch) / columns;
+        const std::size_t column = index % columns;
+        const float* a = left + (batch * rows + row) * shared;
+        const float* b = right + batch * shared * columns + column;
+        float sum = 0.0F;
+        for (std::size_t k = 0; k < shared; ++k) {
+            sum += a[k] * b[k * columns];
+        }
+        out[index] = sum;
+    }
+}
+
+}  // namespace
+
+void launch_dense_matmul(const float* left, const float* right, float* out,
+                         std::size_t batch_count, std::size_t rows,
+                         std::size_t shared, std::size_t columns,
+                         hipStream_t stream) {
+    constexpr std::size_t kLimit = 1ULL << 31;
+    const std::size_t tiles_m = (rows + kTileM - 1) / kTileM;
+    const std::size_t tiles_n = (columns + kTileN - 1) / kTileN;
+    const bool tiled =
+        shared % 4 == 0 && columns % 4 == 0 && rows < kLimit &&
+        shared < kLimit && columns < kLimit && tiles_m <= 65535 &&
+        batch_count <= 65535 &&
+        // a matrix-core tile pays off once there is a tile's worth of work
+        rows * columns >= 1024 &&
+        reinterpret_cast<std::uintptr_t>(left) % 16 == 0 &&
+        reinterpret_cast<std::uintptr_t>(right) % 16 == 0;
+    if (tiled) {
+        MatmulShape shape;
+        shape.rows = static_cast<unsigned>(rows);
+        shape.shared = static_cast<unsigned>(shared);
+        shape.columns = static_cast<unsigned>(columns);
+        const dim3 grid(static_cast<unsigned>(tiles_n),
+                        static_cast<unsigned>(tiles_m),
+                        static_cast<unsigned>(batch_count));
+        dense_matmul_kernel<<<grid, kThreads, 0, stream>>>(left, right, out,
+                                                           shape);
+        return;
+    }
+    const std::size_t outputs = batch_count * rows * columns;
+    std::size_t blocks = (outputs + 255) / 256;
+    if (blocks > 65535 * 16) {
+        blocks = 65535 * 16;
+    }
+    if (blocks == 0) {
+        blocks = 1;
+    }
+    plain_matmul_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
+        left, right, out, batch_count, rows, shared, columns);
+}
+
+}  // namespace rthip

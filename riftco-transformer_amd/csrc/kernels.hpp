@@ -59,6 +59,13 @@ void launch_lora_reduce(const float* x, const float* a, float* reduced,
                         std::size_t rows, std::size_t input_width,
                         std::size_t rank, hipStream_t stream);
 
+// dense_matmul.hip -- out[b] = left[b] [rows, shared] * right[b] [shared,
+// columns], plain fp32.
+void launch_dense_matmul(const float* left, const float* right, float* out,
+                         std::size_t batch_count, std::size_t rows,
+                         std::size_t shared, std::size_t columns,
+                         hipStream_t stream);
+
 // nf4_mfma.hip
 bool mfma_forward_supports(const LinearProblem& problem);
 void launch_mfma_forward(const LinearProblem& problem, hipStream_t stream);

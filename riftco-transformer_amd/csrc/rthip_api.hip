@@ -521,6 +521,38 @@ rthip_status rthip_nf4_lora_linear_forward_with(
         output_width, block_size, stream);
 }
 
+rthip_status rthip_matmul(const float* left, const float* right, float* out,
+                          uint64_t batch_count, uint64_t rows,
+                          uint64_t shared, uint64_t columns, void* stream) {
+    if (left == nullptr || right == nullptr || out == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "matmul operands must not be null");
+    }
+    if (batch_count == 0 || rows == 0 || shared == 0 || columns == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "matmul dimensions must be greater than zero");
+    }
+    constexpr uint64_t kMaxElements = UINT64_MAX / sizeof(float);
+    if (rows > kMaxElements / shared || shared > kMaxElements / columns ||
+        rows > kMaxElements / columns ||
+        batch_count > kMaxElements / (rows * shared) ||
+        batch_count > kMaxElements / (shared * columns) ||
+        batch_count > kMaxElements / (rows * columns)) {
+        return fail(RTHIP_INVALID_ARGUMENT, "matmul dimensions overflow");
+    }
+    if (static_cast<const void*>(out) == static_cast<const void*>(left) ||
+        static_cast<const void*>(out) == static_cast<const void*>(right)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "matmul output must not alias an input");
+    }
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    rthip::launch_dense_matmul(left, right, out, batch_count, rows, shared,
+                               columns, static_cast<hipStream_t>(stream));
+    return finish_launch("matmul launch");
+}
+
 rthip_status rthip_lora_reduce(const float* x, const float* lora_a,
                                float* reduced, uint64_t rows,
                                uint64_t input_width, uint64_t lora_rank,

@@ -87,6 +87,27 @@ def lora_linear_forward(x: torch.Tensor, weight: DeviceWeight,
     return out, reduced
 
 
+def matmul(left: torch.Tensor, right: torch.Tensor,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """left [..., rows, shared] x right [..., shared, columns] through
+    rthip_matmul (identical leading batch dimensions, no broadcasting)."""
+    for tensor in (left, right):
+        assert tensor.is_cuda and tensor.dtype == torch.float32 and \
+            tensor.is_contiguous()
+    assert left.shape[:-2] == right.shape[:-2]
+    assert left.shape[-1] == right.shape[-2]
+    rows, shared, columns = left.shape[-2], left.shape[-1], right.shape[-1]
+    batch = 1
+    for extent in left.shape[:-2]:
+        batch *= extent
+    if out is None:
+        out = torch.empty(tuple(left.shape[:-2]) + (rows, columns),
+                          dtype=torch.float32, device=left.device)
+    load_library().matmul(left.data_ptr(), right.data_ptr(), out.data_ptr(),
+                          batch, rows, shared, columns, _stream())
+    return out
+
+
 def linear_input_backward(dy: torch.Tensor, weight: DeviceWeight,
                           out: Optional[torch.Tensor] = None,
                           algorithm: Optional[int] = None) -> torch.Tensor:

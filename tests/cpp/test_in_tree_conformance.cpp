@@ -123,6 +123,30 @@ int main() {
                         "delegated scale must run on hip storage");
             }
         }
+        // Dense matmul through the runtime: [2 x 3] x [3 x 2], batch of 2,
+        // against the reference CPU adapter on the same values.
+        {
+            const std::vector<float> left = {1, 2, 3, 4, 5, 6,
+                                             -1, 0, 2, 0.5F, 1.5F, -2};
+            const std::vector<float> right = {1, 0, 0, 1, 2, -1,
+                                              3, 1, -1, 2, 0, 0.25F};
+            const backend::MatmulDimensions dimensions{2, 2, 3, 2};
+            auto hip_left = hip.make_storage(left);
+            auto hip_right = hip.make_storage(right);
+            auto hip_out = hip.make_storage(8, 0.0F);
+            hip.matmul({*hip_left, *hip_right, *hip_out, dimensions});
+            auto cpu_left = cpu.make_storage(left);
+            auto cpu_right = cpu.make_storage(right);
+            auto cpu_out = cpu.make_storage(8, 0.0F);
+            cpu.matmul({*cpu_left, *cpu_right, *cpu_out, dimensions});
+            const auto ho = std::as_const(*hip_out).data();
+            const auto co = std::as_const(*cpu_out).data();
+            for (std::size_t i = 0; i < co.size(); ++i) {
+                require(ho[i] == co[i], "matmul differs from the reference "
+                                        "CPU adapter");
+            }
+            require(co[0] == 7.0F && co[1] == -1.0F, "matmul known answer");
+        }
         std::cout << "in-tree conformance tests passed\n";
         return 0;
     } catch (const std::exception& error) {

@@ -14,6 +14,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <vector>
 
 extern "C" void nf4o_linear_forward_rowcached(
     const float*, const uint8_t*, const nf4o_scales*, float*, size_t, size_t,
@@ -263,6 +264,78 @@ rthip_status rthip_nf4_dequantize(
     }
     nf4o_dequantize(codes, &scales, element_count, block_size, out);
     return RTHIP_OK;
+}
+
+rthip_status rthip_matmul(const float* left, const float* right, float* out,
+                          uint64_t batch_count, uint64_t rows,
+                          uint64_t shared, uint64_t columns, void*) {
+    if (left == nullptr || right == nullptr || out == nullptr ||
+        batch_count == 0 || rows == 0 || shared == 0 || columns == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT, "invalid matmul arguments");
+    }
+    for (uint64_t batch = 0; batch < batch_count; ++batch) {
+        nf4o_matmul(left + batch * rows * shared,
+                    right + batch * shared * columns,
+                    out + batch * rows * columns, rows, shared, columns);
+    }
+    return RTHIP_OK;
+}
+
+rthip_status rthip_lora_reduce(const float* x, const float* lora_a,
+                               float* reduced, uint64_t rows,
+                               uint64_t input_width, uint64_t lora_rank,
+                               void*) {
+    if (x == nullptr || lora_a == nullptr || reduced == nullptr ||
+        rows == 0 || input_width == 0 || lora_rank == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT, "invalid LoRA reduce arguments");
+    }
+    nf4o_matmul_nt(x, lora_a, reduced, rows, input_width, lora_rank);
+    return RTHIP_OK;
+}
+
+rthip_status rthip_nf4_lora_linear_forward(
+    const float* x, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, const float* bias_or_null,
+    const float* lora_a, const float* lora_b, uint64_t lora_rank,
+    float lora_scale, float* reduced, float* y, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream) {
+    if (lora_b == nullptr || reduced == nullptr || lora_rank == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT, "invalid LoRA arguments");
+    }
+    if (const rthip_status status = rthip_nf4_linear_forward(
+            x, codes, primary_scales, secondary_scales, encoding,
+            second_level_block, offset, bias_or_null, y, rows, input_width,
+            output_width, block_size, stream);
+        status != RTHIP_OK) {
+        return status;
+    }
+    if (lora_a != nullptr) {
+        nf4o_matmul_nt(x, lora_a, reduced, rows, input_width, lora_rank);
+    }
+    std::vector<float> expanded(rows * output_width);
+    nf4o_matmul_nt(reduced, lora_b, expanded.data(), rows, lora_rank,
+                   output_width);
+    for (size_t index = 0; index < expanded.size(); ++index) {
+        y[index] = y[index] + expanded[index] * lora_scale;
+    }
+    return RTHIP_OK;
+}
+
+rthip_status rthip_nf4_lora_linear_forward_with(
+    int32_t, const float* x, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, const float* bias_or_null,
+    const float* lora_a, const float* lora_b, uint64_t lora_rank,
+    float lora_scale, float* reduced, float* y, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream) {
+    return rthip_nf4_lora_linear_forward(
+        x, codes, primary_scales, secondary_scales, encoding,
+        second_level_block, offset, bias_or_null, lora_a, lora_b, lora_rank,
+        lora_scale, reduced, y, rows, input_width, output_width, block_size,
+        stream);
 }
 
 }  // extern "C"

@@ -104,6 +104,18 @@ def test_lora_arguments_are_checked_before_any_device_work(package, library):
         library.lora_reduce(0x3000, 0x5000, 0x7000, 1, 64, 0)
 
 
+def test_matmul_arguments_are_checked_before_any_device_work(package,
+                                                              library):
+    with pytest.raises(package.InvalidArgument):
+        library.matmul(0, 0x2000, 0x3000, 1, 2, 3, 4)
+    with pytest.raises(package.InvalidArgument):
+        library.matmul(0x1000, 0x2000, 0x3000, 1, 0, 3, 4)
+    with pytest.raises(package.InvalidArgument):
+        library.matmul(0x1000, 0x2000, 0x1000, 1, 2, 3, 4)
+    with pytest.raises(package.InvalidArgument):
+        library.matmul(0x1000, 0x2000, 0x3000, 1, 2 ** 40, 2 ** 40, 4)
+
+
 class _Fake:
     """Stands in for a tensor: only its address is ever passed on."""
 

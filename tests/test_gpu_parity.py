@@ -458,6 +458,47 @@ def test_lora_with_zero_b_equals_the_plain_forward(gpu, package, library,
         helpers.assert_bit_equal(host(fused), plain)
 
 
+# ---- dense fp32 matmul ----------------------------------------------------
+
+@pytest.mark.parametrize("batch,rows,shared,columns", [
+    (1, 2, 3, 2),           # tests/core: tiny, plain kernel
+    (1, 5, 33, 7),          # nothing aligned: plain kernel
+    (3, 40, 64, 48),        # batched
+    (1, 300, 16, 4096),     # adapter second product: K = rank
+    (1, 70, 4096, 16),      # adapter first product: N = rank
+    (1, 16, 300, 1000),     # gradient shape: rows = rank
+    (2, 129, 100, 132),     # every edge of the tile
+    (1, 512, 2048, 1024),
+])
+def test_dense_matmul(gpu, package, library, oracle, batch, rows, shared,
+                      columns):
+    """rthip_matmul against the oracle's restatement of the reference loop and
+    against fp64; tolerance 1e-5 of an output's standard deviation (plus the
+    oracle's own distance from fp64 for the comparison with the oracle)."""
+    left = helpers.normal(130, (batch, rows, shared), 1.0)
+    right = helpers.normal(131, (batch, shared, columns), 0.05)
+    got = host(gpu.matmul(to_device(left), to_device(right)))
+    assert got.shape == (batch, rows, columns)
+    for index in range(batch):
+        exact = left[index].astype(np.float64) @ \
+            right[index].astype(np.float64)
+        unit = helpers.rms(exact)
+        error = np.abs(got[index] - exact).max() / unit
+        assert error <= TOLERANCE, f"matmul vs fp64: {error:.3g}"
+        sample = slice(0, min(rows, 8))
+        cpu = oracle.matmul(left[index][sample], right[index])
+        cpu_error = np.abs(cpu - exact[sample]).max() / unit
+        drift = np.abs(got[index][sample] - cpu).max() / unit
+        assert drift <= TOLERANCE + cpu_error, f"matmul vs oracle: {drift:.3g}"
+
+
+def test_dense_matmul_small_integers_are_exact(gpu, package, library):
+    left = np.arange(12, dtype=np.float32).reshape(1, 3, 4) - 5.0
+    right = np.arange(20, dtype=np.float32).reshape(1, 4, 5) - 9.0
+    got = host(gpu.matmul(to_device(left), to_device(right)))
+    assert np.array_equal(got[0], left[0] @ right[0])
+
+
 # ---- the ABI's error behaviour on a live device --------------------------
 
 def test_abi_rejects_bad_arguments(gpu, package, library, oracle):
