@@ -19,6 +19,8 @@ The same JSON line carries
   small_batch   M in {4, 16, 64} on the three distinct shapes (config 3)
   lora          the fused bias + rank-16 adapter forward beside the plain one
   matmul        dense fp32 matmul at layer and adapter shapes
+  quantizer     the device quantizer on one 11008 x 4096 weight (wall clock,
+                the call returns after the work is done)
   cpu_baseline  the reference CPU backend (oracle/_ref, else the C
                 restatement) timed on this host, single thread, on one layer
 
@@ -311,6 +313,28 @@ def bench_matmul(package, device, torch, steps):
     return results
 
 
+def bench_quantizer(package, device, torch):
+    """The device quantizer on one 11008 x 4096 weight (45 M values)."""
+    results = []
+    dense = torch.randn(11008, 4096, device="cuda") * 0.02
+    for double_quantized in (False, True):
+        device.quantize_weight(dense, BLOCK, double_quantized, 256)
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        repeats = 5
+        for _ in range(repeats):
+            device.quantize_weight(dense, BLOCK, double_quantized, 256)
+        torch.cuda.synchronize()
+        seconds = (time.perf_counter() - begin) / repeats
+        results.append({
+            "shape": "11008x4096",
+            "scales": "double_quantized" if double_quantized else "fp32",
+            "ms": seconds * 1e3,
+            "gvalues_per_s": dense.numel() / seconds / 1e9,
+        })
+    return results
+
+
 def cpu_baseline(budget_seconds=12.0):
     """The reference CPU backend (oracle/_ref when built, else the C
     restatement) on this host, single thread: whole Llama-7B layers (7
@@ -422,6 +446,7 @@ def main():
                                   max(3, arguments.steps // 4))
         line["matmul"] = bench_matmul(package, device, torch,
                                       max(3, arguments.steps // 4))
+        line["quantizer"] = bench_quantizer(package, device, torch)
     if not arguments.skip_cpu:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))

@@ -57,7 +57,9 @@ enum {
     /* any other HIP runtime failure: maps to std::runtime_error */
     RTHIP_RUNTIME_ERROR = 4,
     /* a forced algorithm cannot handle the given shape */
-    RTHIP_UNSUPPORTED = 5
+    RTHIP_UNSUPPORTED = 5,
+    /* a value left the fp32 range: maps to std::overflow_error */
+    RTHIP_OVERFLOW = 6
 };
 
 /* Nf4ScaleEncoding, src/core/backend/nn/quantized_linear/storage.hpp:13-16 */
@@ -259,6 +261,30 @@ rthip_status rthip_nf4_dequantize(
     const float* secondary_scales, int32_t encoding,
     uint64_t second_level_block, float offset, float* out,
     uint64_t element_count, uint64_t block_size, void* stream);
+
+/*
+ * The NF4 quantizer on the device: QuantizedWeight::quantize_nf4 /
+ * quantize_nf4_double_quantized, i.e. pack_nf4 and double_quantize_scales
+ * (src/core/quantization/quantized_weight.cpp:176-206, 208-254), bit for bit.
+ *   values              fp32 [element_count], the weight flattened row-major
+ *   codes               uint8 [ceil(element_count / 2)], overwritten
+ * encoding == RTHIP_NF4_SCALE_FLOAT32:
+ *   primary_scales      float [blocks], overwritten; the other outputs unused
+ * encoding == RTHIP_NF4_SCALE_DOUBLE_QUANTIZED_UINT8:
+ *   primary_scales      uint8 [blocks] scale codes
+ *   secondary_scales    float [ceil(blocks / second_level_block)]
+ *   fp32_scale_scratch  float [blocks]: receives the plain block scales
+ *   host_offset         HOST pointer that receives the offset
+ * Unlike the compute entry points this one returns after the work is done:
+ * a non-finite source value is reported as RTHIP_INVALID_ARGUMENT ("NF4 source
+ * values must be finite") and a non-finite scale mean as RTHIP_OVERFLOW, the
+ * two exceptions the reference throws (:189-191, :224-227).
+ */
+rthip_status rthip_nf4_quantize(
+    const float* values, uint64_t element_count, uint64_t block_size,
+    int32_t encoding, uint64_t second_level_block, uint8_t* codes,
+    void* primary_scales, float* secondary_scales, float* fp32_scale_scratch,
+    float* host_offset, void* stream);
 
 #ifdef __cplusplus
 }

@@ -20,6 +20,7 @@ from .binding import (  # noqa: F401
     DeviceWeight,
     InvalidArgument,
     Library,
+    Overflow,
     RthipError,
     Unavailable,
     Unsupported,

@@ -21,6 +21,7 @@ UNAVAILABLE = 2
 OUT_OF_MEMORY = 3
 RUNTIME_ERROR = 4
 UNSUPPORTED = 5
+OVERFLOW = 6
 
 SCALE_FLOAT32 = 0
 SCALE_DOUBLE_QUANTIZED_UINT8 = 1
@@ -58,12 +59,17 @@ class Unsupported(RthipError):
     pass
 
 
+class Overflow(RthipError, OverflowError):
+    pass
+
+
 _ERRORS = {
     INVALID_ARGUMENT: InvalidArgument,
     UNAVAILABLE: Unavailable,
     OUT_OF_MEMORY: RthipError,
     RUNTIME_ERROR: RthipError,
     UNSUPPORTED: Unsupported,
+    OVERFLOW: Overflow,
 }
 
 _u64 = ctypes.c_uint64
@@ -110,6 +116,9 @@ _PROTOTYPES = {
     "rthip_nf4_select_algorithm": (
         _i32, [_i32, _u64, _u64, _u64, _u64, ctypes.POINTER(_i32)]),
     "rthip_nf4_dequantize": (_i32, _WEIGHT + [_ptr, _u64, _u64, _ptr]),
+    "rthip_nf4_quantize": (
+        _i32, [_ptr, _u64, _u64, _i32, _u64, _ptr, _ptr, _ptr, _ptr,
+               ctypes.POINTER(_f32), _ptr]),
 }
 
 EXPORTED_SYMBOLS = tuple(_PROTOTYPES)
@@ -255,6 +264,18 @@ class Library:
         self._check(self._lib.rthip_matmul(
             left_ptr, right_ptr, out_ptr, batch_count, rows, shared, columns,
             stream))
+
+    def quantize(self, values_ptr: int, element_count: int, block_size: int,
+                 encoding: int, second_level_block: int, codes_ptr: int,
+                 primary_ptr: int, secondary_ptr: Optional[int] = None,
+                 scratch_ptr: Optional[int] = None, stream: int = 0) -> float:
+        """rthip_nf4_quantize; returns the offset (0.0 for fp32 scales)."""
+        offset = _f32(0.0)
+        self._check(self._lib.rthip_nf4_quantize(
+            values_ptr, element_count, block_size, encoding,
+            second_level_block, codes_ptr, primary_ptr, secondary_ptr,
+            scratch_ptr, ctypes.byref(offset), stream))
+        return float(offset.value)
 
     def lora_reduce(self, x_ptr: int, lora_a_ptr: int, reduced_ptr: int,
                     rows: int, input_width: int, rank: int,

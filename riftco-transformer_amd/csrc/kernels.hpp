@@ -66,6 +66,25 @@ void launch_dense_matmul(const float* left, const float* right, float* out,
                          std::size_t shared, std::size_t columns,
                          hipStream_t stream);
 
+// nf4_quantize.hip -- the quantizer.  fp32_scales always receives the block
+// scales; scale_codes == nullptr means plain fp32 scales, otherwise the
+// scales are double-quantised into scale_codes / second_level / *offset.
+// status is a device word the kernels OR error bits into (1: non-finite
+// source value, 2: the scale mean is not finite).
+struct QuantizeProblem {
+    const float* values;
+    std::size_t element_count;
+    unsigned block_shift;
+    std::uint8_t* codes;
+    float* fp32_scales;
+    std::uint8_t* scale_codes;
+    float* second_level;
+    unsigned second_level_shift;
+    float* offset;     // device
+    unsigned* status;  // device, zeroed by the caller
+};
+void launch_quantize(const QuantizeProblem& problem, hipStream_t stream);
+
 // nf4_mfma.hip
 bool mfma_forward_supports(const LinearProblem& problem);
 void launch_mfma_forward(const LinearProblem& problem, hipStream_t stream);

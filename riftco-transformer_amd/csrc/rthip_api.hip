@@ -729,4 +729,99 @@ rthip_status rthip_nf4_dequantize(
     return finish_launch("NF4 dequantize launch");
 }
 
+rthip_status rthip_nf4_quantize(
+    const float* values, uint64_t element_count, uint64_t block_size,
+    int32_t encoding, uint64_t second_level_block, uint8_t* codes,
+    void* primary_scales, float* secondary_scales, float* fp32_scale_scratch,
+    float* host_offset, void* stream
+) {
+    if (values == nullptr || codes == nullptr || primary_scales == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "source values, codes and scales must not be null");
+    }
+    if (element_count == 0 ||
+        element_count > std::numeric_limits<uint64_t>::max() / 8) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "element count must be positive (and addressable)");
+    }
+    rthip::QuantizeProblem problem{};
+    if (!block_shift_for(block_size, &problem.block_shift)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "NF4 block size %llu is not one of 32..4096",
+                    static_cast<unsigned long long>(block_size));
+    }
+    problem.values = values;
+    problem.element_count = element_count;
+    problem.codes = codes;
+    if (encoding == RTHIP_NF4_SCALE_FLOAT32) {
+        problem.fp32_scales = static_cast<float*>(primary_scales);
+    } else if (encoding == RTHIP_NF4_SCALE_DOUBLE_QUANTIZED_UINT8) {
+        if (secondary_scales == nullptr || fp32_scale_scratch == nullptr ||
+            host_offset == nullptr) {
+            return fail(RTHIP_INVALID_ARGUMENT,
+                        "double-quantised scales need the second-level "
+                        "buffer, the fp32 scratch and the offset pointer");
+        }
+        if (!block_shift_for(second_level_block,
+                             &problem.second_level_shift)) {
+            return fail(RTHIP_INVALID_ARGUMENT,
+                        "second-level block size %llu is not one of 32..4096",
+                        static_cast<unsigned long long>(second_level_block));
+        }
+        problem.fp32_scales = fp32_scale_scratch;
+        problem.scale_codes = static_cast<uint8_t*>(primary_scales);
+        problem.second_level = secondary_scales;
+    } else {
+        return fail(RTHIP_INVALID_ARGUMENT, "unknown NF4 scale encoding %d",
+                    static_cast<int>(encoding));
+    }
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+    // [0]: status bits, [1]: the offset (a float)
+    unsigned* words = nullptr;
+    if (const hipError_t error =
+            hipMalloc(reinterpret_cast<void**>(&words), 2 * sizeof(unsigned));
+        error != hipSuccess) {
+        return from_hip(error, "quantizer status allocation");
+    }
+    hipError_t error = hipMemsetAsync(words, 0, 2 * sizeof(unsigned),
+                                      hip_stream);
+    unsigned host_words[2] = {0U, 0U};
+    if (error == hipSuccess) {
+        problem.status = words;
+        problem.offset = reinterpret_cast<float*>(words + 1);
+        rthip::launch_quantize(problem, hip_stream);
+        error = hipGetLastError();
+    }
+    if (error == hipSuccess) {
+        error = hipMemcpyAsync(host_words, words, sizeof(host_words),
+                               hipMemcpyDeviceToHost, hip_stream);
+    }
+    if (error == hipSuccess) {
+        error = hipStreamSynchronize(hip_stream);
+    }
+    const hipError_t released = hipFree(words);
+    if (error != hipSuccess) {
+        return from_hip(error, "NF4 quantize");
+    }
+    if (released != hipSuccess) {
+        return from_hip(released, "quantizer status release");
+    }
+    if ((host_words[0] & 1U) != 0U) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "NF4 source values must be finite");
+    }
+    if ((host_words[0] & 2U) != 0U) {
+        return fail(RTHIP_OVERFLOW,
+                    "NF4 scale mean exceeds the FP32 double-quantization "
+                    "range");
+    }
+    if (host_offset != nullptr) {
+        std::memcpy(host_offset, &host_words[1], sizeof(float));
+    }
+    return ok();
+}
+
 }  // extern "C"

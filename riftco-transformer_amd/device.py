@@ -41,6 +41,39 @@ def upload_weight(output_width: int, input_width: int, block_size: int,
                         secondary, second_level_block, float(offset))
 
 
+def quantize_weight(dense: torch.Tensor, block_size: int = 64,
+                    double_quantized: bool = False,
+                    second_level_block: int = 256) -> DeviceWeight:
+    """Quantizes a dense [output_width, input_width] fp32 device tensor with
+    rthip_nf4_quantize; the payload never leaves the device."""
+    assert dense.is_cuda and dense.dtype == torch.float32 and \
+        dense.is_contiguous() and dense.dim() == 2
+    output_width, input_width = dense.shape
+    count = dense.numel()
+    blocks = (count + block_size - 1) // block_size
+    codes = torch.empty((count + 1) // 2, dtype=torch.uint8,
+                        device=dense.device)
+    library = load_library()
+    if not double_quantized:
+        scales = torch.empty(blocks, dtype=torch.float32, device=dense.device)
+        library.quantize(dense.data_ptr(), count, block_size, SCALE_FLOAT32, 0,
+                         codes.data_ptr(), scales.data_ptr(), None, None,
+                         _stream())
+        return DeviceWeight(output_width, input_width, block_size,
+                            SCALE_FLOAT32, codes, scales, None)
+    groups = (blocks + second_level_block - 1) // second_level_block
+    scale_codes = torch.empty(blocks, dtype=torch.uint8, device=dense.device)
+    second = torch.empty(groups, dtype=torch.float32, device=dense.device)
+    scratch = torch.empty(blocks, dtype=torch.float32, device=dense.device)
+    offset = library.quantize(
+        dense.data_ptr(), count, block_size, SCALE_DOUBLE_QUANTIZED_UINT8,
+        second_level_block, codes.data_ptr(), scale_codes.data_ptr(),
+        second.data_ptr(), scratch.data_ptr(), _stream())
+    return DeviceWeight(output_width, input_width, block_size,
+                        SCALE_DOUBLE_QUANTIZED_UINT8, codes, scale_codes,
+                        second, second_level_block, offset)
+
+
 def linear_forward(x: torch.Tensor, weight: DeviceWeight,
                    bias: Optional[torch.Tensor] = None,
                    out: Optional[torch.Tensor] = None,

@@ -338,4 +338,41 @@ rthip_status rthip_nf4_lora_linear_forward_with(
         stream);
 }
 
+rthip_status rthip_nf4_quantize(
+    const float* values, uint64_t element_count, uint64_t block_size,
+    int32_t encoding, uint64_t second_level_block, uint8_t* codes,
+    void* primary_scales, float* secondary_scales, float* fp32_scale_scratch,
+    float* host_offset, void*) {
+    if (values == nullptr || codes == nullptr || primary_scales == nullptr ||
+        element_count == 0 || !supported_block(block_size)) {
+        return fail(RTHIP_INVALID_ARGUMENT, "invalid quantize arguments");
+    }
+    const bool nested = encoding == RTHIP_NF4_SCALE_DOUBLE_QUANTIZED_UINT8;
+    float* scales =
+        nested ? fp32_scale_scratch : static_cast<float*>(primary_scales);
+    if (scales == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT, "missing scale buffer");
+    }
+    if (nf4o_quantize(values, element_count, block_size, codes, scales) !=
+        NF4O_OK) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "NF4 source values must be finite");
+    }
+    if (nested) {
+        if (secondary_scales == nullptr || host_offset == nullptr ||
+            !supported_block(second_level_block)) {
+            return fail(RTHIP_INVALID_ARGUMENT, "invalid nested arguments");
+        }
+        const size_t blocks = (element_count + block_size - 1) / block_size;
+        if (nf4o_double_quantize_scales(
+                scales, blocks, second_level_block,
+                static_cast<uint8_t*>(primary_scales), secondary_scales,
+                host_offset) != NF4O_OK) {
+            return fail(RTHIP_OVERFLOW, "NF4 scale mean exceeds the FP32 "
+                                        "double-quantization range");
+        }
+    }
+    return RTHIP_OK;
+}
+
 }  // extern "C"

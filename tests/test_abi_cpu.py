@@ -116,6 +116,24 @@ def test_matmul_arguments_are_checked_before_any_device_work(package,
         library.matmul(0x1000, 0x2000, 0x3000, 1, 2 ** 40, 2 ** 40, 4)
 
 
+def test_quantize_arguments_are_checked_before_any_device_work(package,
+                                                                library):
+    fp32, nested = package.SCALE_FLOAT32, package.SCALE_DOUBLE_QUANTIZED_UINT8
+    with pytest.raises(package.InvalidArgument):
+        library.quantize(0, 64, 64, fp32, 0, 0x2000, 0x3000)
+    with pytest.raises(package.InvalidArgument):
+        library.quantize(0x1000, 0, 64, fp32, 0, 0x2000, 0x3000)
+    with pytest.raises(package.InvalidArgument):
+        library.quantize(0x1000, 64, 48, fp32, 0, 0x2000, 0x3000)
+    with pytest.raises(package.InvalidArgument):  # no second-level buffer
+        library.quantize(0x1000, 64, 64, nested, 32, 0x2000, 0x3000)
+    with pytest.raises(package.InvalidArgument):  # bad second-level block
+        library.quantize(0x1000, 64, 64, nested, 40, 0x2000, 0x3000, 0x4000,
+                         0x5000)
+    with pytest.raises(package.InvalidArgument):
+        library.quantize(0x1000, 64, 64, 7, 0, 0x2000, 0x3000)
+
+
 class _Fake:
     """Stands in for a tensor: only its address is ever passed on."""
 

@@ -499,6 +499,94 @@ def test_dense_matmul_small_integers_are_exact(gpu, package, library):
     assert np.array_equal(got[0], left[0] @ right[0])
 
 
+# ---- the quantizer on the device ------------------------------------------
+
+def payload_of(device_weight):
+    import torch
+    torch.cuda.synchronize()
+    return (device_weight.codes.cpu().numpy(),
+            device_weight.primary_scales.cpu().numpy(),
+            None if device_weight.secondary_scales is None
+            else device_weight.secondary_scales.cpu().numpy(),
+            np.float32(device_weight.offset))
+
+
+@pytest.mark.parametrize("shape,block,second", [
+    ((768, 256), 64, 256), ((33, 33), 32, 32), ((17, 96), 32, 64),
+    ((5, 4096), 4096, 32), ((64, 1000), 128, 32), ((1, 1), 32, 32),
+    ((4096, 4096), 64, 256), ((1000, 11008), 64, 256)])
+@pytest.mark.parametrize("double_quantized", [False, True])
+@pytest.mark.parametrize("sigma", [0.02, 1.0])
+def test_device_quantizer_is_bit_exact(gpu, package, library, oracle, shape,
+                                       block, second, double_quantized,
+                                       sigma):
+    """Codes, block scales, scale codes, second-level scales and the offset
+    must equal the oracle's (which is pinned to the compiled reference)."""
+    dense = helpers.normal(140, shape, sigma)
+    dense.ravel()[::7] = 0.0   # exact zeros: ties at code 7
+    if dense.shape[0] > 8:
+        dense[3] = 0.0         # a whole zero block or more
+    want = oracle.quantize(dense, block, double_quantized, second)
+    got = gpu.quantize_weight(to_device(dense), block, double_quantized,
+                              second)
+    codes, primary, secondary, offset = payload_of(got)
+    assert np.array_equal(codes, want.codes)
+    if not double_quantized:
+        helpers.assert_bit_equal(primary, want.fp32_scales)
+    else:
+        assert np.array_equal(primary, want.scale_codes)
+        helpers.assert_bit_equal(secondary, want.second_level)
+        helpers.assert_bit_equal(offset, np.float32(want.offset))
+
+
+def test_device_quantizer_scale_mean_with_a_wide_exponent_range(
+        gpu, package, library, oracle):
+    """Scales that span 2^40: the double sum is then order-dependent and the
+    device must add in index order like the reference."""
+    rng = np.random.default_rng(141)
+    blocks = 5000
+    magnitudes = (2.0 ** rng.integers(-30, 10, blocks)) * \
+        (1.0 + rng.random(blocks))
+    dense = np.zeros((blocks, 32), dtype=np.float32)
+    dense[:, 0] = magnitudes.astype(np.float32)
+    dense[:, 1:] = (dense[:, :1] *
+                    rng.uniform(-1, 1, (blocks, 31))).astype(np.float32)
+    want = oracle.quantize(dense, 32, True, 64)
+    got = gpu.quantize_weight(to_device(dense), 32, True, 64)
+    codes, primary, secondary, offset = payload_of(got)
+    assert np.array_equal(codes, want.codes)
+    assert np.array_equal(primary, want.scale_codes)
+    helpers.assert_bit_equal(secondary, want.second_level)
+    helpers.assert_bit_equal(offset, np.float32(want.offset))
+
+
+def test_device_quantizer_rejects_non_finite_values(gpu, package, library):
+    dense = helpers.normal(142, (64, 64), 0.02)
+    dense[10, 3] = np.inf
+    with pytest.raises(package.InvalidArgument) as error:
+        gpu.quantize_weight(to_device(dense), 64)
+    assert "finite" in error.value.message
+    dense[10, 3] = np.nan
+    with pytest.raises(package.InvalidArgument):
+        gpu.quantize_weight(to_device(dense), 64, True, 32)
+
+
+def test_quantize_then_multiply_on_the_device(gpu, package, library, oracle):
+    """The device quantizer feeds the kernels directly."""
+    dense = helpers.normal(143, (512, 1024), 0.02)
+    weight = gpu.quantize_weight(to_device(dense), 64, True, 256)
+    host_weight = oracle.quantize(dense, 64, True, 256)
+    helpers.assert_bit_equal(host(gpu.dequantize(weight)),
+                             oracle.dequantize(host_weight))
+    x = helpers.normal(144, (3, 1024), 1.0)
+    y = host(gpu.linear_forward(to_device(x), weight))
+    exact = helpers.exact_forward(x, oracle.dequantize(host_weight))
+    error = helpers.normalized_error(
+        y, exact, 1024, helpers.rms(x),
+        helpers.rms(oracle.dequantize(host_weight)))
+    assert error <= TOLERANCE
+
+
 # ---- the ABI's error behaviour on a live device --------------------------
 
 def test_abi_rejects_bad_arguments(gpu, package, library, oracle):
