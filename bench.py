@@ -380,6 +380,9 @@ def main():
     parser.add_argument("--skip-extras", action="store_true",
                         help="only the headline decode workload")
     parser.add_argument("--skip-cpu", action="store_true")
+    parser.add_argument("--gemm-only", action="store_true",
+                        help="run only the M = 2048 GEMM section (for "
+                             "rocprofv3 counter runs)")
     parser.add_argument("--traffic-calibration", action="store_true",
                         help="for rocprofv3 --pmc runs: a 1 GiB elementwise "
                              "copy of known traffic, then one decode step "
@@ -411,6 +414,12 @@ def main():
         print(json.dumps({"traffic_calibration": "done",
                           "copy_bytes_read": 2 ** 30,
                           "copy_bytes_written": 2 ** 30}))
+        return
+
+    if arguments.gemm_only:
+        # For counter runs: nothing but the M = 2048 launches.
+        print(json.dumps({"gemm": bench_gemm(package, device, torch,
+                                             arguments.steps)}))
         return
 
     decode = bench_decode(package, device, torch, arguments.layers,
