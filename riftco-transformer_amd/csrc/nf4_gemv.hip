@@ -19,30 +19,29 @@
 // wavefronts never wait for each other inside the loop, so HBM requests are in
 // flight for the whole life of the workgroup.
 //
-// Decode.  Nibble -> fp32 is a table lookup, and the LDS (128 B per clock per
-// CU) is the unit that bounds this kernel once the loads stream: 4 bytes of
-// table per weight.  Nibbles are therefore decoded two at a time -- a code BYTE
-// indexes a table of (codebook[low nibble], codebook[high nibble]) pairs, one
-// ds_read_b64 per two weights -- and everything else is kept off the LDS.
-// The table is stored entry-major with 16 interleaved replicas: replica k of
-// entry e sits at byte e * 256 + k * 8, and lane l reads replica l % 16.  The 16
-// lanes the LDS serves per clock therefore always touch 16 different bank pairs
-// whatever their codes are, and an entry's address is
-// (byte << 8) | ((l % 16) << 3): ONE v_perm_b32 that drops the code byte into
-// bits 8..15 above the lane's fixed low byte.  The table is built from
-// instruction literals while the first loads are in flight.
+// Decode.  Nibble -> fp32 is a table lookup in LDS, 4 bytes of table per
+// weight.  Nibbles are decoded two at a time -- a code BYTE indexes a table of
+// (codebook[low nibble], codebook[high nibble]) pairs, one ds_read_b64 per two
+// weights -- and everything else is kept off the LDS.  The table is stored
+// entry-major with 32 interleaved replicas (nf4_pair_table.hpp): replica k of
+// entry e sits at byte e * 256 + k * 8, lane l reads replica l % 32, so a
+// lookup never meets a bank conflict whatever the codes are, and an entry's
+// address is (byte << 8) | ((l % 32) << 3): ONE v_perm_b32 that drops the code
+// byte into bits 8..15 above the lane's fixed low byte.  The table is built
+// from instruction literals while the first loads are in flight.
 //
-// Weight bytes and scales are fetched with buffer loads: the address is a
-// per-lane constant offset plus a per-row SCALAR offset, so stepping to the next
-// row costs no vector arithmetic, and the hardware range check turns reads past
-// the end of the payload into zeros.  Nothing branches on data or on bounds:
+// Weight bytes and scales are fetched with buffer loads through per-row
+// descriptors (built with scalar instructions): the per-lane offset is a
+// constant, so stepping to the next row costs no vector arithmetic, and the
+// hardware range check turns reads past the row end into zeros.  Nothing branches on data or on bounds:
 // segments past the row end carry x = 0 and rows past the output width are
 // computed on whatever was read and never written.
 //
 // Reduction.  Row sums are reduced inside each 16-lane DPP row with a transposed
-// butterfly of DPP moves (vector ALU only, no LDS round trips); the 16 row
-// partials per team and batch are parked in LDS, and after ONE barrier at the
-// end of the kernel the team adds them up and writes y.
+// butterfly of DPP moves (vector ALU only), then across the four rows of the
+// wavefront; the four wavefront partials per team and batch are parked in LDS,
+// and after ONE barrier at the end of the kernel the team adds them up and
+// writes y.
 
 #include "kernels.hpp"
 #include "nf4_decode.hpp"
@@ -55,9 +54,9 @@ constexpr int kWave = 64;
 constexpr int kTeamThreads = 256;  // threads that share one weight row
 constexpr int kSegment = 16;       // weights per thread per row visit
 constexpr int kRowLanes = 16;      // lanes of one DPP row
-constexpr int kTeamDppRows = kTeamThreads / kRowLanes;
+constexpr int kTeamWaves = kTeamThreads / kWave;
 constexpr unsigned kComputeUnits = 256;
-// Row totals a team may park in LDS before the final barrier, per DPP row.
+// Row totals a team may park in LDS before the final barrier, per wavefront.
 constexpr unsigned kParkedValues = 128;
 #ifndef RTHIP_GEMV_TEAMS
 #define RTHIP_GEMV_TEAMS 2
@@ -174,7 +173,7 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
     constexpr int kValues = kRows * kX;
     constexpr unsigned kMaxIterations = kParkedValues / kValues;
     __shared__ __attribute__((aligned(256))) char table[kPairTableBytes];
-    __shared__ float partial[kTeams][kMaxIterations][kTeamDppRows][kValues];
+    __shared__ float partial[kTeams][kMaxIterations][kTeamWaves][kValues];
 
     const unsigned team =
         __builtin_amdgcn_readfirstlane(threadIdx.x / kTeamThreads);
@@ -266,8 +265,11 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
     }
 
     // This thread's slice of x, resident for the whole kernel.  Segments past
-    // the row end and rows past x_rows read as zero.
+    // the row end and rows past x_rows read as zero.  The loads are issued
+    // here and consumed only after the table is built, so that their latency
+    // and the build overlap.
     float xs[kX][kSegments][kSegment];
+    bool x_valid[kX][kSegments];
 #pragma unroll
     for (int j = 0; j < kSegments; ++j) {
         const bool segment_valid = thread + kTeamThreads * j < segment_count;
@@ -275,7 +277,7 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
             min(thread + kTeamThreads * j, segment_count - 1) * kSegment;
 #pragma unroll
         for (int r = 0; r < kX; ++r) {
-            const bool valid =
+            x_valid[r][j] =
                 segment_valid && static_cast<unsigned>(r) < x_rows;
             const unsigned source_row =
                 min(static_cast<unsigned>(r), x_rows - 1);
@@ -284,16 +286,27 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
 #pragma unroll
             for (int q = 0; q < kSegment / 4; ++q) {
                 const float4 v = source[q];
-                xs[r][j][4 * q + 0] = valid ? v.x : 0.0F;
-                xs[r][j][4 * q + 1] = valid ? v.y : 0.0F;
-                xs[r][j][4 * q + 2] = valid ? v.z : 0.0F;
-                xs[r][j][4 * q + 3] = valid ? v.w : 0.0F;
+                xs[r][j][4 * q + 0] = v.x;
+                xs[r][j][4 * q + 1] = v.y;
+                xs[r][j][4 * q + 2] = v.z;
+                xs[r][j][4 * q + 3] = v.w;
             }
         }
     }
 
     build_pair_table<kThreads>(table);
     __syncthreads();
+
+#pragma unroll
+    for (int j = 0; j < kSegments; ++j) {
+#pragma unroll
+        for (int r = 0; r < kX; ++r) {
+#pragma unroll
+            for (int i = 0; i < kSegment; ++i) {
+                xs[r][j][i] = x_valid[r][j] ? xs[r][j][i] : 0.0F;
+            }
+        }
+    }
 
     const unsigned lane_bits = pair_table_lane_bits(lane);
 
@@ -371,11 +384,14 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
             __builtin_amdgcn_sched_barrier(0);
         }
 
-        // Park this DPP row's totals; nobody waits here.
-        const float total = transposed_row_sum<kValues>(acc, lane);
-        if (lane % kRowLanes < kValues) {
-            partial[team][iteration][thread / kRowLanes]
-                   [slot_of_lane<kValues>(lane % kRowLanes)] = total;
+        // Totals of each 16-lane DPP row, then of the wavefront's four rows;
+        // the wavefront parks them and nobody waits here.
+        float total = transposed_row_sum<kValues>(acc, lane);
+        total += __shfl_xor(total, 16, kWave);
+        total += __shfl_xor(total, 32, kWave);
+        if (lane < kValues) {
+            partial[team][iteration][thread / kWave]
+                   [slot_of_lane<kValues>(lane)] = total;
         }
     };
 
@@ -391,8 +407,8 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
     }
 
     // The only barrier after the table build: every batch of this workgroup
-    // has been parked.  Each team adds up its 16 row partials per value and
-    // writes y.
+    // has been parked.  Each team adds up its four wavefront partials per
+    // value and writes y.
     __syncthreads();
     for (unsigned index = thread; index < iterations * kValues;
          index += kTeamThreads) {
@@ -404,8 +420,8 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
         if (batch_index < batch_count && o < output_width && r < x_rows) {
             float sum = 0.0F;
 #pragma unroll
-            for (int row = 0; row < kTeamDppRows; ++row) {
-                sum += partial[team][iteration][row][value];
+            for (int wave = 0; wave < kTeamWaves; ++wave) {
+                sum += partial[team][iteration][wave][value];
             }
             if (bias != nullptr) {
                 sum += bias[o];

@@ -2,10 +2,12 @@
 // GEMV and the small-batch kernel use to turn one code BYTE into two fp32
 // codebook levels with one ds_read_b64.
 //
-// Layout: entry-major with 16 interleaved replicas; replica k of entry e sits
-// at byte e * 256 + k * 8 and lane l reads replica l % 16.  The 16 lanes the
-// LDS serves per clock therefore always touch 16 different bank pairs whatever
-// their codes are, and an entry's address is (byte << 8) | ((l % 16) << 3): ONE
+// Layout: entry-major with 32 interleaved replicas; replica k of entry e sits
+// at byte e * 256 + k * 8 and lane l reads replica l % 32.  An entry's 256
+// bytes span all 64 LDS banks of the CU, so the 32 lanes served per clock
+// always touch 32 different bank pairs whatever their codes are (16 replicas
+// in 128 bytes measured 2 conflict cycles per 64-lane read), and an entry's
+// address is (byte << 8) | ((l % 32) << 3): ONE
 // v_perm_b32 that drops the code byte into bits 8..15 above the lane's fixed
 // low byte.  Levels are the literals of src/core/quantization/nf4.cpp:14-31
 // (under /root/reference), built from instruction immediates so that the build
@@ -16,7 +18,7 @@
 
 namespace rthip {
 
-constexpr int kReplicas = 16;      // interleaved copies of the pair table
+constexpr int kReplicas = 32;      // interleaved copies of the pair table
 constexpr int kEntryStride = 256;  // bytes between table entries
 constexpr int kPairTableBytes = 256 * kEntryStride;
 
@@ -56,38 +58,44 @@ __device__ __forceinline__ float level_in_quarter(unsigned quarter) {
 }
 
 // Builds the replicated pair table with all kThreads threads of the
-// workgroup.  A thread fills one replica of 4096 / kThreads consecutive
-// entries, in groups of four that share a high nibble and a low-nibble
-// quarter.
+// workgroup.  A thread fills two neighbouring replicas (one 16-byte store) of
+// 2048 / kThreads consecutive entries, in groups of four that share a high
+// nibble and a low-nibble quarter.  Eight consecutive lanes write the 128
+// bytes of one entry, which is what the LDS takes per clock.
 template <int kThreads>
 __device__ __forceinline__ void build_pair_table(char* table) {
-    constexpr int kEntries = 256 * kReplicas / kThreads;  // per thread
+    // at most 512 threads build (four entries each); the others skip
+    constexpr int kBuilders = kThreads > 512 ? 512 : kThreads;
+    constexpr int kEntries = 256 * (kReplicas / 2) / kBuilders;  // per thread
     static_assert(kEntries >= 4 && kEntries % 4 == 0);
-    const unsigned replica = threadIdx.x % kReplicas;
-    const unsigned first_entry = (threadIdx.x / kReplicas) * kEntries;
-    char* slot = table + replica * sizeof(float2);
+    if (kBuilders < kThreads && threadIdx.x >= kBuilders) {
+        return;
+    }
+    const unsigned replica_pair = threadIdx.x % (kReplicas / 2);
+    const unsigned first_entry = (threadIdx.x / (kReplicas / 2)) * kEntries;
+    char* slot = table + replica_pair * sizeof(float4);
 #pragma unroll
     for (int group = 0; group < kEntries / 4; ++group) {
         const unsigned entry = first_entry + 4 * group;
         const float high_level = codebook_literal(entry >> 4);
         const unsigned quarter = (entry >> 2) & 3U;
-        float2* target =
-            reinterpret_cast<float2*>(slot + entry * kEntryStride);
-        constexpr int kStep = kEntryStride / sizeof(float2);
-        target[0 * kStep] =
-            make_float2(level_in_quarter<0>(quarter), high_level);
-        target[1 * kStep] =
-            make_float2(level_in_quarter<1>(quarter), high_level);
-        target[2 * kStep] =
-            make_float2(level_in_quarter<2>(quarter), high_level);
-        target[3 * kStep] =
-            make_float2(level_in_quarter<3>(quarter), high_level);
+        float4* target =
+            reinterpret_cast<float4*>(slot + entry * kEntryStride);
+        constexpr int kStep = kEntryStride / sizeof(float4);
+        const float low0 = level_in_quarter<0>(quarter);
+        const float low1 = level_in_quarter<1>(quarter);
+        const float low2 = level_in_quarter<2>(quarter);
+        const float low3 = level_in_quarter<3>(quarter);
+        target[0 * kStep] = make_float4(low0, high_level, low0, high_level);
+        target[1 * kStep] = make_float4(low1, high_level, low1, high_level);
+        target[2 * kStep] = make_float4(low2, high_level, low2, high_level);
+        target[3 * kStep] = make_float4(low3, high_level, low3, high_level);
     }
 }
 
 // The lane's fixed low address byte.
 __device__ __forceinline__ unsigned pair_table_lane_bits(unsigned lane) {
-    return (lane % kReplicas) * sizeof(float2);  // < 128
+    return (lane % kReplicas) * sizeof(float2);  // < 256
 }
 
 // (level[low nibble], level[high nibble]) of byte `byte` (0..3) of `word`.

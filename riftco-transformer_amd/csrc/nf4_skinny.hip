@@ -318,22 +318,44 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
     // consecutive values at 64 * quarter.
     const float* fragment = x_tile + (lane % 16) * kStride + quarter * kChunk;
 
-    // The inner loop is software-pipelined by hand so that no LDS latency is
-    // exposed to the matrix pipe: the table lookups of sub-chunk c + 1 and the
-    // x fragment of the next (sub-chunk, block) stage are issued BEFORE the
-    // matrix instructions of the current stage, and the lookups of a round's
-    // first sub-chunk are issued at the end of the previous round.
-    float2 raw[8];  // levels of the sub-chunk being looked up
-    const auto issue_lookups = [&](const Codes& codes, int c) {
+    // The inner loop is software-pipelined by hand.  A stage is the 16 matrix
+    // instructions of one (sub-chunk of 16 contraction values, block of x)
+    // pair; they form a dependent chain, so the wavefront has eight issue
+    // slots free behind each of them.  Everything else is placed in those
+    // slots, two sub-chunks ahead of its use:
+    //   stage (c, 0): table lookups of sub-chunk c + 2, the multiplies that
+    //                 turn the levels of sub-chunk c + 1 into weights,
+    //   every stage:  the x fragment of the next stage,
+    // with sched_group_barrier spelling out the interleaving.  Sub-chunks
+    // count on across rounds (c + 1 == 4 is the next round's first), so the
+    // only exposed LDS latency is the first x fragment after the barrier.
+    // Levels looked up.  With one block of x the lookups of sub-chunk c + 2
+    // are issued in the stage that consumes those of c + 1, so there are two
+    // buffers (by parity); with more blocks the two fall into different
+    // stages and one buffer is enough.
+    constexpr int kRawBuffers = kBlocks == 1 ? 2 : 1;
+    float2 raw[kRawBuffers][8];
+    float w[2][16];    // weights, by sub-chunk parity
+    const auto issue_lookups = [&](float2 (&out)[8], const Codes& codes,
+                                   int c) {
         const unsigned words[2] = {codes.codes[c / 2][2 * (c % 2)],
                                    codes.codes[c / 2][2 * (c % 2) + 1]};
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
 #pragma unroll
             for (int byte = 0; byte < 4; ++byte) {
-                raw[4 * half + byte] =
+                out[4 * half + byte] =
                     pair_table_lookup(table, words[half], byte, lane_bits);
             }
+        }
+    };
+    const auto scale_levels = [&](float (&out)[16], const float2 (&levels)[8],
+                                  float scale) {
+#pragma clang fp contract(off)
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            out[2 * p] = levels[p].x * scale;
+            out[2 * p + 1] = levels[p].y * scale;
         }
     };
     const auto issue_fragment = [&](floatx4 (&a)[4], int c, int b) {
@@ -345,7 +367,9 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
     };
 
     __syncthreads();  // the table is built
-    issue_lookups(ring[0], 0);
+    issue_lookups(raw[0], ring[0], 0);
+    scale_levels(w[0], raw[0], ring[0].scales[0]);
+    issue_lookups(raw[1 % kRawBuffers], ring[0], 1);
 
     for (unsigned step = 0; step < unit_count; ++step) {
         __syncthreads();  // the previous round's fragment reads are done
@@ -361,45 +385,58 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
         }
         load_codes(ring[kDepth - 1], code_cursor);
         advance(code_cursor);
+        // `current` is this round, ring[0] the next one.
 
         floatx4 a[2][4];
         issue_fragment(a[0], 0, 0);
-        // Four sub-chunks of 16 contraction values, kBlocks stages each.
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            float w[16];
-            {
-#pragma clang fp contract(off)
-                const float scale = current.scales[c * kScales / 4];
-#pragma unroll
-                for (int p = 0; p < 8; ++p) {
-                    w[2 * p] = raw[p].x * scale;
-                    w[2 * p + 1] = raw[p].y * scale;
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if (c + 1 < 4) {
-                issue_lookups(current, c + 1);
-            } else {
-                issue_lookups(ring[0], 0);  // the next round's first
-            }
 #pragma unroll
             for (int b = 0; b < kBlocks; ++b) {
                 constexpr int kStages = 4 * kBlocks;
                 const int stage = c * kBlocks + b;
+                __builtin_amdgcn_sched_barrier(0);
                 if (stage + 1 < kStages) {
                     issue_fragment(a[(stage + 1) % 2], (stage + 1) / kBlocks,
                                    (stage + 1) % kBlocks);
                 }
-                __builtin_amdgcn_sched_barrier(0);
+                if (b == 0) {
+                    // weights of sub-chunk c + 1 from the levels fetched
+                    // during sub-chunk c - 1 ...
+                    if (c + 1 < 4) {
+                        scale_levels(
+                            w[(c + 1) % 2], raw[(c + 1) % kRawBuffers],
+                            current.scales[(c + 1) * kScales / 4]);
+                    } else {
+                        scale_levels(w[0], raw[0], ring[0].scales[0]);
+                    }
+                }
+                if (b == kBlocks - 1) {
+                    // ... and, once those levels are consumed, the lookups
+                    // of sub-chunk c + 2 into the same registers' partner.
+                    if (c + 2 < 4) {
+                        issue_lookups(raw[c % kRawBuffers], current, c + 2);
+                    } else {
+                        issue_lookups(raw[c % kRawBuffers], ring[0],
+                                      c + 2 - 4);
+                    }
+                }
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                            a[stage % 2][v][e], w[4 * v + e], acc[b], 0, 0,
-                            0);
+                            a[stage % 2][v][e], w[c % 2][4 * v + e], acc[b],
+                            0, 0, 0);
                     }
+                }
+                // One matrix instruction, then up to two vector-ALU
+                // instructions and one LDS read in its shadow, sixteen times.
+#pragma unroll
+                for (int slot = 0; slot < 16; ++slot) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
