@@ -41,7 +41,7 @@ extern "C" {
 #endif
 
 #define RTHIP_ABI_VERSION_MAJOR 1u
-#define RTHIP_ABI_VERSION_MINOR 0u
+#define RTHIP_ABI_VERSION_MINOR 1u
 
 typedef int32_t rthip_status;
 
