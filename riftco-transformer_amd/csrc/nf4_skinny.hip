@@ -15,27 +15,27 @@
 //     rows].  Lane l feeds x row l % 16, weight row l % 16 and the k-quarter
 //     l / 16.
 //   * A workgroup of eight wavefronts owns a tile of 128 weight rows, 16 per
-//     wavefront, and all eight walk the contraction axis together in rounds
-//     of 256.  The x tile of a round ([rows][256] floats) is copied to LDS
+//     wavefront, and all eight walk the contraction axis together in slabs
+//     of 256.  The x tile of a slab ([rows][256] floats) is copied to LDS
 //     once and read by all eight wavefronts, which divides the L2 traffic for
 //     x by eight compared with one 16-row tile per workgroup.
-//   * In a round a lane owns 64 consecutive weights of its row (two 16-byte
+//   * In a slab a lane owns 64 consecutive weights of its row (two 16-byte
 //     loads; a wavefront reads 128 contiguous bytes of each of its 16 rows)
 //     and, per 16-row block of x, the 64 matching x values from LDS.  MFMA j
-//     of the round contracts k = 64 q + j over the four quarters q -- any
+//     of the slab contracts k = 64 q + j over the four quarters q -- any
 //     assignment of k to lanes is valid as long as A and B agree.
 //   * Decode: code byte -> two levels through the replicated pair table (one
 //     v_perm_b32 + one ds_read_b64 per two weights), times the block scale in
 //     one rounded multiply each.
-//   * Work split ("stream-K"): the (tile, round) pairs, tile-major, are dealt
+//   * Work split ("stream-K"): the (tile, slab) pairs, tile-major, are dealt
 //     in equal contiguous runs to one workgroup per compute unit, so that every
 //     unit carries the same load whatever the shape.  A workgroup that covers a
 //     whole tile writes y directly.  Otherwise it writes a partial tile to a
 //     workspace slot and a second small kernel adds the partial tiles of each
 //     output tile in ascending workgroup order (plus bias), so results do not
 //     depend on scheduling.
-//   * The code bytes of the next two rounds and the x tile of the next round
-//     are in flight while the current round computes.  Every load is a raw
+//   * The code bytes of the next two slabs and the x tile of the next slab
+//     are in flight while the current slab computes.  Every load is a raw
 //     buffer load whose range check (on the per-lane offset) returns zeros for
 //     lanes with nothing to read, so nothing in the loop is predicated.
 
@@ -55,19 +55,19 @@ typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 constexpr int kThreads = 512;
 constexpr int kWaves = 8;
 constexpr int kTileN = 16 * kWaves;  // weight rows per workgroup
-constexpr int kRound = 256;          // contraction values per round
-constexpr int kChunk = kRound / 4;   // weights per lane per round
-constexpr int kStride = kRound + 4;  // padded x row stride in LDS (floats)
-constexpr int kDepth = 2;            // rounds the code bytes run ahead
+constexpr int kSlab = 256;          // contraction values per slab
+constexpr int kChunk = kSlab / 4;   // weights per lane per slab
+constexpr int kStride = kSlab + 4;  // padded x row stride in LDS (floats)
+constexpr int kDepth = 2;            // slabs the code bytes run ahead
 constexpr unsigned kComputeUnits = 256;
 constexpr unsigned kSlotsPerGroup = 2;  // partial tiles one workgroup may write
 // Offset that the range checks always reject (every buffer is smaller).
 constexpr unsigned kRejectedOffset = 0x80000000U;
 
-// How the (tile, round) units are dealt to the workgroups: the first
+// How the (tile, slab) units are dealt to the workgroups: the first
 // `remainder` workgroups take quotient + 1 units, the others quotient.
 struct UnitSplit {
-    unsigned rounds;  // rounds per tile
+    unsigned slabs;  // slabs per tile
     unsigned quotient;
     unsigned remainder;
 
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
 ) {
     constexpr int kRows = 16 * kBlocks;
     // float4 copies per thread to move one x tile
-    constexpr int kCopies = kRows * (kRound / 4) / kThreads;  // 2 * kBlocks
+    constexpr int kCopies = kRows * (kSlab / 4) / kThreads;  // 2 * kBlocks
     extern __shared__ __attribute__((aligned(256))) char shared[];
     char* table = shared;  // kPairTableBytes
     float* x_tile = reinterpret_cast<float*>(shared + kPairTableBytes);
@@ -128,46 +128,46 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
             ? (((block_total - 1) >> weight.second_level_shift) + 1) * 4
             : 0);
 
-    // A position on the unit axis, advanced one round at a time with scalar
+    // A position on the unit axis, advanced one slab at a time with scalar
     // arithmetic only.  Positions past the workgroup's run have left == 0 and
     // make every load return zeros.
     struct Cursor {
         unsigned tile;
-        unsigned round;
+        unsigned slab;
         unsigned left;  // units of the run not yet passed, this one included
     };
     const auto advance = [&](Cursor& c) {
-        c.round += 1;
-        if (c.round == split.rounds) {
-            c.round = 0;
+        c.slab += 1;
+        if (c.slab == split.slabs) {
+            c.slab = 0;
             c.tile += 1;
         }
         c.left = c.left > 0 ? c.left - 1 : 0;
     };
     Cursor compute_cursor;
-    compute_cursor.tile = unit_begin / split.rounds;
-    compute_cursor.round = unit_begin - compute_cursor.tile * split.rounds;
+    compute_cursor.tile = unit_begin / split.slabs;
+    compute_cursor.slab = unit_begin - compute_cursor.tile * split.slabs;
     compute_cursor.left = unit_count;
     Cursor x_cursor = compute_cursor;
     Cursor code_cursor = compute_cursor;
 
     // -- x tile: global -> registers -> LDS -----------------------------------
     // Thread t moves float4 (t + 512 i) of the [kRows][64 float4] tile.
-    unsigned x_source[kCopies];  // byte offset inside x for round 0
+    unsigned x_source[kCopies];  // byte offset inside x for slab 0
 #pragma unroll
     for (int i = 0; i < kCopies; ++i) {
         const unsigned index = thread + kThreads * i;
-        const unsigned row = index / (kRound / 4);
-        const unsigned column = (index % (kRound / 4)) * 4;
+        const unsigned row = index / (kSlab / 4);
+        const unsigned column = (index % (kSlab / 4)) * 4;
         x_source[i] = row < rows ? (row * input_width + column) *
                                        static_cast<unsigned>(sizeof(float))
                                  : kRejectedOffset;
     }
     // kThreads is a multiple of the tile's float4 columns, so a thread's
     // column is the same for all of its copies.
-    const unsigned x_column = (thread % (kRound / 4)) * 4;
+    const unsigned x_column = (thread % (kSlab / 4)) * 4;
     const auto load_x = [&](floatx4 (&staged)[kCopies], const Cursor& c) {
-        const unsigned k0 = c.round * kRound;
+        const unsigned k0 = c.slab * kSlab;
         const bool valid = c.left > 0 && k0 + x_column < input_width;
 #pragma unroll
         for (int i = 0; i < kCopies; ++i) {
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
 #pragma unroll
         for (int i = 0; i < kCopies; ++i) {
             const unsigned index = thread + kThreads * i;
-            const unsigned row = index / (kRound / 4);
+            const unsigned row = index / (kSlab / 4);
             *reinterpret_cast<floatx4*>(x_tile + row * kStride + x_column) =
                 staged[i];
         }
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
     const unsigned lane_row = wave * 16 + lane % 16;  // within the tile
     const auto load_codes = [&](Codes& staged, const Cursor& c) {
         const unsigned n = c.tile * kTileN + lane_row;
-        const unsigned k = c.round * kRound + quarter * kChunk;
+        const unsigned k = c.slab * kSlab + quarter * kChunk;
         const bool valid = c.left > 0 && n < output_width && k < input_width;
         const unsigned flat = n * input_width + k;
         const unsigned code_offset = valid ? flat >> 1 : kRejectedOffset;
@@ -247,7 +247,7 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
     };
     clear_accumulators();
 
-    // Where an output tile goes once its last round of this run is done.
+    // Where an output tile goes once its last slab of this run is done.
     // Accumulator element r of lane l in block b is x row 16 b + 4 (l / 16) + r
     // and weight row l % 16 of the wavefront.
     const auto flush = [&](unsigned tile, bool whole_tile, unsigned slot) {
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
     };
 
     const unsigned first_tile = compute_cursor.tile;
-    unsigned segment_first_round = compute_cursor.round;
+    unsigned segment_first_slab = compute_cursor.slab;
 
     floatx4 x_staged[kCopies];
     Codes ring[kDepth];
@@ -318,44 +318,22 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
     // consecutive values at 64 * quarter.
     const float* fragment = x_tile + (lane % 16) * kStride + quarter * kChunk;
 
-    // The inner loop is software-pipelined by hand.  A stage is the 16 matrix
-    // instructions of one (sub-chunk of 16 contraction values, block of x)
-    // pair; they form a dependent chain, so the wavefront has eight issue
-    // slots free behind each of them.  Everything else is placed in those
-    // slots, two sub-chunks ahead of its use:
-    //   stage (c, 0): table lookups of sub-chunk c + 2, the multiplies that
-    //                 turn the levels of sub-chunk c + 1 into weights,
-    //   every stage:  the x fragment of the next stage,
-    // with sched_group_barrier spelling out the interleaving.  Sub-chunks
-    // count on across rounds (c + 1 == 4 is the next round's first), so the
-    // only exposed LDS latency is the first x fragment after the barrier.
-    // Levels looked up.  With one block of x the lookups of sub-chunk c + 2
-    // are issued in the stage that consumes those of c + 1, so there are two
-    // buffers (by parity); with more blocks the two fall into different
-    // stages and one buffer is enough.
-    constexpr int kRawBuffers = kBlocks == 1 ? 2 : 1;
-    float2 raw[kRawBuffers][8];
-    float w[2][16];    // weights, by sub-chunk parity
-    const auto issue_lookups = [&](float2 (&out)[8], const Codes& codes,
-                                   int c) {
+    // The inner loop is software-pipelined by hand so that no LDS latency is
+    // exposed to the matrix pipe: the table lookups of sub-chunk c + 1 and the
+    // x fragment of the next (sub-chunk, block) stage are issued BEFORE the
+    // matrix instructions of the current stage, and the lookups of a slab's
+    // first sub-chunk are issued at the end of the previous slab.
+    float2 raw[8];  // levels of the sub-chunk being looked up
+    const auto issue_lookups = [&](const Codes& codes, int c) {
         const unsigned words[2] = {codes.codes[c / 2][2 * (c % 2)],
                                    codes.codes[c / 2][2 * (c % 2) + 1]};
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
 #pragma unroll
             for (int byte = 0; byte < 4; ++byte) {
-                out[4 * half + byte] =
+                raw[4 * half + byte] =
                     pair_table_lookup(table, words[half], byte, lane_bits);
             }
-        }
-    };
-    const auto scale_levels = [&](float (&out)[16], const float2 (&levels)[8],
-                                  float scale) {
-#pragma clang fp contract(off)
-#pragma unroll
-        for (int p = 0; p < 8; ++p) {
-            out[2 * p] = levels[p].x * scale;
-            out[2 * p + 1] = levels[p].y * scale;
         }
     };
     const auto issue_fragment = [&](floatx4 (&a)[4], int c, int b) {
@@ -367,12 +345,10 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
     };
 
     __syncthreads();  // the table is built
-    issue_lookups(raw[0], ring[0], 0);
-    scale_levels(w[0], raw[0], ring[0].scales[0]);
-    issue_lookups(raw[1 % kRawBuffers], ring[0], 1);
+    issue_lookups(ring[0], 0);
 
     for (unsigned step = 0; step < unit_count; ++step) {
-        __syncthreads();  // the previous round's fragment reads are done
+        __syncthreads();  // the previous slab's fragment reads are done
         store_x(x_staged);
         __syncthreads();
         load_x(x_staged, x_cursor);
@@ -385,73 +361,60 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
         }
         load_codes(ring[kDepth - 1], code_cursor);
         advance(code_cursor);
-        // `current` is this round, ring[0] the next one.
 
         floatx4 a[2][4];
         issue_fragment(a[0], 0, 0);
+        // Four sub-chunks of 16 contraction values, kBlocks stages each.
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
+            float w[16];
+            {
+#pragma clang fp contract(off)
+                const float scale = current.scales[c * kScales / 4];
+#pragma unroll
+                for (int p = 0; p < 8; ++p) {
+                    w[2 * p] = raw[p].x * scale;
+                    w[2 * p + 1] = raw[p].y * scale;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (c + 1 < 4) {
+                issue_lookups(current, c + 1);
+            } else {
+                issue_lookups(ring[0], 0);  // the next slab's first
+            }
 #pragma unroll
             for (int b = 0; b < kBlocks; ++b) {
                 constexpr int kStages = 4 * kBlocks;
                 const int stage = c * kBlocks + b;
-                __builtin_amdgcn_sched_barrier(0);
                 if (stage + 1 < kStages) {
                     issue_fragment(a[(stage + 1) % 2], (stage + 1) / kBlocks,
                                    (stage + 1) % kBlocks);
                 }
-                if (b == 0) {
-                    // weights of sub-chunk c + 1 from the levels fetched
-                    // during sub-chunk c - 1 ...
-                    if (c + 1 < 4) {
-                        scale_levels(
-                            w[(c + 1) % 2], raw[(c + 1) % kRawBuffers],
-                            current.scales[(c + 1) * kScales / 4]);
-                    } else {
-                        scale_levels(w[0], raw[0], ring[0].scales[0]);
-                    }
-                }
-                if (b == kBlocks - 1) {
-                    // ... and, once those levels are consumed, the lookups
-                    // of sub-chunk c + 2 into the same registers' partner.
-                    if (c + 2 < 4) {
-                        issue_lookups(raw[c % kRawBuffers], current, c + 2);
-                    } else {
-                        issue_lookups(raw[c % kRawBuffers], ring[0],
-                                      c + 2 - 4);
-                    }
-                }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                            a[stage % 2][v][e], w[c % 2][4 * v + e], acc[b],
-                            0, 0, 0);
+                            a[stage % 2][v][e], w[4 * v + e], acc[b], 0, 0,
+                            0);
                     }
-                }
-                // One matrix instruction, then up to two vector-ALU
-                // instructions and one LDS read in its shadow, sixteen times.
-#pragma unroll
-                for (int slot = 0; slot < 16; ++slot) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
 
         // End of this run's part of the tile?
-        const bool tile_done = compute_cursor.round + 1 == split.rounds;
+        const bool tile_done = compute_cursor.slab + 1 == split.slabs;
         if (tile_done || step + 1 == unit_count) {  // uniform
-            const bool whole_tile = segment_first_round == 0 && tile_done;
+            const bool whole_tile = segment_first_slab == 0 && tile_done;
             const unsigned slot =
                 group * kSlotsPerGroup +
                 (compute_cursor.tile == first_tile ? 0U : 1U);
             flush(compute_cursor.tile, whole_tile, slot);
             clear_accumulators();
-            segment_first_round = 0;
+            segment_first_slab = 0;
         }
         advance(compute_cursor);
     }
@@ -469,9 +432,9 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(
     constexpr int kRows = 16 * kBlocks;
     constexpr int kBatch = 8;  // partial tiles fetched together
     const unsigned tile = blockIdx.x;
-    const unsigned first_unit = tile * split.rounds;
+    const unsigned first_unit = tile * split.slabs;
     const unsigned first_group = split.owner(first_unit);
-    const unsigned last_group = split.owner(first_unit + split.rounds - 1);
+    const unsigned last_group = split.owner(first_unit + split.slabs - 1);
     if (first_group == last_group) {
         return;  // written directly by its only workgroup
     }
@@ -492,7 +455,7 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(
             // A workgroup's slot 0 holds the first tile of its run.
             const unsigned slot =
                 g * kSlotsPerGroup +
-                (tile == split.begin(g) / split.rounds ? 0U : 1U);
+                (tile == split.begin(g) / split.slabs ? 0U : 1U);
             part[j] = g <= last_group
                           ? source[static_cast<std::size_t>(slot) * kRows *
                                    kTileN]
@@ -574,9 +537,9 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     const unsigned tiles =
         static_cast<unsigned>((p.output_width + kTileN - 1) / kTileN);
     UnitSplit split;
-    split.rounds =
-        static_cast<unsigned>((p.input_width + kRound - 1) / kRound);
-    const unsigned units = tiles * split.rounds;
+    split.slabs =
+        static_cast<unsigned>((p.input_width + kSlab - 1) / kSlab);
+    const unsigned units = tiles * split.slabs;
     // One workgroup per compute unit; with at least that many tiles, one
     // workgroup per tile (no partial tiles at all).
     const unsigned groups =

@@ -248,7 +248,7 @@ def test_ragged_shapes_and_block_sizes(gpu, package, library, oracle, out_w,
 
 @pytest.mark.parametrize("out_w,in_w,block,double_quantized", [
     (33000, 64, 32, False),    # >= 256 output tiles: one workgroup per tile
-    (300, 1280, 64, True),     # fewer (tile, round) units than compute units
+    (300, 1280, 64, True),     # fewer (tile, slab) units than compute units
     (2000, 1600, 64, False),   # last round and last tile partly empty
     (5000, 2048, 64, True),    # runs of one and two units, tiles shared
     (1000, 16384, 128, False),  # many workgroups per output tile
@@ -256,7 +256,7 @@ def test_ragged_shapes_and_block_sizes(gpu, package, library, oracle, out_w,
 ])
 def test_small_batch_work_split(gpu, package, library, oracle, out_w, in_w,
                                 block, double_quantized):
-    """Shapes chosen for how the small-batch family deals (tile, round) units
+    """Shapes chosen for how the small-batch family deals (tile, slab) units
     to workgroups: whole tiles written directly, partial tiles added by the
     second kernel, with bias."""
     dense = helpers.normal(65, (out_w, in_w), 0.02)
