@@ -35,10 +35,13 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <map>
+#include <mutex>
 #include <new>
 #include <stdexcept>
 #include <string>
 #include <utility>
+#include <vector>
 
 namespace riftco_transformer::backend_detail {
 namespace {
@@ -81,34 +84,155 @@ void check(const HipRuntime& runtime, rthip_status status,
     }
 }
 
-// Owning handle of one HBM allocation.
+bool environment_flag(const char* name) noexcept {
+    const char* value = std::getenv(name);
+    return value != nullptr && std::strcmp(value, "1") == 0;
+}
+
+// Activation buffers come and go with every operation
+// (src/nn/quantized_linear.cpp:41 allocates the output of each forward), and
+// a device allocation costs far more than the decode kernels do.  Released
+// buffers are therefore kept, by power-of-two size class, and handed out
+// again.  Every launch and copy of the adapter goes to the default stream, so
+// a buffer that is reused is only touched after the work that last used it.
+// RIFTCO_TRANSFORMER_HIP_POOL=0 turns the pool off; it holds at most
+// kPoolLimitBytes and never buffers above kLargestPooledBytes.
+class BufferPool final {
+public:
+    static BufferPool& instance() {
+        static BufferPool* pool = new BufferPool();  // outlives every tensor
+        return *pool;
+    }
+
+    // Capacity actually allocated for a request (the size class).
+    [[nodiscard]] static std::size_t capacity_for(std::size_t bytes) noexcept {
+        if (bytes > kLargestPooledBytes) {
+            return bytes;
+        }
+        std::size_t capacity = kSmallestClassBytes;
+        while (capacity < bytes) {
+            capacity *= 2;
+        }
+        return capacity;
+    }
+
+    [[nodiscard]] void* acquire(std::size_t capacity) {
+        if (enabled_ && capacity <= kLargestPooledBytes) {
+            const std::lock_guard<std::mutex> lock(guard_);
+            auto& free_list = free_[capacity];
+            if (!free_list.empty()) {
+                void* pointer = free_list.back();
+                free_list.pop_back();
+                held_bytes_ -= capacity;
+                return pointer;
+            }
+        }
+        const HipRuntime& runtime = require_runtime();
+        void* pointer = nullptr;
+        rthip_status status = runtime.malloc(&pointer, capacity);
+        if (status == RTHIP_OUT_OF_MEMORY && trim()) {
+            status = runtime.malloc(&pointer, capacity);
+        }
+        check(runtime, status, "device allocation");
+        return pointer;
+    }
+
+    void release(void* pointer, std::size_t capacity) noexcept {
+        if (enabled_ && capacity <= kLargestPooledBytes) {
+            const std::lock_guard<std::mutex> lock(guard_);
+            if (held_bytes_ + capacity <= kPoolLimitBytes) {
+                try {
+                    free_[capacity].push_back(pointer);
+                    held_bytes_ += capacity;
+                    return;
+                } catch (...) {
+                    // fall through to a plain free
+                }
+            }
+        }
+        static_cast<void>(hip_runtime().free(pointer));
+    }
+
+private:
+    static constexpr std::size_t kSmallestClassBytes = 256;
+    static constexpr std::size_t kLargestPooledBytes = std::size_t{1} << 28;
+    static constexpr std::size_t kPoolLimitBytes = std::size_t{1} << 31;
+
+    BufferPool() {
+        const char* value = std::getenv("RIFTCO_TRANSFORMER_HIP_POOL");
+        enabled_ = value == nullptr || std::strcmp(value, "0") != 0;
+    }
+
+    // Gives everything back to the driver; true if that freed anything.
+    bool trim() noexcept {
+        const std::lock_guard<std::mutex> lock(guard_);
+        bool freed = false;
+        for (auto& [capacity, free_list] : free_) {
+            for (void* pointer : free_list) {
+                static_cast<void>(hip_runtime().free(pointer));
+                freed = true;
+            }
+            free_list.clear();
+        }
+        held_bytes_ = 0;
+        return freed;
+    }
+
+    bool enabled_ = true;
+    std::mutex guard_;
+    std::map<std::size_t, std::vector<void*>> free_;
+    std::size_t held_bytes_ = 0;
+};
+
+// Owning handle of one HBM allocation.  Pooled buffers (activations) come
+// from BufferPool; exact ones (weight payloads, which live as long as the
+// model) are allocated and freed directly.
 class DeviceBuffer final {
 public:
+    enum class Kind { Exact, Pooled };
+
     DeviceBuffer() = default;
-    explicit DeviceBuffer(std::size_t bytes) : bytes_(bytes) {
-        if (bytes_ != 0) {
+    explicit DeviceBuffer(std::size_t bytes, Kind kind = Kind::Exact)
+        : bytes_(bytes), kind_(kind) {
+        if (bytes_ == 0) {
+            return;
+        }
+        if (kind_ == Kind::Pooled) {
+            capacity_ = BufferPool::capacity_for(bytes_);
+            pointer_ = BufferPool::instance().acquire(capacity_);
+        } else {
+            capacity_ = bytes_;
             const HipRuntime& runtime = require_runtime();
             check(runtime, runtime.malloc(&pointer_, bytes_),
                   "device allocation");
         }
     }
-    DeviceBuffer(const void* host, std::size_t bytes) : DeviceBuffer(bytes) {
+    DeviceBuffer(const void* host, std::size_t bytes, Kind kind = Kind::Exact)
+        : DeviceBuffer(bytes, kind) {
         if (bytes_ != 0) {
             const HipRuntime& runtime = require_runtime();
-            check(runtime, runtime.copy_to_device(pointer_, host, bytes_),
-                  "host-to-device copy");
+            const rthip_status status =
+                runtime.copy_to_device(pointer_, host, bytes_);
+            if (status != RTHIP_OK) {
+                release();
+                check(runtime, status, "host-to-device copy");
+            }
         }
     }
     DeviceBuffer(const DeviceBuffer&) = delete;
     DeviceBuffer& operator=(const DeviceBuffer&) = delete;
     DeviceBuffer(DeviceBuffer&& other) noexcept
         : pointer_(std::exchange(other.pointer_, nullptr)),
-          bytes_(std::exchange(other.bytes_, 0)) {}
+          bytes_(std::exchange(other.bytes_, 0)),
+          capacity_(std::exchange(other.capacity_, 0)),
+          kind_(other.kind_) {}
     DeviceBuffer& operator=(DeviceBuffer&& other) noexcept {
         if (this != &other) {
             release();
             pointer_ = std::exchange(other.pointer_, nullptr);
             bytes_ = std::exchange(other.bytes_, 0);
+            capacity_ = std::exchange(other.capacity_, 0);
+            kind_ = other.kind_;
         }
         return *this;
     }
@@ -119,34 +243,57 @@ public:
 
 private:
     void release() noexcept {
-        if (pointer_ != nullptr) {
-            static_cast<void>(hip_runtime().free(pointer_));
-            pointer_ = nullptr;
+        if (pointer_ == nullptr) {
+            return;
         }
+        if (kind_ == Kind::Pooled) {
+            BufferPool::instance().release(pointer_, capacity_);
+        } else {
+            static_cast<void>(hip_runtime().free(pointer_));
+        }
+        pointer_ = nullptr;
     }
 
     void* pointer_ = nullptr;
     std::size_t bytes_ = 0;
+    std::size_t capacity_ = 0;
+    Kind kind_ = Kind::Exact;
 };
+
+// The reference contract is that an adapter has finished writing its output
+// when it returns (docs/BACKENDS_AND_PYTHON.md:168), and that is the default
+// here: every launch is followed by a synchronisation.  Host code can only
+// see a hip tensor through data(), which copies from the device with a call
+// that itself waits for the default stream, so the synchronisation per
+// operation is not needed for correctness; RIFTCO_TRANSFORMER_HIP_ASYNC=1
+// drops it, and operations then queue behind each other on the device.
+// (Errors of a queued kernel surface at the next synchronising call.)
+void finish_operation(const HipRuntime& runtime, std::string_view operation) {
+    static const bool deferred =
+        environment_flag("RIFTCO_TRANSFORMER_HIP_ASYNC");
+    if (!deferred) {
+        check(runtime, runtime.stream_synchronize(nullptr), operation);
+    }
+}
 
 class HipTensorStorage final : public TensorStorage {
 public:
     HipTensorStorage(std::size_t element_count, float fill_value)
         : count_(element_count),
-          device_(checked_bytes(element_count)),
+          device_(checked_bytes(element_count), DeviceBuffer::Kind::Pooled),
           freshest_(Freshest::Device) {
         const HipRuntime& runtime = require_runtime();
         check(runtime,
               runtime.fill_f32(static_cast<float*>(device_.get()), fill_value,
                                count_, nullptr),
               "tensor fill");
-        check(runtime, runtime.stream_synchronize(nullptr),
-              "tensor fill synchronisation");
+        finish_operation(runtime, "tensor fill synchronisation");
     }
 
     explicit HipTensorStorage(std::vector<float> values)
         : count_(values.size()),
-          device_(values.data(), checked_bytes(values.size())),
+          device_(values.data(), checked_bytes(values.size()),
+                  DeviceBuffer::Kind::Pooled),
           host_(std::move(values)),
           freshest_(Freshest::Both) {}
 
@@ -270,8 +417,7 @@ private:
 };
 
 bool scale_mirror_requested() noexcept {
-    const char* value = std::getenv("RIFTCO_TRANSFORMER_HIP_SCALE_MIRROR");
-    return value != nullptr && std::strcmp(value, "1") == 0;
+    return environment_flag("RIFTCO_TRANSFORMER_HIP_SCALE_MIRROR");
 }
 
 class HipNf4WeightStorage final : public QuantizedWeightStorage,
@@ -453,8 +599,8 @@ public:
                   request.dimensions.output_width,
                   request.dimensions.block_size, nullptr),
               operation);
-        check(runtime, runtime.stream_synchronize(nullptr),
-              "quantized-linear forward synchronisation");
+        finish_operation(runtime,
+                         "quantized-linear forward synchronisation");
     }
 
     void quantized_linear_input_backward(
@@ -482,8 +628,8 @@ public:
                   request.dimensions.output_width,
                   request.dimensions.block_size, nullptr),
               operation);
-        check(runtime, runtime.stream_synchronize(nullptr),
-              "quantized-linear input-backward synchronisation");
+        finish_operation(runtime,
+                         "quantized-linear input-backward synchronisation");
     }
 
 #if defined(RIFTCO_TRANSFORMER_IN_TREE)
@@ -510,8 +656,7 @@ public:
                              request.dimensions.shared,
                              request.dimensions.columns, nullptr),
               operation);
-        check(runtime, runtime.stream_synchronize(nullptr),
-              "matmul synchronisation");
+        finish_operation(runtime, "matmul synchronisation");
     }
     void unary_elementwise(
         const UnaryElementwiseRequest& request) const override {

@@ -592,7 +592,10 @@ void test_out_of_memory_maps_to_bad_alloc() {
     setenv("FAKE_RTHIP_OUT_OF_MEMORY", "1", 1);
     require_throws<std::bad_alloc>(
         [&] {
-            static_cast<void>(backend::make_tensor_storage(kHip, 16, 0.0F));
+            // larger than anything the adapter's buffer pool keeps, so the
+            // request always reaches the runtime
+            static_cast<void>(backend::make_tensor_storage(
+                kHip, (std::size_t{1} << 26) + 1, 0.0F));
         },
         "device out-of-memory must surface as std::bad_alloc");
     unsetenv("FAKE_RTHIP_OUT_OF_MEMORY");

@@ -42,6 +42,17 @@ def test_adapter_on_the_host_only_runtime():
                     FAKE_RTHIP_CAN_FAIL="1"))
 
 
+@pytest.mark.parametrize("options", [
+    {"RIFTCO_TRANSFORMER_HIP_POOL": "0"},
+    {"RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
+    {"RIFTCO_TRANSFORMER_HIP_POOL": "0", "RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
+])
+def test_adapter_options_on_the_host_only_runtime(options):
+    """Without the buffer pool, and without the per-operation synchronise."""
+    expect_pass(run(RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE,
+                    RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1", **options))
+
+
 def test_adapter_keeps_a_counted_mirror_without_host_visible_memory():
     expect_pass(run(RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE,
                     RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1",
@@ -95,3 +106,16 @@ def test_adapter_on_the_real_library():
                  RIFTCO_TRANSFORMER_HIP_REJECT_TEST_PLUGIN="1")
     expect_pass(result)
     assert "unavailable" not in result.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("options", [
+    {"RIFTCO_TRANSFORMER_HIP_POOL": "0"},
+    {"RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
+])
+def test_adapter_options_on_the_real_library(options):
+    """The pool switched off, and operations queued without a synchronise per
+    call: same results, because host reads go through a synchronising copy."""
+    result = run(RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1",
+                 RIFTCO_TRANSFORMER_HIP_REJECT_TEST_PLUGIN="1", **options)
+    expect_pass(result)
