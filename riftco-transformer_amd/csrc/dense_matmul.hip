@@ -17,6 +17,12 @@
 // 16-byte aligned pointers are required -- other shapes take the plain kernel
 // below, which is also the exact restatement of the reference loop (one fp32
 // accumulator per output, ascending k).
+//
+// Narrow products (an adapter's x A^T, its gradients) have few output tiles and
+// a long contraction; they would occupy a handful of compute units.  For a
+// single matrix with fewer than 128 tiles the contraction is therefore cut
+// into slices, one workgroup per (tile, slice) writes its partial tile to the
+// stream's workspace, and a second kernel adds the slices in ascending order.
 
 #include "kernels.hpp"
 
@@ -36,6 +42,9 @@ struct MatmulShape {
     unsigned rows;     // M
     unsigned shared;   // K
     unsigned columns;  // N
+    // 0: blockIdx.z is the batch.  Otherwise blockIdx.z is a slice of this
+    // many contraction values and `out` is the workspace of partial results.
+    unsigned slice;
 };
 
 struct Staged {
@@ -121,10 +130,19 @@ __global__ __launch_bounds__(kThreads, 2) void dense_matmul_kernel(
     const unsigned wave_n = wave % 2;
     const unsigned row0 = blockIdx.y * kTileM;
     const unsigned col0 = blockIdx.x * kTileN;
-    const std::size_t batch = blockIdx.z;
-    left += batch * shape.rows * shape.shared;
-    right += batch * shape.shared * shape.columns;
-    out += batch * shape.rows * shape.columns;
+    unsigned k_begin = 0;
+    unsigned k_end = shape.shared;
+    if (shape.slice == 0) {
+        const std::size_t batch = blockIdx.z;
+        left += batch * shape.rows * shape.shared;
+        right += batch * shape.shared * shape.columns;
+        out += batch * shape.rows * shape.columns;
+    } else {
+        k_begin = blockIdx.z * shape.slice;
+        k_end = min(k_begin + shape.slice, shape.shared);
+        out += static_cast<std::size_t>(blockIdx.z) * shape.rows *
+               shape.columns;
+    }
 
     floatx16 acc[2][2];
     floatx16 total[2][2];
@@ -141,22 +159,24 @@ __global__ __launch_bounds__(kThreads, 2) void dense_matmul_kernel(
     }
     unsigned steps_since_flush = 0;
 
+    // (loads past k_end of a slice are not masked: slices are multiples of
+    // the step, so only the last slice ends inside a step, at the matrix edge)
     Staged staged;
-    load_left(staged, left, shape, row0, 0);
-    load_right(staged, right, shape, col0, 0);
+    load_left(staged, left, shape, row0, k_begin);
+    load_right(staged, right, shape, col0, k_begin);
 
     const float* left_fragment =
         left_tile + (wave_m * 64 + lane % 32) * kStride + 4 * (lane / 32);
     const float* right_fragment =
         right_tile + (wave_n * 64 + lane % 32) * kStride + 4 * (lane / 32);
 
-    for (unsigned k0 = 0; k0 < shape.shared; k0 += kTileK) {
+    for (unsigned k0 = k_begin; k0 < k_end; k0 += kTileK) {
         __syncthreads();  // previous step's fragment reads are done
         store_tiles(staged, left_tile, right_tile);
         __syncthreads();
 
         const unsigned next = k0 + kTileK;
-        if (next < shape.shared) {
+        if (next < k_end) {
             load_left(staged, left, shape, row0, next);
             load_right(staged, right, shape, col0, next);
         }
@@ -229,6 +249,22 @@ __global__ __launch_bounds__(kThreads, 2) void dense_matmul_kernel(
     }
 }
 
+// out[i] = sum over slices of partial[slice][i], ascending.
+__global__ __launch_bounds__(256) void add_slices_kernel(
+    const float* __restrict__ partial, float* __restrict__ out,
+    unsigned count, unsigned slices
+) {
+    const unsigned index = blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= count) {
+        return;
+    }
+    float sum = 0.0F;
+    for (unsigned s = 0; s < slices; ++s) {
+        sum += partial[static_cast<std::size_t>(s) * count + index];
+    }
+    out[index] = sum;
+}
+
 // Any shape: one thread per output, one fp32 accumulator, ascending k --
 // the reference loop itself.  Neighbouring threads take neighbouring columns.
 __global__ __launch_bounds__(256) void plain_matmul_kernel(
@@ -258,10 +294,10 @@ __global__ __launch_bounds__(256) void plain_matmul_kernel(
 
 }  // namespace
 
-void launch_dense_matmul(const float* left, const float* right, float* out,
-                         std::size_t batch_count, std::size_t rows,
-                         std::size_t shared, std::size_t columns,
-                         hipStream_t stream) {
+hipError_t launch_dense_matmul(const float* left, const float* right,
+                               float* out, std::size_t batch_count,
+                               std::size_t rows, std::size_t shared,
+                               std::size_t columns, hipStream_t stream) {
     constexpr std::size_t kLimit = 1ULL << 31;
     const std::size_t tiles_m = (rows + kTileM - 1) / kTileM;
     const std::size_t tiles_n = (columns + kTileN - 1) / kTileN;
@@ -278,12 +314,48 @@ void launch_dense_matmul(const float* left, const float* right, float* out,
         shape.rows = static_cast<unsigned>(rows);
         shape.shared = static_cast<unsigned>(shared);
         shape.columns = static_cast<unsigned>(columns);
+        shape.slice = 0;
+        const std::size_t tiles = tiles_m * tiles_n;
+        const std::size_t steps = (shared + kTileK - 1) / kTileK;
+        // Slices: enough workgroups for the device, at least four steps each,
+        // and partial results that fit the workspace.
+        std::size_t slices = 1;
+        if (batch_count == 1 && tiles < 128 && steps >= 8) {
+            slices = (256 + tiles - 1) / tiles;
+            if (slices > steps / 4) {
+                slices = steps / 4;
+            }
+            const std::size_t fit =
+                kStreamWorkspaceBytes / (rows * columns * sizeof(float));
+            if (slices > fit) {
+                slices = fit;
+            }
+        }
+        if (slices > 1) {
+            const std::size_t steps_per_slice = (steps + slices - 1) / slices;
+            shape.slice = static_cast<unsigned>(steps_per_slice * kTileK);
+            slices = (shared + shape.slice - 1) / shape.slice;
+            float* workspace = nullptr;
+            if (const hipError_t status = stream_workspace(stream, &workspace);
+                status != hipSuccess) {
+                return status;
+            }
+            const dim3 grid(static_cast<unsigned>(tiles_n),
+                            static_cast<unsigned>(tiles_m),
+                            static_cast<unsigned>(slices));
+            dense_matmul_kernel<<<grid, kThreads, 0, stream>>>(
+                left, right, workspace, shape);
+            const unsigned count = static_cast<unsigned>(rows * columns);
+            add_slices_kernel<<<(count + 255) / 256, 256, 0, stream>>>(
+                workspace, out, count, static_cast<unsigned>(slices));
+            return hipSuccess;
+        }
         const dim3 grid(static_cast<unsigned>(tiles_n),
                         static_cast<unsigned>(tiles_m),
                         static_cast<unsigned>(batch_count));
         dense_matmul_kernel<<<grid, kThreads, 0, stream>>>(left, right, out,
                                                            shape);
-        return;
+        return hipSuccess;
     }
     const std::size_t outputs = batch_count * rows * columns;
     std::size_t blocks = (outputs + 255) / 256;
@@ -295,6 +367,7 @@ void launch_dense_matmul(const float* left, const float* right, float* out,
     }
     plain_matmul_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
         left, right, out, batch_count, rows, shared, columns);
+    return hipSuccess;
 }
 
 }  // namespace rthip

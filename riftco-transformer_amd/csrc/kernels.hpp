@@ -45,6 +45,11 @@ constexpr std::size_t kGemvMaxRows = 4;
 bool gemv_forward_supports(const LinearProblem& problem);
 void launch_gemv_forward(const LinearProblem& problem, hipStream_t stream);
 
+// workspace.hip -- scratch memory shared by the kernels that pass partial
+// results between workgroups; one fixed-size buffer per (device, stream).
+constexpr std::size_t kStreamWorkspaceBytes = std::size_t{32} << 20;
+hipError_t stream_workspace(hipStream_t stream, float** out);
+
 // nf4_skinny.hip -- forward only, up to 64 rows, decode straight into MFMA
 // operands.  Shapes whose output tiles are shared between workgroups use a
 // per-stream workspace that is allocated on first use, so the launcher can
@@ -61,10 +66,10 @@ void launch_lora_reduce(const float* x, const float* a, float* reduced,
 
 // dense_matmul.hip -- out[b] = left[b] [rows, shared] * right[b] [shared,
 // columns], plain fp32.
-void launch_dense_matmul(const float* left, const float* right, float* out,
-                         std::size_t batch_count, std::size_t rows,
-                         std::size_t shared, std::size_t columns,
-                         hipStream_t stream);
+hipError_t launch_dense_matmul(const float* left, const float* right,
+                               float* out, std::size_t batch_count,
+                               std::size_t rows, std::size_t shared,
+                               std::size_t columns, hipStream_t stream);
 
 // nf4_quantize.hip -- the quantizer.  fp32_scales always receives the block
 // scales; scale_codes == nullptr means plain fp32 scales, otherwise the

@@ -43,9 +43,6 @@
 #include "nf4_decode.hpp"
 #include "nf4_pair_table.hpp"
 
-#include <mutex>
-#include <unordered_map>
-
 namespace rthip {
 namespace {
 
@@ -475,49 +472,12 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(
     y[static_cast<std::size_t>(m) * output_width + n] = sum;
 }
 
-// One workspace per (device, stream): calls on one stream are ordered, so
-// they can share it.  Sized for the largest case; kept until the process
-// ends.
+// Partial tiles of the largest case: two slots of [64][128] floats per
+// workgroup.
 constexpr std::size_t kWorkspaceBytes =
     static_cast<std::size_t>(kComputeUnits) * kSlotsPerGroup * 64 * kTileN *
     sizeof(float);
-
-hipError_t workspace_for(hipStream_t stream, float** out) {
-    static std::mutex guard;
-    static std::unordered_map<std::uintptr_t, float*> buffers;
-    int device = 0;
-    hipError_t status = hipGetDevice(&device);
-    if (status != hipSuccess) {
-        return status;
-    }
-    const std::uintptr_t key = reinterpret_cast<std::uintptr_t>(stream) * 64 +
-                               static_cast<std::uintptr_t>(device);
-    const std::lock_guard<std::mutex> lock(guard);
-    const auto found = buffers.find(key);
-    if (found != buffers.end()) {
-        *out = found->second;
-        return hipSuccess;
-    }
-    // The stream may be recording a graph: allocation is legal there only in
-    // the relaxed capture mode.  The buffer outlives the graph.
-    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
-    status = hipThreadExchangeStreamCaptureMode(&mode);
-    if (status != hipSuccess) {
-        return status;
-    }
-    void* fresh = nullptr;
-    status = hipMalloc(&fresh, kWorkspaceBytes);
-    const hipError_t restored = hipThreadExchangeStreamCaptureMode(&mode);
-    if (status != hipSuccess) {
-        return status;
-    }
-    if (restored != hipSuccess) {
-        return restored;
-    }
-    buffers.emplace(key, static_cast<float*>(fresh));
-    *out = static_cast<float*>(fresh);
-    return hipSuccess;
-}
+static_assert(kWorkspaceBytes <= kStreamWorkspaceBytes);
 
 template <int kBlocks, int kScales, bool kDoubleQuantized>
 hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
@@ -551,7 +511,7 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     const bool partial_tiles = groups != tiles;
     float* workspace = nullptr;
     if (partial_tiles) {
-        const hipError_t status = workspace_for(stream, &workspace);
+        const hipError_t status = stream_workspace(stream, &workspace);
         if (status != hipSuccess) {
             return status;
         }

@@ -548,8 +548,12 @@ rthip_status rthip_matmul(const float* left, const float* right, float* out,
     if (const rthip_status status = require_device(); status != RTHIP_OK) {
         return status;
     }
-    rthip::launch_dense_matmul(left, right, out, batch_count, rows, shared,
-                               columns, static_cast<hipStream_t>(stream));
+    if (const hipError_t status = rthip::launch_dense_matmul(
+            left, right, out, batch_count, rows, shared, columns,
+            static_cast<hipStream_t>(stream));
+        status != hipSuccess) {
+        return from_hip(status, "matmul workspace allocation");
+    }
     return finish_launch("matmul launch");
 }
 

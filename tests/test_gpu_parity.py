@@ -469,6 +469,8 @@ def test_lora_with_zero_b_equals_the_plain_forward(gpu, package, library,
     (1, 16, 300, 1000),     # gradient shape: rows = rank
     (2, 129, 100, 132),     # every edge of the tile
     (1, 512, 2048, 1024),
+    (1, 200, 1000, 260),    # sliced contraction, last slice ends mid-step
+    (1, 2048, 4096, 16),    # sliced contraction, many row tiles
 ])
 def test_dense_matmul(gpu, package, library, oracle, batch, rows, shared,
                       columns):
@@ -490,6 +492,15 @@ def test_dense_matmul(gpu, package, library, oracle, batch, rows, shared,
         cpu_error = np.abs(cpu - exact[sample]).max() / unit
         drift = np.abs(got[index][sample] - cpu).max() / unit
         assert drift <= TOLERANCE + cpu_error, f"matmul vs oracle: {drift:.3g}"
+
+
+def test_sliced_matmul_is_deterministic(gpu, package, library):
+    """A sliced contraction adds its partial results in a fixed order."""
+    left = to_device(helpers.normal(132, (1, 70, 4096), 1.0))
+    right = to_device(helpers.normal(133, (1, 4096, 16), 0.05))
+    first = host(gpu.matmul(left, right))
+    for _ in range(3):
+        helpers.assert_bit_equal(host(gpu.matmul(left, right)), first)
 
 
 def test_dense_matmul_small_integers_are_exact(gpu, package, library):
