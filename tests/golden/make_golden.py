@@ -130,8 +130,56 @@ def llama(reference):
     return arrays, meta
 
 
+def packed_state(reference):
+    """A three-entry packed model state (edge fp32, edge nested, aligned
+    nested) written by oracle/packed_state.py, kept only because the
+    reference's own reader (oracle/_ref/libstateref.so) returns exactly the
+    fields it was written from; and, for each malformed variant of it, what
+    that reader throws."""
+    from oracle import packed_state as restated
+    reader = restated.ReferenceReader()
+    weights = [
+        reference.quantize(helpers.edge_weight(), 32, False, 32),
+        reference.quantize(helpers.edge_weight(), 32, True, 32),
+        reference.quantize(helpers.aligned_weight(), 32, True, 32),
+    ]
+    entries = [restated.from_nf4_weight(weight) for weight in weights]
+    blob = restated.serialize(entries)
+    parsed = reader.parse(blob)
+    assert len(parsed) == len(entries)
+    for got, want in zip(parsed, entries):
+        assert got.shape == list(want.shape)
+        assert got.block_size == want.block_size
+        assert got.double_quantized == want.double_quantized
+        assert np.array_equal(got.packed_codes, want.packed_codes)
+        assert np.array_equal(bits_of(got.block_scales),
+                              bits_of(want.block_scales))
+        if want.double_quantized:
+            assert np.array_equal(got.scale_codes, want.scale_codes)
+            assert np.array_equal(bits_of(got.second_level_scales),
+                                  bits_of(want.second_level_scales))
+            assert got.scale_block_size == want.scale_block_size
+            assert np.float32(got.offset).view(np.uint32) == \
+                np.float32(want.offset).view(np.uint32)
+    outcomes = {}
+    for name, data in helpers.packed_state_mutations(blob):
+        try:
+            outcomes[name] = ["ok", len(reader.parse(data))]
+        except (ValueError, OverflowError) as error:
+            outcomes[name] = [type(error).__name__, str(error)]
+    with open(os.path.join(HERE, "packed_state.bin"), "wb") as handle:
+        handle.write(blob)
+    with open(os.path.join(HERE, "packed_state_outcomes.json"), "w") as handle:
+        json.dump(outcomes, handle, indent=1, sort_keys=True)
+
+
+def bits_of(array):
+    return np.ascontiguousarray(array, dtype=np.float32).view(np.uint32)
+
+
 def main():
     reference = Reference()
+    packed_state(reference)
     np.savez_compressed(os.path.join(HERE, "closed_form.npz"),
                         **closed_form(reference))
     arrays, meta1 = config1(reference)

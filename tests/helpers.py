@@ -133,3 +133,57 @@ def exact_forward(x, dense) -> np.ndarray:
 def exact_input_backward(dy, dense) -> np.ndarray:
     """fp64-accumulated dy . dense."""
     return np.asarray(dy, np.float64) @ np.asarray(dense, np.float64)
+
+
+# ---- packed model state (src/c_api/model_state.cpp under /root/reference) --
+
+def packed_state_mutations(blob: bytes):
+    """(name, bytes) pairs: malformed variants of a valid packed model state
+    whose first entry uses fp32 block scales and whose second is nested.
+    Offsets follow the entry header: rank 0, block size 8, packed codes 16,
+    block scales 24, scale codes 32, second-level scales 40, second-level
+    block size 48, offset 56, flags 60, dimensions 64."""
+    import struct
+
+    def patched(position, fmt, value):
+        data = bytearray(blob)
+        struct.pack_into(fmt, data, position, value)
+        return bytes(data)
+
+    first = 16
+    # the second entry starts after the first one's header, dimensions and
+    # payload
+    packed, scales = struct.unpack_from("<2Q", blob, first + 16)
+    second = first + 64 + 16 + packed + 4 * scales
+    big = (1 << 64) - 1
+    cases = [("intact", blob)]
+    for cut in (0, 4, 7, 8, 12, 15, 16, 20, 50, 79, 80, 95, 96, second - 1,
+                second, second + 30, second + 80, len(blob) - 1):
+        cases.append((f"cut_{cut}", blob[:cut]))
+    cases += [
+        ("magic", b"RTNF4S2\x00" + blob[8:]),
+        ("count_zero", patched(8, "<Q", 0)),
+        ("count_huge", patched(8, "<Q", big)),
+        ("count_more", patched(8, "<Q", 4)),
+        ("count_fewer", patched(8, "<Q", 1)),
+        ("rank_three", patched(first, "<Q", 3)),
+        ("rank_zero", patched(first, "<Q", 0)),
+        ("flags_two", patched(first + 60, "<I", 2)),
+        ("flags_flipped_first", patched(first + 60, "<I", 1)),
+        ("flags_flipped_second", patched(second + 60, "<I", 0)),
+        ("fp32_with_scale_codes", patched(first + 32, "<Q", 1)),
+        ("fp32_with_second_level", patched(first + 40, "<Q", 1)),
+        ("fp32_with_scale_block", patched(first + 48, "<Q", 32)),
+        ("fp32_with_offset", patched(first + 56, "<I", 1)),
+        ("nested_with_block_scales", patched(second + 24, "<Q", 1)),
+        ("nested_without_scale_block", patched(second + 48, "<Q", 0)),
+        ("packed_overflow", patched(first + 16, "<Q", big)),
+        ("scales_overflow", patched(first + 24, "<Q", 1 << 62)),
+        ("second_level_overflow", patched(second + 40, "<Q", 1 << 62)),
+        ("packed_too_long", patched(first + 16, "<Q", 1 << 40)),
+        ("packed_one_more", patched(first + 16, "<Q", packed + 1)),
+        ("packed_one_fewer", patched(first + 16, "<Q", packed - 1)),
+        ("trailing", blob + b"\x00"),
+        ("block_size_unchecked", patched(first + 8, "<Q", 7)),
+    ]
+    return cases
