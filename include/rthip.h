@@ -41,7 +41,7 @@ extern "C" {
 #endif
 
 #define RTHIP_ABI_VERSION_MAJOR 1u
-#define RTHIP_ABI_VERSION_MINOR 1u
+#define RTHIP_ABI_VERSION_MINOR 2u
 
 typedef int32_t rthip_status;
 
@@ -285,6 +285,28 @@ rthip_status rthip_nf4_quantize(
     int32_t encoding, uint64_t second_level_block, uint8_t* codes,
     void* primary_scales, float* secondary_scales, float* fp32_scale_scratch,
     float* host_offset, void* stream);
+
+/*
+ * The content rules of QuantizedWeight::from_packed_nf4's
+ * require_canonical_payload (src/core/quantization/quantized_weight.cpp:
+ * 102-174) applied to a payload that is already in device memory -- what a
+ * loader runs after copying a checkpoint's packed state
+ * (src/c_api/model_state.cpp:166-300) straight into HBM, instead of a pass
+ * over host vectors before the upload.  The array lengths are the caller's to
+ * check; this call reads
+ *   codes [ceil(element_count / 2)], primary_scales [blocks] (float or uint8),
+ *   secondary_scales [ceil(blocks / second_level_block)] (nested only)
+ * and returns, after the work is done, RTHIP_OK or RTHIP_INVALID_ARGUMENT
+ * with the message of the exception the reference would throw first:
+ * a non-zero unused high nibble, a negative or non-finite offset,
+ * second-level scale or decoded block scale, or a block with an fp32 scale of
+ * zero that holds a code other than 7.
+ */
+rthip_status rthip_nf4_check_payload(
+    const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, uint64_t element_count,
+    uint64_t block_size, void* stream);
 
 #ifdef __cplusplus
 }

@@ -6,14 +6,20 @@
 // (RIFTCO_TRANSFORMER_HIP_POOL, RIFTCO_TRANSFORMER_HIP_ASYNC).
 //
 //   bench_adapter [calls]
+//   bench_adapter --packed-state [repeats]
+//       restoring one Llama-7B layer (seven projections, block 64) from a
+//       checkpoint's packed model state into HBM, and writing it back:
+//       hip_load_packed_model_state / hip_packed_model_state_bytes
 
 #include "dispatch.hpp"
+#include "packed_state.hpp"
 
 #include <chrono>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <random>
+#include <string_view>
 #include <vector>
 
 namespace {
@@ -29,9 +35,91 @@ double seconds_since(std::chrono::steady_clock::time_point begin) {
         .count();
 }
 
+int bench_packed_state(int repeats) {
+    struct Shape {
+        std::size_t out_w, in_w;
+    };
+    const Shape layer[] = {{4096, 4096},  {4096, 4096},  {4096, 4096},
+                           {4096, 4096},  {11008, 4096}, {11008, 4096},
+                           {4096, 11008}};
+    std::mt19937 random(9);
+    for (const bool nested : {false, true}) {
+        std::vector<std::unique_ptr<backend::QuantizedWeightStorage>> weights;
+        std::vector<std::vector<std::size_t>> shapes;
+        for (const Shape shape : layer) {
+            const std::size_t count = shape.out_w * shape.in_w;
+            std::vector<std::uint8_t> codes(count / 2);
+            for (auto& byte : codes) {
+                byte = static_cast<std::uint8_t>(random() & 0xFFU);
+            }
+            backend::Nf4ScaleStorageData scales;
+            if (nested) {
+                scales.encoding =
+                    backend::Nf4ScaleEncoding::DoubleQuantizedUInt8;
+                scales.quantized_scales.resize(count / 64);
+                for (auto& code : scales.quantized_scales) {
+                    code = static_cast<std::uint8_t>(random() & 0xFFU);
+                }
+                scales.second_level_scales.assign(count / 64 / 256, 0.01F);
+                scales.second_level_block_size = 256;
+                scales.offset = 0.05F;
+            } else {
+                scales.fp32_scales.assign(count / 64, 0.05F);
+            }
+            weights.push_back(backend::make_nf4_weight_storage(
+                kHip, std::move(codes), std::move(scales)));
+            shapes.push_back({shape.out_w, shape.in_w});
+        }
+        std::vector<backend::HipPackedWeightSource> sources;
+        for (std::size_t index = 0; index < weights.size(); ++index) {
+            sources.push_back({shapes[index], 64, weights[index].get()});
+        }
+        double write_seconds = 0.0;
+        double parse_seconds = 0.0;
+        double load_seconds = 0.0;
+        std::vector<std::uint8_t> state;
+        for (int repeat = -1; repeat < repeats; ++repeat) {  // -1: warm-up
+            auto begin = std::chrono::steady_clock::now();
+            state = backend::hip_packed_model_state_bytes(sources);
+            const double wrote = seconds_since(begin);
+            begin = std::chrono::steady_clock::now();
+            const auto views = backend::parse_packed_model_state(state);
+            const double parsed = seconds_since(begin);
+            begin = std::chrono::steady_clock::now();
+            const auto loaded = backend::hip_load_packed_model_state(state);
+            const double restored = seconds_since(begin);
+            if (loaded.size() != views.size()) {
+                return 1;
+            }
+            if (repeat >= 0) {
+                write_seconds += wrote;
+                parse_seconds += parsed;
+                load_seconds += restored;
+            }
+        }
+        const double megabytes = static_cast<double>(state.size()) / 1e6;
+        std::printf(
+            "packed state, %s scales: %.1f MB; load %.2f ms (%.1f GB/s, of "
+            "which parsing %.3f ms); write %.2f ms (%.1f GB/s)\n",
+            nested ? "nested" : "fp32", megabytes,
+            load_seconds / repeats * 1e3,
+            megabytes / 1e3 / (load_seconds / repeats),
+            parse_seconds / repeats * 1e3, write_seconds / repeats * 1e3,
+            megabytes / 1e3 / (write_seconds / repeats));
+    }
+    return 0;
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
+    if (argc > 1 && std::string_view(argv[1]) == "--packed-state") {
+        if (!riftco_transformer::execution_backend_available(kHip)) {
+            std::fprintf(stderr, "hip backend unavailable\n");
+            return 2;
+        }
+        return bench_packed_state(argc > 2 ? std::atoi(argv[2]) : 5);
+    }
     const int calls = argc > 1 ? std::atoi(argv[1]) : 2000;
     if (!riftco_transformer::execution_backend_available(kHip)) {
         std::fprintf(stderr, "hip backend unavailable: %s\n",

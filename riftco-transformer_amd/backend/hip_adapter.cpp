@@ -24,6 +24,7 @@
 #include "hip_adapter.hpp"
 
 #include "hip_runtime.hpp"
+#include "packed_state.hpp"
 
 #if defined(RIFTCO_TRANSFORMER_IN_TREE)
 #include "core/backend/attention/reference/flash_causal.hpp"
@@ -397,6 +398,19 @@ public:
         }
     }
 
+    // From `count` elements stored as bytes that need not be aligned (a
+    // checkpoint's packed state): copied to HBM from where they lie.
+    WeightArray(std::span<const std::uint8_t> bytes, bool keep_host_copy)
+        : count_(bytes.size() / sizeof(Element)),
+          device_(bytes.data(), bytes.size()) {
+        if (keep_host_copy && count_ != 0) {
+            host_.resize(count_);
+            std::memcpy(host_.data(), bytes.data(), bytes.size());
+        }
+    }
+
+    [[nodiscard]] std::size_t size() const noexcept { return count_; }
+
     [[nodiscard]] std::span<const Element> values() const noexcept {
         if (!host_.empty()) {
             return host_;
@@ -435,6 +449,22 @@ public:
                                !host_visible || scale_mirror_requested()),
           second_level_block_size_(scales.second_level_block_size),
           offset_(scales.offset) {}
+
+    // From one entry of a packed model state: every array goes from the
+    // caller's bytes to HBM without an intermediate vector.
+    HipNf4WeightStorage(const PackedWeightView& weight, bool host_visible)
+        : encoding_(weight.double_quantized
+                        ? Nf4ScaleEncoding::DoubleQuantizedUInt8
+                        : Nf4ScaleEncoding::Float32),
+          packed_codes_(weight.packed_codes, !host_visible),
+          fp32_scales_(weight.block_scale_bytes,
+                       !host_visible || scale_mirror_requested()),
+          quantized_scales_(weight.scale_codes,
+                            !host_visible || scale_mirror_requested()),
+          second_level_scales_(weight.second_level_scale_bytes,
+                               !host_visible || scale_mirror_requested()),
+          second_level_block_size_(weight.scale_block_size),
+          offset_(weight.offset) {}
 
     [[nodiscard]] ExecutionBackend backend() const noexcept override {
         return kHipBackend;
@@ -493,6 +523,28 @@ public:
         return second_level_block_size_;
     }
     [[nodiscard]] float offset() const noexcept { return offset_; }
+
+    [[nodiscard]] std::size_t packed_code_count() const noexcept {
+        return packed_codes_.size();
+    }
+    [[nodiscard]] std::size_t fp32_scale_count() const noexcept {
+        return fp32_scales_.size();
+    }
+    [[nodiscard]] std::size_t scale_code_count() const noexcept {
+        return quantized_scales_.size();
+    }
+    [[nodiscard]] std::size_t second_level_scale_count() const noexcept {
+        return second_level_scales_.size();
+    }
+    [[nodiscard]] const float* fp32_scales_device() const noexcept {
+        return fp32_scales_.device();
+    }
+    [[nodiscard]] const std::uint8_t* scale_codes_device() const noexcept {
+        return quantized_scales_.device();
+    }
+    [[nodiscard]] const float* second_level_scales_device() const noexcept {
+        return second_level_scales_.device();
+    }
 
 private:
     Nf4ScaleEncoding encoding_;
@@ -764,6 +816,105 @@ public:
 const BackendAdapter& hip_backend_adapter() noexcept {
     static const HipBackendAdapter adapter;
     return adapter;
+}
+
+std::vector<HipPackedWeight> hip_load_packed_model_state(
+    std::span<const std::uint8_t> state
+) {
+    const std::vector<PackedWeightView> entries =
+        parse_packed_model_state(state);
+    const HipRuntime& runtime = require_runtime();
+    std::vector<HipPackedWeight> result;
+    result.reserve(entries.size());
+    for (const PackedWeightView& entry : entries) {
+        const std::size_t element_count = require_payload_lengths(entry);
+        auto storage = std::make_unique<HipNf4WeightStorage>(
+            entry, runtime.host_visible_memory);
+        const rthip_status status = runtime.nf4_check_payload(
+            static_cast<const std::uint8_t*>(
+                storage->packed_codes_native_handle()),
+            storage->primary_scales_native_handle(),
+            static_cast<const float*>(
+                storage->secondary_scales_native_handle()),
+            static_cast<std::int32_t>(storage->encoding()),
+            storage->second_level_block_size(), storage->offset(),
+            element_count, entry.block_size, nullptr);
+        if (status == RTHIP_INVALID_ARGUMENT) {
+            // the reference's own message, as from_packed_nf4 throws it
+            throw std::invalid_argument(runtime.last_error());
+        }
+        check(runtime, status, "packed payload check");
+        // The content rules include every rule the dispatcher re-checks
+        // before each launch.
+        storage->mark_scales_validated();
+        result.push_back({entry.shape, entry.block_size, std::move(storage)});
+    }
+    return result;
+}
+
+std::vector<std::uint8_t> hip_packed_model_state_bytes(
+    std::span<const HipPackedWeightSource> weights
+) {
+    const HipRuntime& runtime = require_runtime();
+    // One allocation of the final size: the headers are appended in place
+    // and nothing written so far is ever moved.
+    std::size_t total = 16;
+    for (const HipPackedWeightSource& source : weights) {
+        if (source.storage != nullptr) {
+            total += 64 + 8 * source.shape.size() +
+                     source.storage->packed_codes().size() +
+                     nf4_scale_payload_bytes(source.storage->scale_storage());
+        }
+    }
+    std::vector<std::uint8_t> output;
+    output.reserve(total);
+    append_packed_state_prologue(output, weights.size());
+    struct Pending {
+        const HipNf4WeightStorage* storage;
+        PackedWeightLayout layout;
+    };
+    std::vector<Pending> pending;
+    pending.reserve(weights.size());
+    for (const HipPackedWeightSource& source : weights) {
+        if (source.storage == nullptr) {
+            throw std::invalid_argument(
+                "packed model state needs hip quantized-weight storage");
+        }
+        const HipNf4WeightStorage& storage =
+            require_hip_weight(*source.storage, "packed model state");
+        const bool nested =
+            storage.encoding() == Nf4ScaleEncoding::DoubleQuantizedUInt8;
+        pending.push_back(
+            {&storage,
+             append_packed_weight_header(
+                 output, source.shape, source.block_size,
+                 storage.packed_code_count(), storage.fp32_scale_count(),
+                 nested, storage.scale_code_count(),
+                 storage.second_level_scale_count(),
+                 storage.second_level_block_size(), storage.offset())});
+    }
+    // The vector no longer grows: copy every array from HBM to its place.
+    const auto fetch = [&](std::size_t offset, const void* device,
+                           std::size_t bytes) {
+        if (bytes != 0) {
+            check(runtime,
+                  runtime.copy_to_host(output.data() + offset, device, bytes),
+                  "packed payload read-back");
+        }
+    };
+    for (const Pending& item : pending) {
+        const HipNf4WeightStorage& storage = *item.storage;
+        fetch(item.layout.packed_codes, storage.packed_codes_native_handle(),
+              storage.packed_code_count());
+        fetch(item.layout.block_scales, storage.fp32_scales_device(),
+              storage.fp32_scale_count() * sizeof(float));
+        fetch(item.layout.scale_codes, storage.scale_codes_device(),
+              storage.scale_code_count());
+        fetch(item.layout.second_level_scales,
+              storage.second_level_scales_device(),
+              storage.second_level_scale_count() * sizeof(float));
+    }
+    return output;
 }
 
 }  // namespace riftco_transformer::backend_detail

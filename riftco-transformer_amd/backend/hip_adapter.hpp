@@ -10,6 +10,12 @@
 #include "interface.hpp"
 #endif
 
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <span>
+#include <vector>
+
 namespace riftco_transformer::backend_detail {
 
 // ExecutionBackend::Hip.  Spelled as a cast so that this file also compiles
@@ -20,6 +26,36 @@ inline constexpr ExecutionBackend kHipBackend =
 // Process-lifetime singleton, like cpu_backend_adapter()
 // (src/core/backend/adapters/cpu/adapter.cpp:368-371).
 [[nodiscard]] const BackendAdapter& hip_backend_adapter() noexcept;
+
+// A checkpoint's packed model state (src/c_api/model_state.cpp:34-113,
+// 166-300) and the hip backend.
+//
+// hip_load_packed_model_state is what rt_model_packed_state_load
+// (src/c_api/model_state.cpp:343-376) does up to the point where the model
+// takes the weights -- parse, QuantizedWeight::from_packed_nf4 for every
+// entry, nothing returned unless all entries are valid -- except that each
+// payload array is copied from `state` straight into HBM and the content
+// rules of require_canonical_payload are checked there by a kernel, instead
+// of being copied into vectors, scanned on the host and copied again.
+// Exceptions and messages are the reference's.
+struct HipPackedWeight {
+    std::vector<std::size_t> shape;
+    std::size_t block_size = 0;
+    std::unique_ptr<QuantizedWeightStorage> storage;
+};
+[[nodiscard]] std::vector<HipPackedWeight> hip_load_packed_model_state(
+    std::span<const std::uint8_t> state);
+
+// packed_model_state_bytes (src/c_api/model_state.cpp:34-113) for weights that
+// live in hip storage: the arrays are read from HBM into their place in the
+// result.
+struct HipPackedWeightSource {
+    std::span<const std::size_t> shape;
+    std::size_t block_size = 0;
+    const QuantizedWeightStorage* storage = nullptr;
+};
+[[nodiscard]] std::vector<std::uint8_t> hip_packed_model_state_bytes(
+    std::span<const HipPackedWeightSource> weights);
 
 // Optional extension implemented by hip weight storage: the O(#blocks) scale
 // validation that the dispatcher runs before every launch

@@ -84,7 +84,9 @@ void load(HipRuntime& runtime) {
               runtime.nf4_linear_input_backward, reason) ||
         !bind(library, "rthip_nf4_dequantize", runtime.nf4_dequantize,
               reason) ||
-        !bind(library, "rthip_matmul", runtime.matmul, reason)) {
+        !bind(library, "rthip_matmul", runtime.matmul, reason) ||
+        !bind(library, "rthip_nf4_check_payload", runtime.nf4_check_payload,
+              reason)) {
         return;
     }
     if ((abi_version() >> 16) != RTHIP_ABI_VERSION_MAJOR) {

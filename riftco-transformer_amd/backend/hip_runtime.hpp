@@ -39,6 +39,7 @@ struct HipRuntime {
         nullptr;
     decltype(&rthip_nf4_dequantize) nf4_dequantize = nullptr;
     decltype(&rthip_matmul) matmul = nullptr;
+    decltype(&rthip_nf4_check_payload) nf4_check_payload = nullptr;
 };
 
 // Process-lifetime runtime; loading happens once, on the first call.

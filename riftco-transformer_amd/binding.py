@@ -119,6 +119,7 @@ _PROTOTYPES = {
     "rthip_nf4_quantize": (
         _i32, [_ptr, _u64, _u64, _i32, _u64, _ptr, _ptr, _ptr, _ptr,
                ctypes.POINTER(_f32), _ptr]),
+    "rthip_nf4_check_payload": (_i32, _WEIGHT + [_u64, _u64, _ptr]),
 }
 
 EXPORTED_SYMBOLS = tuple(_PROTOTYPES)
@@ -313,6 +314,16 @@ class Library:
             status = self._lib.rthip_nf4_linear_input_backward_with(
                 algorithm, dy_ptr, *weight.abi_arguments(), *tail)
         self._check(status)
+
+    def check_payload(self, weight: DeviceWeight,
+                      element_count: Optional[int] = None,
+                      stream: int = 0) -> None:
+        """Raises InvalidArgument, with the reference's message, unless the
+        payload satisfies the content rules of a canonical NF4 payload."""
+        if element_count is None:
+            element_count = weight.output_width * weight.input_width
+        self._check(self._lib.rthip_nf4_check_payload(
+            *weight.abi_arguments(), element_count, weight.block_size, stream))
 
     def dequantize(self, weight: DeviceWeight, out_ptr: int,
                    element_count: Optional[int] = None,

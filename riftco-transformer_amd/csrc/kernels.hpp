@@ -90,6 +90,22 @@ struct QuantizeProblem {
 };
 void launch_quantize(const QuantizeProblem& problem, hipStream_t stream);
 
+// nf4_check.hip: content rules of a canonical payload.  words is a device
+// array of three 64-bit words that the launch initialises and fills;
+// classify_payload reads a host copy of it.
+enum class PayloadViolation {
+    None,
+    UnusedNibble,
+    SecondLevelScale,
+    BlockScale,
+    ZeroBlockCode,
+};
+void launch_check_payload(const Nf4WeightView& weight,
+                          std::size_t element_count, unsigned block_shift,
+                          std::size_t second_level_count,
+                          unsigned long long* words, hipStream_t stream);
+PayloadViolation classify_payload(const unsigned long long words[3]);
+
 // nf4_mfma.hip
 bool mfma_forward_supports(const LinearProblem& problem);
 void launch_mfma_forward(const LinearProblem& problem, hipStream_t stream);

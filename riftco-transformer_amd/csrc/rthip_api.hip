@@ -828,4 +828,91 @@ rthip_status rthip_nf4_quantize(
     return ok();
 }
 
+rthip_status rthip_nf4_check_payload(
+    const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, uint64_t element_count,
+    uint64_t block_size, void* stream
+) {
+    if (element_count == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "element count must be positive");
+    }
+    unsigned block_shift = 0;
+    if (!block_shift_for(block_size, &block_shift)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "NF4 block size %llu is not one of 32..4096",
+                    static_cast<unsigned long long>(block_size));
+    }
+    rthip::Nf4WeightView weight{};
+    if (const rthip_status status = make_weight_view(
+            codes, primary_scales, secondary_scales, encoding,
+            second_level_block, offset, &weight);
+        status != RTHIP_OK) {
+        return status;
+    }
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    std::size_t second_level_count = 0;
+    if (encoding == RTHIP_NF4_SCALE_DOUBLE_QUANTIZED_UINT8) {
+        const uint64_t blocks =
+            (element_count + block_size - 1) >> block_shift;
+        second_level_count = (blocks + second_level_block - 1) >>
+                             weight.second_level_shift;
+    }
+    const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+    unsigned long long* words = nullptr;
+    if (const hipError_t error = hipMalloc(reinterpret_cast<void**>(&words),
+                                           3 * sizeof(unsigned long long));
+        error != hipSuccess) {
+        return from_hip(error, "payload check allocation");
+    }
+    unsigned long long host_words[3] = {0, 0, 0};
+    rthip::launch_check_payload(weight, element_count, block_shift,
+                                second_level_count, words, hip_stream);
+    hipError_t error = hipGetLastError();
+    if (error == hipSuccess) {
+        error = hipMemcpyAsync(host_words, words, sizeof(host_words),
+                               hipMemcpyDeviceToHost, hip_stream);
+    }
+    if (error == hipSuccess) {
+        error = hipStreamSynchronize(hip_stream);
+    }
+    const hipError_t released = hipFree(words);
+    if (error != hipSuccess) {
+        return from_hip(error, "NF4 payload check");
+    }
+    if (released != hipSuccess) {
+        return from_hip(released, "payload check release");
+    }
+    // The reference's order: unused nibble, offset, second-level scales,
+    // then the blocks.
+    const rthip::PayloadViolation violation =
+        rthip::classify_payload(host_words);
+    if (violation == rthip::PayloadViolation::UnusedNibble) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "NF4 unused high nibble must be zero");
+    }
+    if (encoding == RTHIP_NF4_SCALE_DOUBLE_QUANTIZED_UINT8 &&
+        (!std::isfinite(offset) || offset < 0.0F)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "double-quantized NF4 scale offset must be finite and "
+                    "nonnegative");
+    }
+    switch (violation) {
+    case rthip::PayloadViolation::SecondLevelScale:
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "NF4 second-level scales must be finite and nonnegative");
+    case rthip::PayloadViolation::BlockScale:
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "NF4 block scales must be finite and nonnegative");
+    case rthip::PayloadViolation::ZeroBlockCode:
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "zero-scale NF4 blocks must use canonical zero code 7");
+    default:
+        return ok();
+    }
+}
+
 }  // extern "C"

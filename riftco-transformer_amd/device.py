@@ -155,6 +155,14 @@ def linear_input_backward(dy: torch.Tensor, weight: DeviceWeight,
     return out
 
 
+def check_payload(weight: DeviceWeight) -> None:
+    """The content rules of require_canonical_payload
+    (src/core/quantization/quantized_weight.cpp:102-174 under /root/reference)
+    on a payload in device memory; raises InvalidArgument with the reference's
+    message for the first rule that is broken."""
+    load_library().check_payload(weight, stream=_stream())
+
+
 def dequantize(weight: DeviceWeight) -> torch.Tensor:
     """deq(W) as an fp32 tensor through rthip_nf4_dequantize (checking aid)."""
     out = torch.empty((weight.output_width, weight.input_width),

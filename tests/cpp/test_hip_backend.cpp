@@ -8,6 +8,8 @@
 //   backend identity / unknown ids
 //       tests/core/backend/test_backend.cpp:172-240
 //   byte-preserving transfer   tests/core/test_quantization.cpp:400-435
+//   packed model state: copy -> load -> copy is byte-identical, a truncated
+//   state is refused      tests/abi/test_c_api.c:3267-3302
 //
 // Plain main(), as the reference's tests are.  Modes:
 //   test_hip_backend                 run against whatever runtime the adapter
@@ -15,9 +17,13 @@
 //   test_hip_backend --expect-unavailable
 //                                    the runtime must be unavailable and the
 //                                    adapter must fail the documented way
+//   test_hip_backend --parse-state FILE...
+//                                    prints, per file, what the packed model
+//                                    state reader makes of it (no runtime)
 // RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP=1 turns "unavailable" into a failure.
 
 #include "../../riftco-transformer_amd/backend/dispatch.hpp"
+#include "../../riftco-transformer_amd/backend/packed_state.hpp"
 
 extern "C" {
 #include "../../oracle/nf4_oracle.h"
@@ -27,7 +33,10 @@ extern "C" {
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <fstream>
 #include <iostream>
+#include <iterator>
+#include <limits>
 #include <new>
 #include <stdexcept>
 #include <string>
@@ -584,6 +593,279 @@ void test_dispatch_validation() {
         "unsupported second-level block", "invalid representation");
 }
 
+// ---- packed model state ---------------------------------------------------
+
+std::vector<std::uint8_t> state_of(
+    const std::vector<const HostWeight*>& weights,
+    const std::vector<std::unique_ptr<backend::QuantizedWeightStorage>>&
+        storages
+) {
+    std::vector<std::vector<std::size_t>> shapes;
+    std::vector<backend::HipPackedWeightSource> sources;
+    for (const HostWeight* weight : weights) {
+        shapes.push_back({weight->output_width, weight->input_width});
+    }
+    for (std::size_t index = 0; index < weights.size(); ++index) {
+        sources.push_back({shapes[index], weights[index]->block_size,
+                           storages[index].get()});
+    }
+    return backend::hip_packed_model_state_bytes(sources);
+}
+
+// What the oracle says about one parsed entry after `damage` was applied.
+std::string oracle_verdict(const backend::PackedWeightView& entry) {
+    std::vector<float> fp32(entry.block_scale_bytes.size() / 4);
+    if (!fp32.empty()) {
+        std::memcpy(fp32.data(), entry.block_scale_bytes.data(),
+                    entry.block_scale_bytes.size());
+    }
+    std::vector<float> second(entry.second_level_scale_bytes.size() / 4);
+    if (!second.empty()) {
+        std::memcpy(second.data(), entry.second_level_scale_bytes.data(),
+                    entry.second_level_scale_bytes.size());
+    }
+    nf4o_scales scales{};
+    scales.encoding = entry.double_quantized ? 1 : 0;
+    scales.fp32_scales = fp32.data();
+    scales.fp32_count = fp32.size();
+    scales.quantized_scales = entry.scale_codes.data();
+    scales.quantized_count = entry.scale_codes.size();
+    scales.second_level = second.data();
+    scales.second_level_count = second.size();
+    scales.second_level_block = entry.scale_block_size;
+    scales.offset = entry.offset;
+    const char* message = "";
+    const int status = nf4o_validate_payload(
+        entry.shape[0] * entry.shape[1], entry.block_size,
+        entry.packed_codes.data(), entry.packed_codes.size(), &scales,
+        &message);
+    return status == NF4O_OK ? std::string() : std::string(message);
+}
+
+void test_packed_model_state() {
+    // Three weights as a model would hold them: fp32 scales with an odd
+    // element count, nested scales, and a larger nested one with whole zero
+    // rows (zero-scale blocks).
+    const HostWeight edge = quantize(edge_weight(), kEdgeWidth, kEdgeWidth, 32,
+                                     false, 32);
+    const HostWeight nested_edge = quantize(edge_weight(), kEdgeWidth,
+                                            kEdgeWidth, 32, true, 32);
+    std::vector<float> dense = pseudo_normal(96 * 256, 0.02F, 7);
+    std::fill(dense.begin() + 256, dense.begin() + 3 * 256, 0.0F);
+    const HostWeight zero_rows = quantize(dense, 96, 256, 64, false, 32);
+    const HostWeight nested_rows = quantize(dense, 96, 256, 64, true, 256);
+    const std::vector<const HostWeight*> weights{&edge, &nested_edge,
+                                                 &zero_rows, &nested_rows};
+    std::vector<std::unique_ptr<backend::QuantizedWeightStorage>> storages;
+    for (const HostWeight* weight : weights) {
+        storages.push_back(to_hip(*weight));
+    }
+
+    // copy -> load -> copy is byte-identical (tests/abi/test_c_api.c:3284-3302)
+    const std::vector<std::uint8_t> state = state_of(weights, storages);
+    const auto entries = backend::parse_packed_model_state(state);
+    require(entries.size() == weights.size(), "packed state entry count");
+    for (std::size_t index = 0; index < weights.size(); ++index) {
+        const HostWeight& weight = *weights[index];
+        const auto& entry = entries[index];
+        require(entry.shape == std::vector<std::size_t>{weight.output_width,
+                                                        weight.input_width} &&
+                    entry.block_size == weight.block_size,
+                "packed state shape and block size");
+        require(std::equal(entry.packed_codes.begin(),
+                           entry.packed_codes.end(), weight.codes.begin(),
+                           weight.codes.end()),
+                "packed state codes must be the stored bytes");
+        require(oracle_verdict(entry).empty(),
+                "a written state must hold canonical payloads");
+    }
+    auto loaded = backend::hip_load_packed_model_state(state);
+    require(loaded.size() == weights.size(), "loaded weight count");
+    std::vector<std::unique_ptr<backend::QuantizedWeightStorage>> restored;
+    for (std::size_t index = 0; index < loaded.size(); ++index) {
+        const HostWeight& weight = *weights[index];
+        require(loaded[index].shape ==
+                        std::vector<std::size_t>{weight.output_width,
+                                                 weight.input_width} &&
+                    loaded[index].block_size == weight.block_size,
+                "loaded shape and block size");
+        require(loaded[index].storage != nullptr &&
+                    loaded[index].storage->backend() == kHip,
+                "loaded storage must be hip storage");
+        require_byte_preserving(*loaded[index].storage, weight,
+                                "loaded packed state");
+        restored.push_back(std::move(loaded[index].storage));
+    }
+    require(state_of(weights, restored) == state,
+            "copy -> load -> copy must be byte-identical");
+
+    // a restored weight computes what the original does
+    const std::vector<float> input = edge_input();
+    require(hip_forward(input, *restored[1], nested_edge) ==
+                hip_forward(input, *storages[1], nested_edge),
+            "a restored weight must compute like the original");
+    require_close(hip_forward(input, *restored[0], edge),
+                  oracle_forward(input, edge), "restored forward");
+
+    // a truncated state is refused (tests/abi/test_c_api.c:3289-3293)
+    require_throws<std::invalid_argument>(
+        [&] {
+            static_cast<void>(backend::hip_load_packed_model_state(
+                std::span(state).first(state.size() - 1)));
+        },
+        "a truncated packed state must be refused",
+        "truncated packed model state");
+    require_throws<std::invalid_argument>(
+        [&] {
+            std::vector<std::uint8_t> other = state;
+            other[6] = '2';
+            static_cast<void>(backend::hip_load_packed_model_state(other));
+        },
+        "an unknown format must be refused",
+        "unknown packed model state format");
+
+    // Damaged payloads: the loader must throw std::invalid_argument with the
+    // message the oracle's require_canonical_payload gives for the same bytes.
+    // A patch overwrites bytes of one array of one entry: 0 codes, 1 block
+    // scales, 2 scale codes, 3 second-level scales, 4 the entry's header
+    // (offset in bytes from its start).
+    struct Patch {
+        std::size_t entry;
+        int array;
+        std::size_t offset;
+        std::vector<std::uint8_t> bytes;
+    };
+    struct Damage {
+        const char* name;
+        std::vector<Patch> patches;
+    };
+    const auto f32 = [](float value) {
+        std::vector<std::uint8_t> bytes(4);
+        std::memcpy(bytes.data(), &value, 4);
+        return bytes;
+    };
+    const auto u64 = [](std::uint64_t value) {
+        std::vector<std::uint8_t> bytes(8);
+        std::memcpy(bytes.data(), &value, 8);
+        return bytes;
+    };
+    const float infinity = std::numeric_limits<float>::infinity();
+    const float nan = std::numeric_limits<float>::quiet_NaN();
+    const std::vector<Damage> damages{
+        {"unused nibble", {{0, 0, edge.codes.size() - 1, {0xF7}}}},
+        {"negative scale", {{0, 1, 4 * 5, f32(-1.0F)}}},
+        {"infinite scale", {{0, 1, 4 * 30, f32(infinity)}}},
+        {"nan scale", {{2, 1, 4 * 100, f32(nan)}}},
+        {"zero block with a code", {{2, 0, 128 + 17, {0x78}}}},
+        {"zero block with a code, last byte", {{2, 0, 3 * 128 - 1, {0x87}}}},
+        {"zeroed scale of a used block", {{2, 1, 4 * 200, f32(0.0F)}}},
+        // the lowest offending block decides which rule is reported
+        {"bad scale below a bad zero block",
+         {{2, 1, 4 * 2, f32(-2.0F)}, {2, 0, 128 + 17, {0x78}}}},
+        {"bad zero block below a bad scale",
+         {{2, 1, 4 * 300, f32(-2.0F)}, {2, 0, 128 + 17, {0x78}}}},
+        // the unused nibble is reported before anything else
+        {"unused nibble and a bad scale",
+         {{0, 0, edge.codes.size() - 1, {0xF7}}, {0, 1, 0, f32(nan)}}},
+        {"nested: second-level nan", {{1, 3, 0, f32(nan)}}},
+        {"nested: second-level negative", {{3, 3, 0, f32(-1.0F)}}},
+        {"nested: offset infinite", {{1, 4, 56, f32(infinity)}}},
+        {"nested: offset negative", {{3, 4, 56, f32(-0.5F)}}},
+        {"nested: offset before second-level scales",
+         {{3, 4, 56, f32(nan)}, {3, 3, 0, f32(nan)}}},
+        {"nested: unused nibble",
+         {{1, 0, nested_edge.codes.size() - 1, {0xF7}}}},
+        {"block size", {{0, 4, 8, u64(48)}}},
+        {"second-level block size", {{1, 4, 48, u64(48)}}},
+        {"rows", {{2, 4, 64, u64(95)}}},
+        {"zero rows", {{2, 4, 64, u64(0)}}},
+        {"huge shape", {{2, 4, 64, u64(1ULL << 63)}}},
+        {"block size and scale count", {{2, 4, 8, u64(128)}}},
+    };
+    for (const Damage& damage : damages) {
+        std::vector<std::uint8_t> damaged = state;
+        for (const Patch& patch : damage.patches) {
+            const auto views = backend::parse_packed_model_state(damaged);
+            const auto& view = views[patch.entry];
+            const std::uint8_t* base = nullptr;
+            switch (patch.array) {
+            case 0: base = view.packed_codes.data(); break;
+            case 1: base = view.block_scale_bytes.data(); break;
+            case 2: base = view.scale_codes.data(); break;
+            case 3: base = view.second_level_scale_bytes.data(); break;
+            default:
+                // the entry's header starts 64 + 16 bytes before its codes
+                base = view.packed_codes.data() - 80;
+                break;
+            }
+            const std::size_t position =
+                static_cast<std::size_t>(base - damaged.data()) +
+                patch.offset;
+            std::copy(patch.bytes.begin(), patch.bytes.end(),
+                      damaged.begin() + static_cast<std::ptrdiff_t>(position));
+        }
+        // The expected outcome: the length rules first (host), then the
+        // oracle's verdict on the content.
+        std::string expected;
+        bool overflow = false;
+        const auto views = backend::parse_packed_model_state(damaged);
+        for (const auto& view : views) {
+            try {
+                static_cast<void>(backend::require_payload_lengths(view));
+            } catch (const std::overflow_error& error) {
+                expected = error.what();
+                overflow = true;
+            } catch (const std::invalid_argument& error) {
+                expected = error.what();
+            }
+            if (expected.empty()) {
+                expected = oracle_verdict(view);
+            }
+            if (!expected.empty()) {
+                break;
+            }
+        }
+        require(!expected.empty(),
+                std::string("damage must be detectable: ") + damage.name);
+        try {
+            static_cast<void>(backend::hip_load_packed_model_state(damaged));
+            throw std::runtime_error(std::string("damaged state accepted: ") +
+                                     damage.name);
+        } catch (const std::overflow_error& error) {
+            require(overflow && expected == error.what(),
+                    std::string(damage.name) + ": " + error.what() +
+                        " instead of " + expected);
+        } catch (const std::invalid_argument& error) {
+            require(!overflow && expected == error.what(),
+                    std::string(damage.name) + ": " + error.what() +
+                        " instead of " + expected);
+        }
+    }
+
+    // The committed fixture, which the reference's own reader accepted.
+    if (const char* golden = std::getenv("RIFTCO_TRANSFORMER_TEST_GOLDEN")) {
+        std::ifstream file(std::string(golden) + "/packed_state.bin",
+                           std::ios::binary);
+        require(file.good(), "tests/golden/packed_state.bin must be readable");
+        const std::vector<std::uint8_t> fixture(
+            (std::istreambuf_iterator<char>(file)),
+            std::istreambuf_iterator<char>());
+        auto golden_weights = backend::hip_load_packed_model_state(fixture);
+        require(golden_weights.size() == 3, "fixture weight count");
+        std::vector<backend::HipPackedWeightSource> sources;
+        for (const auto& weight : golden_weights) {
+            sources.push_back(
+                {weight.shape, weight.block_size, weight.storage.get()});
+        }
+        require(backend::hip_packed_model_state_bytes(sources) == fixture,
+                "the fixture must survive load -> copy byte for byte");
+        // its first two entries are the edge weight, as quantised above
+        require(std::equal(edge.codes.begin(), edge.codes.end(),
+                           golden_weights[0].storage->packed_codes().begin()),
+                "fixture codes must equal the oracle quantizer's");
+    }
+}
+
 void test_out_of_memory_maps_to_bad_alloc() {
     // Only the fake runtime can be told to fail an allocation.
     if (std::getenv("FAKE_RTHIP_CAN_FAIL") == nullptr) {
@@ -601,10 +883,39 @@ void test_out_of_memory_maps_to_bad_alloc() {
     unsetenv("FAKE_RTHIP_OUT_OF_MEMORY");
 }
 
+
+// One line per file: "ok <entries>", "ValueError <message>" or
+// "OverflowError <message>" -- the vocabulary of the Python oracle.
+int parse_states(int count, char** paths) {
+    for (int index = 0; index < count; ++index) {
+        std::ifstream file(paths[index], std::ios::binary);
+        if (!file.good()) {
+            std::cerr << "cannot read " << paths[index] << '\n';
+            return 1;
+        }
+        const std::vector<std::uint8_t> bytes(
+            (std::istreambuf_iterator<char>(file)),
+            std::istreambuf_iterator<char>());
+        try {
+            const std::size_t entries =
+                backend::parse_packed_model_state(bytes).size();
+            std::cout << "ok " << entries << '\n';
+        } catch (const std::invalid_argument& error) {
+            std::cout << "ValueError " << error.what() << '\n';
+        } catch (const std::overflow_error& error) {
+            std::cout << "OverflowError " << error.what() << '\n';
+        }
+    }
+    return 0;
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
     try {
+        if (argc >= 2 && std::string_view(argv[1]) == "--parse-state") {
+            return parse_states(argc - 2, argv + 2);
+        }
         const bool expect_unavailable =
             argc == 2 && std::string_view(argv[1]) == "--expect-unavailable";
         if (argc > 2 || (argc == 2 && !expect_unavailable)) {
@@ -638,6 +949,7 @@ int main(int argc, char** argv) {
         test_transformer_sized_layer();
         test_tensor_storage();
         test_dispatch_validation();
+        test_packed_model_state();
         test_out_of_memory_maps_to_bad_alloc();
         std::cout << "hip backend tests passed\n";
         return 0;

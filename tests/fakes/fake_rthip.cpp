@@ -375,4 +375,30 @@ rthip_status rthip_nf4_quantize(
     return RTHIP_OK;
 }
 
+rthip_status rthip_nf4_check_payload(
+    const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, uint64_t element_count,
+    uint64_t block_size, void*) {
+    if (codes == nullptr || element_count == 0 ||
+        !supported_block(block_size)) {
+        return fail(RTHIP_INVALID_ARGUMENT, "invalid payload description");
+    }
+    const size_t blocks = (element_count + block_size - 1) / block_size;
+    nf4o_scales scales;
+    if (const rthip_status status =
+            make_scales(primary_scales, secondary_scales, encoding,
+                        second_level_block, offset, blocks, &scales);
+        status != RTHIP_OK) {
+        return status;
+    }
+    const char* message = "";
+    if (nf4o_validate_payload(element_count, block_size, codes,
+                              (element_count + 1) / 2, &scales,
+                              &message) != NF4O_OK) {
+        return fail(RTHIP_INVALID_ARGUMENT, message);
+    }
+    return RTHIP_OK;
+}
+
 }  // extern "C"

@@ -24,6 +24,7 @@ CONFORMANCE = os.path.join(BUILD, "test_in_tree_conformance")
 def run(arguments=(), **environment):
     env = {k: v for k, v in os.environ.items()
            if not k.startswith(("RIFTCO_TRANSFORMER_", "FAKE_RTHIP_"))}
+    env["RIFTCO_TRANSFORMER_TEST_GOLDEN"] = os.path.join(HERE, "golden")
     env.update(environment)
     assert os.path.exists(BINARY), \
         "tests/cpp/build/test_hip_backend is not built (make -C tests/cpp)"
@@ -57,6 +58,33 @@ def test_adapter_keeps_a_counted_mirror_without_host_visible_memory():
     expect_pass(run(RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE,
                     RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1",
                     FAKE_RTHIP_NO_BAR="1"))
+
+
+def test_packed_state_reader_fails_as_the_reference_reader_does(tmp_path):
+    """The adapter's reader of the packed model state on every malformed
+    variant of the fixture: outcome and message must be the ones the
+    reference's compiled reader gave (tests/golden/make_golden.py)."""
+    import json
+    import helpers
+    golden = os.path.join(HERE, "golden")
+    with open(os.path.join(golden, "packed_state.bin"), "rb") as handle:
+        blob = handle.read()
+    with open(os.path.join(golden, "packed_state_outcomes.json")) as handle:
+        expected = json.load(handle)
+    cases = helpers.packed_state_mutations(blob)
+    paths = []
+    for name, data in cases:
+        path = tmp_path / name
+        path.write_bytes(data)
+        paths.append(str(path))
+    result = run(["--parse-state", *paths])
+    assert result.returncode == 0, result.stdout + result.stderr
+    lines = result.stdout.splitlines()
+    assert len(lines) == len(cases)
+    for (name, _), line in zip(cases, lines):
+        kind, _, rest = line.partition(" ")
+        want = expected[name]
+        assert [kind, rest] == [want[0], str(want[1])], name
 
 
 def test_unavailable_when_the_runtime_sees_no_device():

@@ -645,3 +645,114 @@ def test_memory_entry_points(gpu, package, library):
     library.free(pointer)
     assert "MI355X" in library.device_description() or \
         "gfx950" in library.device_description()
+
+
+# ---- content rules of a canonical payload, checked on the device -----------
+
+def verdict(function, *arguments):
+    try:
+        function(*arguments)
+        return ""
+    except ValueError as error:
+        # the library's message without the binding's "rthip status N: "
+        return getattr(error, "message", str(error))
+
+
+def damaged_payloads(oracle):
+    """(name, weight) pairs: valid payloads and payloads that break one or
+    several rules of require_canonical_payload, in places chosen so that the
+    rule the reference reports first differs from case to case."""
+    import copy
+    dense = helpers.normal(150, (300, 1000), 0.02)
+    dense[3:5] = 0.0                      # whole zero blocks
+    dense.ravel()[-1] = 0.01
+    plain = oracle.quantize(dense, 64, False, 256)
+    nested = oracle.quantize(dense, 64, True, 256)
+    odd = oracle.quantize(helpers.normal(151, (33, 33), 0.02), 32, False, 32)
+    odd_nested = oracle.quantize(helpers.normal(151, (33, 33), 0.02), 32,
+                                 True, 32)
+    zero_block = 3 * 1000 // 64 + 1       # a block inside the zero rows
+    cases = [("plain", plain), ("nested", nested), ("odd", odd),
+             ("odd nested", odd_nested)]
+
+    def changed(name, base, **edits):
+        weight = copy.deepcopy(base)
+        for field, (index, value) in edits.items():
+            if field == "offset":
+                weight.offset = value
+            else:
+                getattr(weight, field)[index] = value
+        cases.append((name, weight))
+
+    changed("unused nibble", odd, codes=(-1, 0xF7))
+    changed("unused nibble nested", odd_nested, codes=(-1, 0x17))
+    changed("negative scale", plain, fp32_scales=(17, -1.0))
+    changed("infinite scale", plain, fp32_scales=(4000, np.inf))
+    changed("nan scale at the end", plain, fp32_scales=(-1, np.nan))
+    changed("negative zero scale is a zero scale", plain,
+            fp32_scales=(zero_block, -0.0))
+    changed("code in a zero block", plain, codes=(zero_block * 32 + 5, 0x70))
+    changed("code in a zero block, first byte", plain,
+            codes=(zero_block * 32, 0x87))
+    changed("zeroed scale of a used block", plain, fp32_scales=(2000, 0.0))
+    changed("zero block below a bad scale", plain,
+            codes=(zero_block * 32 + 5, 0x70), fp32_scales=(3000, -1.0))
+    changed("bad scale below a zero block", plain,
+            codes=(zero_block * 32 + 5, 0x70), fp32_scales=(2, np.nan))
+    changed("nibble before everything", odd, codes=(-1, 0xF7),
+            fp32_scales=(0, np.nan))
+    changed("nested tolerates codes under a zero scale", nested,
+            codes=(zero_block * 32 + 5, 0x70))
+    changed("second-level nan", nested, second_level=(3, np.nan))
+    changed("second-level negative", nested, second_level=(-1, -1.0e-3))
+    changed("second-level infinite", nested, second_level=(0, np.inf))
+    changed("offset nan", nested, offset=(None, float("nan")))
+    changed("offset negative", nested, offset=(None, -1.0))
+    changed("offset before second-level", nested, offset=(None, float("inf")),
+            second_level=(0, np.nan))
+    # a huge second-level scale saturates the decoded scale instead of
+    # overflowing it, which the rules accept
+    changed("saturating second-level scale", nested,
+            second_level=(1, np.float32(3.0e38)))
+    return cases
+
+
+def test_device_payload_check_follows_the_reference_rules(gpu, package,
+                                                          library, oracle):
+    """rthip_nf4_check_payload accepts and refuses exactly what the oracle's
+    require_canonical_payload does, with the same message."""
+    seen = set()
+    for name, weight in damaged_payloads(oracle):
+        expected = verdict(oracle.validate_payload, weight)
+        got = verdict(gpu.check_payload, upload(gpu, weight))
+        assert got == expected, f"{name}: {got!r} instead of {expected!r}"
+        seen.add(expected)
+    assert len(seen) == 6, seen   # valid + the five content rules
+
+
+def test_device_payload_check_on_a_transformer_layer(gpu, package, library,
+                                                     oracle):
+    """A full 11008 x 4096 layer: valid as quantised on the device, refused
+    after one byte of a zero block or one scale is damaged."""
+    import torch
+    dense = helpers.normal(152, (11008, 4096), 0.02)
+    dense[100] = 0.0
+    for nested in (False, True):
+        weight = gpu.quantize_weight(to_device(dense), 64, nested, 256)
+        gpu.check_payload(weight)
+        if nested:
+            weight.secondary_scales[-1] = float("nan")
+            torch.cuda.synchronize()
+            assert verdict(gpu.check_payload, weight) == \
+                "NF4 second-level scales must be finite and nonnegative"
+        else:
+            weight.codes[100 * 2048 + 77] = 0x72
+            torch.cuda.synchronize()
+            assert verdict(gpu.check_payload, weight) == \
+                "zero-scale NF4 blocks must use canonical zero code 7"
+            weight.primary_scales[-1] = -1.0
+            assert verdict(gpu.check_payload, weight) == \
+                "zero-scale NF4 blocks must use canonical zero code 7"
+            weight.codes[100 * 2048 + 77] = 0x77
+            assert verdict(gpu.check_payload, weight) == \
+                "NF4 block scales must be finite and nonnegative"
