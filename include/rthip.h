@@ -80,7 +80,10 @@ enum {
     RTHIP_NF4_ALGORITHM_MFMA = 3,
     /* small batches (forward, up to 64 rows): weights decoded straight into
      * MFMA operands, no LDS tile */
-    RTHIP_NF4_ALGORITHM_SKINNY = 4
+    RTHIP_NF4_ALGORITHM_SKINNY = 4,
+    /* up to 16 rows (forward) with a row width of 1024..4096: like SKINNY, but
+     * x stays in registers and the wavefronts split the contraction axis */
+    RTHIP_NF4_ALGORITHM_RESIDENT = 5
 };
 
 /* ---- library / device ------------------------------------------------- */

@@ -10,6 +10,7 @@ from .binding import (  # noqa: F401
     ALGORITHM_GENERIC,
     ALGORITHM_MFMA,
     ALGORITHM_NAMES,
+    ALGORITHM_RESIDENT,
     ALGORITHM_SKINNY,
     EXPORTED_SYMBOLS,
     FORWARD,

@@ -31,8 +31,9 @@ ALGORITHM_GENERIC = 1
 ALGORITHM_GEMV = 2
 ALGORITHM_MFMA = 3
 ALGORITHM_SKINNY = 4
+ALGORITHM_RESIDENT = 5
 ALGORITHM_NAMES = {0: "auto", 1: "generic", 2: "gemv", 3: "mfma",
-                   4: "skinny"}
+                   4: "skinny", 5: "resident"}
 
 FORWARD = 0
 INPUT_BACKWARD = 1

@@ -1,0 +1,373 @@
+// Forward product for up to 16 rows when a row of the weight is short enough
+// for x to live in registers (row width 1024, 2048, 3072 or 4096):
+//     y[r, o] = sum_i x[r, i] * codebook[code(o, i)] * scale(o, i / B)
+// restating reference_quantized_linear_forward
+// (src/core/backend/nn/quantized_linear/reference/operations.cpp:49-81).
+//
+// The small-batch kernel of nf4_skinny.hip stages x through LDS slab by slab,
+// which costs two workgroup barriers per 256 contraction values; with 16 rows
+// those barriers and the copies take longer than the matrix instructions.
+// Here the contraction axis is cut ACROSS the eight wavefronts of a workgroup
+// instead: wavefront w owns contraction values [w I/8, (w+1) I/8) of every
+// weight row, its 16 x I/8 slice of x is loaded into registers once (I/32
+// values per lane, at most 128; coalesced loads passed through a per-wavefront
+// LDS area) and stays there, and a workgroup streams 16-row tiles of the weight
+// with no barrier and no LDS traffic for x in the loop -- the structure of the
+// GEMV, with matrix instructions instead of lane sums.  What it pays for this
+// is that every workgroup reads all of x (256 KB for 16 x 4096) once.
+//
+//   * v_mfma_f32_16x16x4_f32: A is x[16 rows][4 k], B is W^T[4 k][16 weight
+//     rows].  Lane l supplies x row l % 16, weight row l % 16 and contraction
+//     quarter q = l / 16.  The 128 values of contraction group g of a wavefront
+//     are dealt to the quarters in runs of 32: lane (n, q) owns
+//         k = w I/8 + 128 g + 32 q + [0, 32)
+//     of weight row n (one 16-byte load; the four lanes of a row read 64
+//     contiguous bytes) and the same k of x row n.  Any assignment of k to
+//     (quarter, instruction) is valid as long as A and B agree.
+//   * Decode as everywhere: a code byte indexes the replicated pair table in
+//     LDS (one v_perm_b32 + one ds_read_b64 per two weights), each level times
+//     its block scale in one rounded multiply.  The lookups of the next 16
+//     weights are issued before the 16 matrix instructions of the current
+//     ones.
+//   * Tiles are dealt round-robin to one persistent workgroup per compute
+//     unit; the codes of tile t + 1 are requested before tile t is computed.
+//   * A wavefront parks its 16 x 16 partial tile in LDS; after the ONLY
+//     barrier, at the end of the kernel, the workgroup adds the eight partial
+//     tiles of each of its output tiles in wavefront order and writes y with
+//     bias and adapter term.  Nothing depends on scheduling.
+
+#include "kernels.hpp"
+#include "nf4_decode.hpp"
+#include "nf4_pair_table.hpp"
+
+namespace rthip {
+namespace {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 512;
+constexpr int kWaves = 8;
+constexpr int kTileRows = 16;        // weight rows per tile
+constexpr int kGroupWeights = 128;   // contraction values per wavefront group
+constexpr int kLaneWeights = 32;     // of which one lane owns this many
+constexpr unsigned kComputeUnits = 256;
+constexpr unsigned kMaxIterations = 8;  // tiles one workgroup may park
+// Per-wavefront LDS area that x passes through on its way into registers:
+// [16 rows][128 values], rows padded by four floats.
+constexpr unsigned kStagingStride = kGroupWeights + 4;
+constexpr unsigned kStagingFloats = kTileRows * kStagingStride;
+constexpr std::size_t kStagingBytes =
+    static_cast<std::size_t>(kWaves) * kStagingFloats * sizeof(float);
+constexpr unsigned kRejectedOffset = 0x80000000U;  // fails every range check
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_buffer(const void* base,
+                                                            std::size_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+// kGroups: contraction groups per wavefront; the row width is 1024 * kGroups.
+template <int kGroups, bool kDoubleQuantized>
+__global__ __launch_bounds__(kThreads) void resident_forward_kernel(
+    const float* __restrict__ x, Nf4WeightView weight,
+    const float* __restrict__ bias, float* __restrict__ y, unsigned rows,
+    unsigned output_width, unsigned block_shift, unsigned tile_count,
+    unsigned iterations, LoraEpilogue lora
+) {
+    constexpr unsigned kInputWidth = 1024U * kGroups;
+    constexpr int kSubChunks = 2 * kGroups;  // 16 weights each
+    extern __shared__ __attribute__((aligned(256))) char shared[];
+    char* table = shared;  // kPairTableBytes
+    // parked[iteration][wavefront][lane]: accumulator of that lane
+    floatx4* parked = reinterpret_cast<floatx4*>(shared + kPairTableBytes);
+
+    const unsigned thread = threadIdx.x;
+    const unsigned lane = thread % 64;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(thread / 64);
+    const unsigned quarter = lane / 16;
+    const unsigned lane_row = lane % 16;
+    // first contraction value of this lane in group 0
+    const unsigned k_base =
+        wave * (kInputWidth / kWaves) + quarter * kLaneWeights;
+
+    const std::size_t elements =
+        static_cast<std::size_t>(output_width) * kInputWidth;  // < 2^32
+    const std::size_t block_total =
+        (elements + (std::size_t{1} << block_shift) - 1) >> block_shift;
+    const __amdgpu_buffer_rsrc_t x_buffer = raw_buffer(
+        x, static_cast<std::size_t>(rows) * kInputWidth * sizeof(float));
+    const __amdgpu_buffer_rsrc_t code_buffer =
+        raw_buffer(weight.codes, elements / 2);
+    const __amdgpu_buffer_rsrc_t primary_buffer = raw_buffer(
+        weight.primary_scales, block_total * (kDoubleQuantized ? 1 : 4));
+    const __amdgpu_buffer_rsrc_t secondary_buffer = raw_buffer(
+        weight.secondary_scales,
+        kDoubleQuantized
+            ? (((block_total - 1) >> weight.second_level_shift) + 1) * 4
+            : 0);
+
+    struct Codes {
+        uintx4 codes[kGroups];  // 32 nibbles each
+        float scales[kGroups];
+    };
+    // Tiles past the workgroup's last one, and weight rows past the output
+    // width, read as zeros.
+    const auto load_codes = [&](Codes& staged, unsigned tile) {
+        const unsigned n = tile * kTileRows + lane_row;
+        const bool valid = tile < tile_count && n < output_width;
+        const unsigned flat = n * kInputWidth + k_base;
+#pragma unroll
+        for (int g = 0; g < kGroups; ++g) {
+            const unsigned first = flat + kGroupWeights * g;
+            staged.codes[g] = __builtin_bit_cast(
+                uintx4,
+                __builtin_amdgcn_raw_buffer_load_b128(
+                    code_buffer, valid ? first >> 1 : kRejectedOffset, 0, 0));
+            const unsigned block = first >> block_shift;
+            if constexpr (!kDoubleQuantized) {
+                staged.scales[g] = __builtin_bit_cast(
+                    float, __builtin_amdgcn_raw_buffer_load_b32(
+                               primary_buffer,
+                               valid ? block * 4 : kRejectedOffset, 0, 0));
+            } else {
+                const std::uint8_t scale_code =
+                    __builtin_amdgcn_raw_buffer_load_b8(
+                        primary_buffer, valid ? block : kRejectedOffset, 0, 0);
+                const float second = __builtin_bit_cast(
+                    float,
+                    __builtin_amdgcn_raw_buffer_load_b32(
+                        secondary_buffer,
+                        valid ? (block >> weight.second_level_shift) * 4
+                              : kRejectedOffset,
+                        0, 0));
+                // Lanes with nothing to read decode (0, 0.0) into the
+                // offset: finite, and never written.
+                staged.scales[g] = decode_double_quantized_scale(
+                    scale_code, second, weight.offset);
+            }
+        }
+    };
+
+    // Tiles are dealt round-robin: iteration i of workgroup b takes tile
+    // b + i * gridDim.x.
+    Codes ring[2];
+    load_codes(ring[0], blockIdx.x);
+
+    // This lane's slice of x: row lane % 16, resident for the whole kernel.
+    // A lane's values are 128 contiguous bytes of one x row, and the 16 rows
+    // of a wavefront lie a whole row apart, so loading them directly would
+    // touch 64 cache lines per instruction.  Each wavefront therefore reads
+    // its [16 rows][128] piece of group g with coalesced loads (two x rows per
+    // instruction, 512 contiguous bytes each), passes it through a private
+    // LDS area and picks up its own values from there.  Rows past `rows` read
+    // as zero.
+    float* staging =
+        reinterpret_cast<float*>(shared + kPairTableBytes) + wave * kStagingFloats;
+    float xs[kGroups][kLaneWeights];
+    {
+        // chunk c = lane + 64 j of the piece: row c / 32, floats 4 (c % 32)
+        const unsigned piece_row = lane / 32;
+        const unsigned piece_column = (lane % 32) * 4;
+        const auto load_piece = [&](floatx4 (&piece)[8], int g) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const unsigned row = piece_row + 2 * j;
+                piece[j] = __builtin_bit_cast(
+                    floatx4,
+                    __builtin_amdgcn_raw_buffer_load_b128(
+                        x_buffer,
+                        row < rows
+                            ? (row * kInputWidth +
+                               wave * (kInputWidth / kWaves) +
+                               kGroupWeights * g + piece_column) *
+                                  static_cast<unsigned>(sizeof(float))
+                            : kRejectedOffset,
+                        0, 0));
+            }
+        };
+        floatx4 pieces[2][8];
+        load_piece(pieces[0], 0);
+#pragma unroll
+        for (int g = 0; g < kGroups; ++g) {
+            if (g + 1 < kGroups) {
+                load_piece(pieces[(g + 1) % 2], g + 1);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                *reinterpret_cast<floatx4*>(
+                    staging + (piece_row + 2 * j) * kStagingStride +
+                    piece_column) = pieces[g % 2][j];
+            }
+            // (LDS operations of one wavefront complete in order)
+#pragma unroll
+            for (int v = 0; v < kLaneWeights / 4; ++v) {
+                const floatx4 values = *reinterpret_cast<const floatx4*>(
+                    staging + lane_row * kStagingStride +
+                    quarter * kLaneWeights + 4 * v);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    xs[g][4 * v + e] = values[e];
+                }
+            }
+        }
+    }
+
+    build_pair_table<kThreads>(table);
+    const unsigned lane_bits = pair_table_lane_bits(lane);
+    // The table is built, and every wavefront is done with its staging area,
+    // which the parked tiles reuse.
+    __syncthreads();
+
+    // Sub-chunk s of a tile: 16 weights = two code words of group s / 2.
+    float2 raw[8];
+    const auto issue_lookups = [&](const Codes& codes, int s) {
+        const unsigned words[2] = {codes.codes[s / 2][2 * (s % 2)],
+                                   codes.codes[s / 2][2 * (s % 2) + 1]};
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+            for (int byte = 0; byte < 4; ++byte) {
+                raw[4 * half + byte] =
+                    pair_table_lookup(table, words[half], byte, lane_bits);
+            }
+        }
+    };
+
+    const auto compute = [&](const Codes& current, const Codes& next,
+                             unsigned iteration) {
+        floatx4 acc = {0.0F, 0.0F, 0.0F, 0.0F};
+#pragma unroll
+        for (int s = 0; s < kSubChunks; ++s) {
+            float w[16];
+            {
+#pragma clang fp contract(off)
+                const float scale = current.scales[s / 2];
+#pragma unroll
+                for (int p = 0; p < 8; ++p) {
+                    w[2 * p] = raw[p].x * scale;
+                    w[2 * p + 1] = raw[p].y * scale;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (s + 1 < kSubChunks) {
+                issue_lookups(current, s + 1);
+            } else {
+                issue_lookups(next, 0);  // the next tile's first
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                    xs[s / 2][16 * (s % 2) + i], w[i], acc, 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        parked[(iteration * kWaves + wave) * 64 + lane] = acc;
+    };
+
+    issue_lookups(ring[0], 0);
+    for (unsigned iteration = 0; iteration < iterations; iteration += 2) {
+        load_codes(ring[1], blockIdx.x + (iteration + 1) * gridDim.x);
+        compute(ring[0], ring[1], iteration);
+        if (iteration + 1 < iterations) {  // uniform
+            load_codes(ring[0], blockIdx.x + (iteration + 2) * gridDim.x);
+            compute(ring[1], ring[0], iteration + 1);
+        }
+    }
+
+    // The only barrier after the table build.  Accumulator element r of lane
+    // l is x row 4 (l / 16) + r and weight row l % 16 of the tile.
+    __syncthreads();
+    for (unsigned index = thread; index < iterations * 256; index += kThreads) {
+        const unsigned iteration = index / 256;
+        const unsigned m = (index % 256) / 16;
+        const unsigned column = index % 16;
+        const unsigned tile = blockIdx.x + iteration * gridDim.x;
+        const unsigned n = tile * kTileRows + column;
+        if (tile >= tile_count || n >= output_width || m >= rows) {
+            continue;
+        }
+        const float* source = reinterpret_cast<const float*>(
+                                  parked + iteration * kWaves * 64 +
+                                  (m / 4) * 16 + column) +
+                              m % 4;
+        float sum = 0.0F;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            sum += source[w * 64 * 4];  // wavefront order
+        }
+        if (bias != nullptr) {
+            sum += bias[n];
+        }
+        if (lora.reduced != nullptr) {
+            sum += lora_term(lora, m, n);
+        }
+        y[static_cast<std::size_t>(m) * output_width + n] = sum;
+    }
+}
+
+template <int kGroups, bool kDoubleQuantized>
+hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
+    const unsigned tiles = static_cast<unsigned>(
+        (p.output_width + kTileRows - 1) / kTileRows);
+    // One workgroup per compute unit, more only if a workgroup would
+    // otherwise have to park more tiles than it has room for.
+    unsigned groups = tiles < kComputeUnits ? tiles : kComputeUnits;
+    unsigned iterations = (tiles + groups - 1) / groups;
+    if (iterations > kMaxIterations) {
+        iterations = kMaxIterations;
+        groups = (tiles + iterations - 1) / iterations;
+    }
+    const std::size_t parked_bytes =
+        static_cast<std::size_t>(iterations) * kWaves * 64 * sizeof(floatx4);
+    const std::size_t shared_bytes =
+        kPairTableBytes +
+        (parked_bytes > kStagingBytes ? parked_bytes : kStagingBytes);
+    const auto kernel = resident_forward_kernel<kGroups, kDoubleQuantized>;
+    // More than the default 64 KB of LDS.
+    static const hipError_t configured = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel),
+        hipFuncAttributeMaxDynamicSharedMemorySize,
+        static_cast<int>(kPairTableBytes + kStagingBytes));
+    static_assert(kStagingBytes >=
+                  kMaxIterations * kWaves * 64 * sizeof(floatx4));
+    if (configured != hipSuccess) {
+        return configured;
+    }
+    kernel<<<groups, kThreads, shared_bytes, stream>>>(
+        p.activations, p.weight, p.bias, p.result,
+        static_cast<unsigned>(p.rows), static_cast<unsigned>(p.output_width),
+        p.block_shift, tiles, iterations, p.lora);
+    return hipSuccess;
+}
+
+template <int kGroups>
+hipError_t launch_groups(const LinearProblem& p, hipStream_t stream) {
+    return p.weight.encoding == 0 ? launch_instance<kGroups, false>(p, stream)
+                                  : launch_instance<kGroups, true>(p, stream);
+}
+
+}  // namespace
+
+bool resident_forward_supports(const LinearProblem& p) {
+    return p.rows >= 1 && p.rows <= kResidentMaxRows &&
+           p.input_width % 1024 == 0 && p.input_width <= 4096 &&
+           // 32-bit flat weight indices; byte offsets into x, the codes and
+           // the scales all stay below the rejected offset
+           p.output_width * p.input_width < (1ULL << 32) &&
+           reinterpret_cast<std::uintptr_t>(p.weight.codes) % 16 == 0 &&
+           reinterpret_cast<std::uintptr_t>(p.activations) % 16 == 0;
+}
+
+hipError_t launch_resident_forward(const LinearProblem& p,
+                                   hipStream_t stream) {
+    switch (p.input_width / 1024) {
+    case 1: return launch_groups<1>(p, stream);
+    case 2: return launch_groups<2>(p, stream);
+    case 3: return launch_groups<3>(p, stream);
+    default: return launch_groups<4>(p, stream);
+    }
+}
+
+}  // namespace rthip

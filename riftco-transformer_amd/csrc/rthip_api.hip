@@ -180,6 +180,10 @@ int32_t select_forward(const rthip::LinearProblem& problem) {
         rthip::gemv_forward_supports(problem)) {
         return RTHIP_NF4_ALGORITHM_GEMV;
     }
+    if (problem.rows <= rthip::kResidentMaxRows &&
+        rthip::resident_forward_supports(problem)) {
+        return RTHIP_NF4_ALGORITHM_RESIDENT;
+    }
     if (problem.rows <= rthip::kSkinnyMaxRows &&
         rthip::skinny_forward_supports(problem)) {
         return RTHIP_NF4_ALGORITHM_SKINNY;
@@ -441,6 +445,19 @@ rthip_status linear_forward_common(
             return from_hip(status, "small-batch workspace allocation");
         }
         break;
+    case RTHIP_NF4_ALGORITHM_RESIDENT:
+        if (!rthip::resident_forward_supports(problem)) {
+            return fail(RTHIP_UNSUPPORTED,
+                        "the resident family needs rows <= %zu, a row width "
+                        "of 1024, 2048, 3072 or 4096 and aligned pointers",
+                        rthip::kResidentMaxRows);
+        }
+        if (const hipError_t status =
+                rthip::launch_resident_forward(problem, hip_stream);
+            status != hipSuccess) {
+            return from_hip(status, "resident kernel configuration");
+        }
+        break;
     default:
         return fail(RTHIP_INVALID_ARGUMENT, "unknown algorithm %d",
                     static_cast<int>(algorithm));
@@ -677,6 +694,7 @@ rthip_status rthip_nf4_linear_input_backward_with(
         break;
     case RTHIP_NF4_ALGORITHM_GEMV:
     case RTHIP_NF4_ALGORITHM_SKINNY:
+    case RTHIP_NF4_ALGORITHM_RESIDENT:
         return fail(RTHIP_UNSUPPORTED,
                     "this family implements the forward product only");
     default:

@@ -49,7 +49,8 @@ def families(package):
     """AUTO plus every pinned kernel family; a family that does not accept a
     shape answers RTHIP_UNSUPPORTED and is skipped by `run`."""
     return (None, package.ALGORITHM_GENERIC, package.ALGORITHM_GEMV,
-            package.ALGORITHM_MFMA, package.ALGORITHM_SKINNY)
+            package.ALGORITHM_MFMA, package.ALGORITHM_SKINNY,
+            package.ALGORITHM_RESIDENT)
 
 
 def run(package, function, *args, algorithm):
@@ -267,6 +268,32 @@ def test_small_batch_work_split(gpu, package, library, oracle, out_w, in_w,
         dy = helpers.normal(68 + rows, (rows, out_w), 1.0e-2)
         check_layer(gpu, package, library, oracle, weight, x, dy, bias=bias,
                     oracle_rows=min(rows, 5))
+
+
+@pytest.mark.parametrize("out_w,in_w,block,second,double_quantized", [
+    (4096, 4096, 64, 256, False),   # one tile per workgroup
+    (11008, 4096, 64, 256, True),   # two or three tiles per workgroup
+    (1000, 3072, 32, 32, True),     # block size 32, last tile partly empty
+    (33, 2048, 128, 64, False),     # fewer tiles than compute units
+    (530, 1024, 4096, 32, False),   # a quantisation block spans four rows
+    (40000, 1024, 64, 64, True),    # more than eight tiles per compute unit
+])
+def test_resident_small_batch_family(gpu, package, library, oracle, out_w,
+                                     in_w, block, second, double_quantized):
+    """Up to 16 rows with x resident in registers: every row count from the
+    GEMV's to the family's limit, with bias, against the oracle, fp64 and the
+    other families (check_layer runs each that accepts the shape)."""
+    dense = helpers.normal(73, (out_w, in_w), 0.02)
+    dense[1] = 0.0
+    weight = oracle.quantize(dense, block, double_quantized, second)
+    assert library.select_algorithm(package.FORWARD, 16, in_w, out_w,
+                                    block) == package.ALGORITHM_RESIDENT
+    bias = helpers.normal(74, (out_w,), 0.01)
+    for rows in (1, 5, 11, 16):
+        x = helpers.normal(75 + rows, (rows, in_w), 1.0)
+        dy = helpers.normal(76 + rows, (rows, out_w), 1.0e-2)
+        check_layer(gpu, package, library, oracle, weight, x, dy, bias=bias,
+                    oracle_rows=min(rows, 3))
 
 
 def test_zero_scale_blocks_and_saturated_scales(gpu, package, library,
