@@ -77,10 +77,13 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
 ) {
     constexpr unsigned kInputWidth = 1024U * kGroups;
     constexpr int kSubChunks = 2 * kGroups;  // 16 weights each
+    // The table is a static array so that its LDS address is a compile-time
+    // constant (zero) that folds into the lookups; the rest is sized at
+    // launch.
+    __shared__ __attribute__((aligned(256))) char table[kPairTableBytes];
     extern __shared__ __attribute__((aligned(256))) char shared[];
-    char* table = shared;  // kPairTableBytes
     // parked[iteration][wavefront][lane]: accumulator of that lane
-    floatx4* parked = reinterpret_cast<floatx4*>(shared + kPairTableBytes);
+    floatx4* parked = reinterpret_cast<floatx4*>(shared);
 
     const unsigned thread = threadIdx.x;
     const unsigned lane = thread % 64;
@@ -163,7 +166,7 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
     // LDS area and picks up its own values from there.  Rows past `rows` read
     // as zero.
     float* staging =
-        reinterpret_cast<float*>(shared + kPairTableBytes) + wave * kStagingFloats;
+        reinterpret_cast<float*>(shared) + wave * kStagingFloats;
     float xs[kGroups][kLaneWeights];
     {
         // chunk c = lane + 64 j of the piece: row c / 32, floats 4 (c % 32)
@@ -186,18 +189,21 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
                         0, 0));
             }
         };
-        floatx4 pieces[2][8];
-        load_piece(pieces[0], 0);
+        // All pieces are requested at once (their registers are free until
+        // xs fills up), so the slice costs one round trip to L2, not one per
+        // group.
+        floatx4 pieces[kGroups][8];
 #pragma unroll
         for (int g = 0; g < kGroups; ++g) {
-            if (g + 1 < kGroups) {
-                load_piece(pieces[(g + 1) % 2], g + 1);
-            }
+            load_piece(pieces[g], g);
+        }
+#pragma unroll
+        for (int g = 0; g < kGroups; ++g) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 *reinterpret_cast<floatx4*>(
                     staging + (piece_row + 2 * j) * kStagingStride +
-                    piece_column) = pieces[g % 2][j];
+                    piece_column) = pieces[g][j];
             }
             // (LDS operations of one wavefront complete in order)
 #pragma unroll
@@ -322,14 +328,13 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     const std::size_t parked_bytes =
         static_cast<std::size_t>(iterations) * kWaves * 64 * sizeof(floatx4);
     const std::size_t shared_bytes =
-        kPairTableBytes +
-        (parked_bytes > kStagingBytes ? parked_bytes : kStagingBytes);
+        parked_bytes > kStagingBytes ? parked_bytes : kStagingBytes;
     const auto kernel = resident_forward_kernel<kGroups, kDoubleQuantized>;
     // More than the default 64 KB of LDS.
     static const hipError_t configured = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kernel),
         hipFuncAttributeMaxDynamicSharedMemorySize,
-        static_cast<int>(kPairTableBytes + kStagingBytes));
+        static_cast<int>(kStagingBytes));
     static_assert(kStagingBytes >=
                   kMaxIterations * kWaves * 64 * sizeof(floatx4));
     if (configured != hipSuccess) {

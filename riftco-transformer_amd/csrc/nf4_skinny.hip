@@ -97,9 +97,12 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
     constexpr int kRows = 16 * kBlocks;
     // float4 copies per thread to move one x tile
     constexpr int kCopies = kRows * (kSlab / 4) / kThreads;  // 2 * kBlocks
+    // The table is a static array so that its LDS address is a compile-time
+    // constant (zero) that folds into the lookups; the x tile is sized at
+    // launch.
+    __shared__ __attribute__((aligned(256))) char table[kPairTableBytes];
     extern __shared__ __attribute__((aligned(256))) char shared[];
-    char* table = shared;  // kPairTableBytes
-    float* x_tile = reinterpret_cast<float*>(shared + kPairTableBytes);
+    float* x_tile = reinterpret_cast<float*>(shared);
 
     const unsigned thread = threadIdx.x;
     const unsigned lane = thread % 64;
@@ -482,7 +485,6 @@ static_assert(kWorkspaceBytes <= kStreamWorkspaceBytes);
 template <int kBlocks, int kScales, bool kDoubleQuantized>
 hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     constexpr std::size_t kSharedBytes =
-        kPairTableBytes +
         static_cast<std::size_t>(16 * kBlocks) * kStride * sizeof(float);
     const auto kernel =
         skinny_forward_kernel<kBlocks, kScales, kDoubleQuantized>;
