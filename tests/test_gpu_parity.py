@@ -783,3 +783,62 @@ def test_device_payload_check_on_a_transformer_layer(gpu, package, library,
             weight.codes[100 * 2048 + 77] = 0x77
             assert verdict(gpu.check_payload, weight) == \
                 "NF4 block scales must be finite and nonnegative"
+
+
+# ---- replay from a HIP graph ----------------------------------------------
+
+def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
+    """A decode loop is launch-bound and runs from a HIP graph (the benchmark
+    does).  One graph holds a launch of every forward family, the partial-tile
+    path of the small-batch family with its second kernel and workspace, the
+    adapter epilogue and the input backward; each of several replays, with
+    eager launches and synchronisations in between and fresh inputs written
+    into the captured buffers, must equal the eager result bit for bit."""
+    import torch
+    weight = oracle.quantize(helpers.normal(160, (1000, 2048), 0.02), 64,
+                             True, 256)
+    device_weight = upload(gpu, weight)
+    bias = to_device(helpers.normal(161, (1000,), 0.01))
+    lora_a = to_device(helpers.normal(162, (8, 2048), 0.05))
+    lora_b = to_device(helpers.normal(163, (1000, 8), 0.05))
+    row_counts = {"gemv": 2, "resident": 9, "skinny": 40, "mfma": 130}
+    inputs = {name: torch.zeros((rows, 2048), device="cuda")
+              for name, rows in row_counts.items()}
+    upstream = torch.zeros((130, 1000), device="cuda")
+    for name, rows in row_counts.items():
+        assert package.ALGORITHM_NAMES[library.select_algorithm(
+            package.FORWARD, rows, 2048, 1000, 64)] == name
+
+    def launch_all():
+        outputs = {name: gpu.linear_forward(x, device_weight, bias)
+                   for name, x in inputs.items()}
+        outputs["adapter"], _ = gpu.lora_linear_forward(
+            inputs["resident"], device_weight, lora_a, lora_b, 0.5, bias)
+        outputs["backward"] = gpu.linear_input_backward(upstream,
+                                                        device_weight)
+        return outputs
+
+    def refill(seed):
+        for index, x in enumerate(inputs.values()):
+            x.copy_(to_device(helpers.normal(seed + index, tuple(x.shape),
+                                             1.0)))
+        upstream.copy_(to_device(helpers.normal(seed + 9, (130, 1000),
+                                                1.0e-2)))
+
+    refill(170)
+    launch_all()                      # first use allocates the workspace
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            captured = launch_all()
+    for replay in range(4):
+        refill(180 + 10 * replay)
+        eager = {name: host(value) for name, value in launch_all().items()}
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, value in captured.items():
+            helpers.assert_bit_equal(host(value), eager[name],
+                                     f"replay {replay}, {name}")
