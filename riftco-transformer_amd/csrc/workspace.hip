@@ -9,21 +9,21 @@
 
 #include "kernels.hpp"
 
+#include <map>
 #include <mutex>
-#include <unordered_map>
+#include <utility>
 
 namespace rthip {
 
 hipError_t stream_workspace(hipStream_t stream, float** out) {
     static std::mutex guard;
-    static std::unordered_map<std::uintptr_t, float*> buffers;
+    static std::map<std::pair<int, hipStream_t>, float*> buffers;
     int device = 0;
     hipError_t status = hipGetDevice(&device);
     if (status != hipSuccess) {
         return status;
     }
-    const std::uintptr_t key = reinterpret_cast<std::uintptr_t>(stream) * 64 +
-                               static_cast<std::uintptr_t>(device);
+    const std::pair<int, hipStream_t> key(device, stream);
     const std::lock_guard<std::mutex> lock(guard);
     const auto found = buffers.find(key);
     if (found != buffers.end()) {
@@ -41,10 +41,11 @@ hipError_t stream_workspace(hipStream_t stream, float** out) {
     if (status != hipSuccess) {
         return status;
     }
+    // kept even if the capture mode could not be restored: the buffer exists
+    buffers.emplace(key, static_cast<float*>(fresh));
     if (restored != hipSuccess) {
         return restored;
     }
-    buffers.emplace(key, static_cast<float*>(fresh));
     *out = static_cast<float*>(fresh);
     return hipSuccess;
 }

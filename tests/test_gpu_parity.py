@@ -842,3 +842,40 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
         for name, value in captured.items():
             helpers.assert_bit_equal(host(value), eager[name],
                                      f"replay {replay}, {name}")
+
+
+# ---- a seeded sweep over small random problems -------------------------------
+
+def test_random_small_problems(gpu, package, library, oracle):
+    """Forty seeded problems with every quantity drawn at random -- widths that
+    are and are not multiples of the kernels' tile sizes, every block size up
+    to 512, both encodings, with and without bias -- through every family that
+    accepts them, against the oracle and fp64."""
+    generator = np.random.default_rng(2024)
+    widths = [16, 32, 33, 48, 64, 80, 96, 128, 160, 192, 256, 320, 512, 1024,
+              2048]
+    for case in range(40):
+        in_w = int(generator.choice(widths))
+        out_w = int(generator.integers(1, 400))
+        rows = int(generator.choice([1, 2, 3, 4, 5, 8, 15, 16, 17, 31, 64, 65,
+                                     100]))
+        block = int(generator.choice([32, 64, 128, 256, 512]))
+        second = int(generator.choice([32, 64, 256]))
+        nested = bool(generator.integers(0, 2))
+        with_bias = bool(generator.integers(0, 2))
+        dense = helpers.normal(3000 + case, (out_w, in_w), 0.02)
+        if case % 4 == 0:
+            dense[generator.integers(0, out_w)] = 0.0
+        weight = oracle.quantize(dense, block, nested, second)
+        x = helpers.normal(3100 + case, (rows, in_w), 1.0)
+        dy = helpers.normal(3200 + case, (rows, out_w), 1.0e-2)
+        bias = helpers.normal(3300 + case, (out_w,), 0.01) \
+            if with_bias else None
+        try:
+            check_layer(gpu, package, library, oracle, weight, x, dy,
+                        bias=bias, oracle_rows=min(rows, 4))
+        except AssertionError as error:
+            raise AssertionError(
+                f"case {case}: rows={rows} out={out_w} in={in_w} "
+                f"block={block} second={second} nested={nested} "
+                f"bias={with_bias}: {error}") from error
