@@ -51,10 +51,9 @@ namespace rthip {
 namespace {
 
 constexpr int kWave = 64;
-constexpr int kTeamThreads = 256;  // threads that share one weight row
+constexpr int kWorkgroupThreads = 512;
 constexpr int kSegment = 16;       // weights per thread per row visit
 constexpr int kRowLanes = 16;      // lanes of one DPP row
-constexpr int kTeamWaves = kTeamThreads / kWave;
 constexpr unsigned kComputeUnits = 256;
 // Row totals a team may park in LDS before the final barrier, per wavefront.
 constexpr unsigned kParkedValues = 128;
@@ -160,16 +159,20 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base,
 
 // kX: x rows held per thread (1, 2 or 4; a 3-row call runs as 4 with a zero
 // row).  kSegments: segments per thread.  kRows: weight rows per batch.
-// kTeams: teams per workgroup.
+// kTeams: teams per workgroup (2 teams of four wavefronts, or 1 team of eight
+// for rows so wide that four wavefronts' threads could not hold their x).
 template <int kX, int kSegments, int kRows, int kTeams, int kDepth,
           bool kDoubleQuantized>
-__global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
+__global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
     const float* __restrict__ x, Nf4WeightView weight, unsigned secondary_bytes,
     const float* __restrict__ bias, float* __restrict__ y, unsigned x_rows,
     unsigned input_width, unsigned output_width, unsigned block_shift,
     unsigned batch_count, unsigned iterations, LoraEpilogue lora
 ) {
-    constexpr int kThreads = kTeamThreads * kTeams;
+    constexpr int kThreads = kWorkgroupThreads;
+    // threads that share one weight row
+    constexpr int kTeamThreads = kWorkgroupThreads / kTeams;
+    constexpr int kTeamWaves = kTeamThreads / kWave;
     constexpr int kValues = kRows * kX;
     constexpr unsigned kMaxIterations = kParkedValues / kValues;
     __shared__ __attribute__((aligned(256))) char table[kPairTableBytes];
@@ -434,17 +437,31 @@ __global__ __launch_bounds__(kTeamThreads * kTeams) void gemv_forward_kernel(
     }
 }
 
-std::size_t segments_per_thread(const LinearProblem& p) {
-    return (p.input_width / kSegment + kTeamThreads - 1) / kTeamThreads;
+std::size_t segments_per_thread(const LinearProblem& p,
+                                std::size_t team_threads) {
+    return (p.input_width / kSegment + team_threads - 1) / team_threads;
 }
 
-template <int kX, int kSegments, bool kDoubleQuantized>
+// x rows held per thread (a 3-row call runs as 4 with a zero row).
+std::size_t held_rows(const LinearProblem& p) {
+    return p.rows == 3 ? 4 : p.rows;
+}
+
+// A thread's register-resident slice of x is held_rows x segments x 16
+// values; beyond 8 x 16 it no longer fits.  Two teams of 256 threads per
+// workgroup measured best; rows too wide for that get one team of 512.
+constexpr std::size_t kMaxHeldSegments = 8;
+bool wide_team(const LinearProblem& p) {
+    return held_rows(p) * segments_per_thread(p, 256) > kMaxHeldSegments;
+}
+
+template <int kX, int kSegments, bool kDoubleQuantized, bool kWide = false>
 void launch_instance(const LinearProblem& p, hipStream_t stream) {
     // Two teams (eight wavefronts) per workgroup measured best on MI355X; a
     // thread that carries more x rows or segments takes fewer weight rows per
     // batch so that its registers fit.
     constexpr bool kLight = kX * kSegments == 1;
-    constexpr int kTeams = kLight ? RTHIP_GEMV_TEAMS : 2;
+    constexpr int kTeams = kWide ? 1 : (kLight ? RTHIP_GEMV_TEAMS : 2);
     constexpr int kRows =
         kLight ? RTHIP_GEMV_ROWS : (kX * kSegments <= 4 ? 4 : 2);
     constexpr int kDepth = kLight ? RTHIP_GEMV_DEPTH : 2;
@@ -468,7 +485,7 @@ void launch_instance(const LinearProblem& p, hipStream_t stream) {
     }
     const unsigned iterations = (team_groups + blocks - 1) / blocks;
     gemv_forward_kernel<kX, kSegments, kRows, kTeams, kDepth, kDoubleQuantized>
-        <<<blocks, kTeamThreads * kTeams, 0, stream>>>(
+        <<<blocks, kWorkgroupThreads, 0, stream>>>(
             p.activations, p.weight, secondary_bytes, p.bias, p.result,
             static_cast<unsigned>(p.rows),
             static_cast<unsigned>(p.input_width),
@@ -478,7 +495,15 @@ void launch_instance(const LinearProblem& p, hipStream_t stream) {
 
 template <int kX, bool kDoubleQuantized>
 void launch_segments(const LinearProblem& p, hipStream_t stream) {
-    switch (segments_per_thread(p)) {
+    if (wide_team(p)) {
+        // four x rows and a row wider than 8192: two segments per thread of a
+        // 512-thread team
+        if constexpr (kX == 4) {
+            launch_instance<kX, 2, kDoubleQuantized, true>(p, stream);
+        }
+        return;
+    }
+    switch (segments_per_thread(p, 256)) {
     case 1: launch_instance<kX, 1, kDoubleQuantized>(p, stream); break;
     case 2: launch_instance<kX, 2, kDoubleQuantized>(p, stream); break;
     case 3: launch_instance<kX, 3, kDoubleQuantized>(p, stream); break;
@@ -499,12 +524,13 @@ void launch_rows(const LinearProblem& p, hipStream_t stream) {
 
 bool gemv_forward_supports(const LinearProblem& p) {
     constexpr std::size_t kMaxWidth =
-        static_cast<std::size_t>(kSegment) * kTeamThreads * 4;
-    // x rows (3 runs as 4) times segments per thread bounds the
-    // register-resident x slice.
-    const std::size_t held_rows = p.rows == 3 ? 4 : p.rows;
+        static_cast<std::size_t>(kSegment) * 256 * 4;
     return p.rows >= 1 && p.rows <= kGemvMaxRows &&
-           held_rows * segments_per_thread(p) <= 8 &&
+           // the register-resident x slice must fit, with two teams of 256
+           // threads or, for three and four rows, one team of 512
+           (!wide_team(p) ||
+            (held_rows(p) == 4 && held_rows(p) * segments_per_thread(p, 512) <=
+                                      kMaxHeldSegments)) &&
            p.input_width % kSegment == 0 && p.input_width <= kMaxWidth &&
            // rows start on block boundaries (scalar row offset into scales)
            p.input_width % (std::size_t{1} << p.block_shift) == 0 &&

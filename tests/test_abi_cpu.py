@@ -39,6 +39,11 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(fwd, 1, 4096, 4096, 64) == package.ALGORITHM_GEMV
     assert select(fwd, 1, 4096, 11008, 64) == package.ALGORITHM_GEMV
     assert select(fwd, 1, 11008, 4096, 64) == package.ALGORITHM_GEMV
+    # three and four rows of a wide layer: one 512-thread team per weight row
+    assert select(fwd, 2, 11008, 4096, 64) == package.ALGORITHM_GEMV
+    assert select(fwd, 3, 11008, 4096, 64) == package.ALGORITHM_GEMV
+    assert select(fwd, 4, 16384, 4096, 64) == package.ALGORITHM_GEMV
+    assert select(fwd, 4, 16384 + 64, 4096, 64) == package.ALGORITHM_SKINNY
     # prefill / training -> MFMA GEMM, both directions
     assert select(fwd, 2048, 4096, 11008, 64) == package.ALGORITHM_MFMA
     # small batches -> weights decoded straight into MFMA operands

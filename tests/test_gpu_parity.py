@@ -296,6 +296,27 @@ def test_resident_small_batch_family(gpu, package, library, oracle, out_w,
                     oracle_rows=min(rows, 3))
 
 
+@pytest.mark.parametrize("out_w,in_w,block,double_quantized", [
+    (4096, 11008, 64, False),   # down_proj
+    (300, 16384, 128, True),    # the widest row the GEMV takes
+    (77, 8192 + 256, 32, True),  # just past two segments per 256 threads
+])
+def test_wide_rows_at_three_and_four_rows(gpu, package, library, oracle, out_w,
+                                          in_w, block, double_quantized):
+    """Rows wider than 8192 with three or four x rows run the GEMV with one
+    512-thread team per weight row."""
+    weight = oracle.quantize(helpers.normal(77, (out_w, in_w), 0.02), block,
+                             double_quantized, 256)
+    bias = helpers.normal(78, (out_w,), 0.01)
+    for rows in (3, 4):
+        assert library.select_algorithm(package.FORWARD, rows, in_w, out_w,
+                                        block) == package.ALGORITHM_GEMV
+        x = helpers.normal(79 + rows, (rows, in_w), 1.0)
+        dy = helpers.normal(80 + rows, (rows, out_w), 1.0e-2)
+        check_layer(gpu, package, library, oracle, weight, x, dy, bias=bias,
+                    oracle_rows=2)
+
+
 def test_zero_scale_blocks_and_saturated_scales(gpu, package, library,
                                                 oracle):
     dense = helpers.normal(70, (64, 128), 0.02)
