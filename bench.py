@@ -383,6 +383,9 @@ def main():
     parser.add_argument("--gemm-only", action="store_true",
                         help="run only the M = 2048 GEMM section (for "
                              "rocprofv3 counter runs)")
+    parser.add_argument("--small-batch-only", action="store_true",
+                        help="run only the M in {1, 4, 16, 64} launches "
+                             "(for counter runs)")
     parser.add_argument("--traffic-calibration", action="store_true",
                         help="for rocprofv3 --pmc runs: a 1 GiB elementwise "
                              "copy of known traffic, then one decode step "
@@ -420,6 +423,11 @@ def main():
         # For counter runs: nothing but the M = 2048 launches.
         print(json.dumps({"gemm": bench_gemm(package, device, torch,
                                              arguments.steps)}))
+        return
+
+    if arguments.small_batch_only:
+        print(json.dumps({"small_batch": bench_small_batch(
+            package, device, torch, arguments.steps)}))
         return
 
     decode = bench_decode(package, device, torch, arguments.layers,

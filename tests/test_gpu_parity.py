@@ -317,6 +317,30 @@ def test_wide_rows_at_three_and_four_rows(gpu, package, library, oracle, out_w,
                     oracle_rows=2)
 
 
+def test_shared_output_tiles_are_added_in_a_fixed_order(gpu, package, library,
+                                                        oracle):
+    """When several workgroups hold parts of an output tile, the parts are
+    added in ascending workgroup order whatever the timing of the launch.
+    Twenty launches each at two shapes, interleaved with other work on the
+    device, all bit-identical."""
+    import torch
+    for out_w, in_w, rows in ((1000, 4096 + 256, 40), (4096, 11008, 16)):
+        weight = oracle.quantize(helpers.normal(90, (out_w, in_w), 0.02), 64,
+                                 False, 256)
+        device_weight = upload(gpu, weight)
+        assert library.select_algorithm(
+            package.FORWARD, rows, in_w, out_w, 64) == package.ALGORITHM_SKINNY
+        x = to_device(helpers.normal(91, (rows, in_w), 1.0))
+        first = host(gpu.linear_forward(x, device_weight))
+        filler = torch.zeros(1 << 22, device="cuda")
+        for launch in range(20):
+            if launch % 3 == 0:
+                filler.add_(1.0)      # something else in flight before it
+            helpers.assert_bit_equal(
+                host(gpu.linear_forward(x, device_weight)), first,
+                f"launch {launch}")
+
+
 def test_zero_scale_blocks_and_saturated_scales(gpu, package, library,
                                                 oracle):
     dense = helpers.normal(70, (64, 128), 0.02)
