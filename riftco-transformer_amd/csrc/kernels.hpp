@@ -47,7 +47,7 @@ void launch_gemv_forward(const LinearProblem& problem, hipStream_t stream);
 
 // workspace.hip -- scratch memory shared by the kernels that pass partial
 // results between workgroups; one fixed-size buffer per (device, stream).
-constexpr std::size_t kStreamWorkspaceBytes = std::size_t{32} << 20;
+constexpr std::size_t kStreamWorkspaceBytes = std::size_t{64} << 20;
 hipError_t stream_workspace(hipStream_t stream, float** out);
 
 // nf4_skinny.hip -- forward only, up to 64 rows, decode straight into MFMA
@@ -114,9 +114,10 @@ PayloadViolation classify_payload(const unsigned long long words[3]);
 
 // nf4_mfma.hip
 bool mfma_forward_supports(const LinearProblem& problem);
-void launch_mfma_forward(const LinearProblem& problem, hipStream_t stream);
+hipError_t launch_mfma_forward(const LinearProblem& problem,
+                               hipStream_t stream);
 bool mfma_input_backward_supports(const LinearProblem& problem);
-void launch_mfma_input_backward(const LinearProblem& problem,
-                                hipStream_t stream);
+hipError_t launch_mfma_input_backward(const LinearProblem& problem,
+                                      hipStream_t stream);
 
 }  // namespace rthip

@@ -22,12 +22,24 @@
 // valid because both operands use the same one.  Global loads for step t+1 are
 // issued before the MFMAs of step t.
 //
+// Work split.  Output tiles are dealt to workgroups whole while they fill the
+// device evenly (two workgroups per compute unit).  What is left over -- 1376
+// tiles on 512 places leave 352 -- would occupy the device for a whole further
+// round at 69 % occupancy, so those tiles are cut along the contraction
+// instead: their (tile, step) units are dealt in equal contiguous runs to as
+// many workgroups as there are places, a workgroup whose run covers a whole
+// tile writes it as usual, the others write partial tiles to the stream's
+// workspace and a second kernel adds the parts of each tile in ascending
+// workgroup order (plus bias and adapter term).  Nothing depends on timing.
+//
 // The two directions share everything except the weight-tile loader: forward
 // reads 128 weight rows x 32 contiguous columns, backward reads 32 weight rows
 // (the contraction) x 128 contiguous columns and transposes while writing LDS.
 
 #include "kernels.hpp"
 #include "nf4_decode.hpp"
+
+#include <algorithm>
 
 namespace rthip {
 namespace {
@@ -48,6 +60,33 @@ struct GemmShape {
     unsigned columns;      // O (forward) or I (backward)
     unsigned input_width;  // I: the weight's row length
 };
+
+// How a launch covers the tile grid.  Tiles are numbered row-major (tile /
+// tiles_n is the tile row).  The first `whole_tiles` workgroups take one whole
+// tile each.  The tiles after those are cut into (tile, step) units -- one
+// contraction step of one tile, tile-major -- which are dealt to the remaining
+// workgroups in contiguous runs: the first `remainder` of them take
+// quotient + 1 units, the others quotient.  A run never exceeds one tile's
+// worth of steps, so it touches at most two tiles.  Whole-tile workgroups
+// come first in the grid and the shorter runs last, which is also the order
+// in which the device starts them.
+struct GemmPlan {
+    unsigned tiles_n;      // output tiles per tile row
+    unsigned whole_tiles;  // tiles computed by one workgroup each
+    unsigned steps;        // contraction steps per tile
+    unsigned quotient;
+    unsigned remainder;
+
+    __host__ __device__ unsigned begin(unsigned group) const {
+        return group * quotient + (group < remainder ? group : remainder);
+    }
+    __host__ __device__ unsigned owner(unsigned unit) const {
+        const unsigned boundary = remainder * (quotient + 1);
+        return unit < boundary ? unit / (quotient + 1)
+                               : remainder + (unit - boundary) / quotient;
+    }
+};
+constexpr unsigned kSlotsPerGroup = 2;  // partial tiles a workgroup may write
 
 // Registers holding one step's global loads of a thread.
 struct Staged {
@@ -178,24 +217,28 @@ __device__ __forceinline__ void store_weight_tile(
     }
 }
 
+// One segment: contraction values [k_begin, k_end) of the output tile at
+// (row0, col0).  `partial` null: the segment is the whole contraction and the
+// tile goes to `result` with bias and adapter term; otherwise the 128 x 128
+// partial sums go to `partial`.
 template <bool kDoubleQuantized, bool kBackward>
-__global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
-    const float* __restrict__ activations, Nf4WeightView weight,
+__device__ __forceinline__ void gemm_segment(
+    const float* __restrict__ activations, const Nf4WeightView& weight,
     const float* __restrict__ bias, float* __restrict__ result,
-    GemmShape shape, unsigned block_shift, LoraEpilogue lora
+    float* __restrict__ partial, const GemmShape& shape, unsigned block_shift,
+    const LoraEpilogue& lora, float* __restrict__ a_tile,
+    float* __restrict__ b_tile, const float* __restrict__ table,
+    unsigned row0, unsigned col0, unsigned k_begin, unsigned k_end
 ) {
-    __shared__ __attribute__((aligned(16))) float a_tile[kTileM * kStride];
-    __shared__ __attribute__((aligned(16))) float b_tile[kTileN * kStride];
-    __shared__ float table[16];
-    load_codebook_to_lds(table);
-
     const unsigned thread = threadIdx.x;
     const unsigned lane = thread % 64;
     const unsigned wave = thread / 64;
     const unsigned wave_m = wave / 2;
     const unsigned wave_n = wave % 2;
-    const unsigned row0 = blockIdx.y * kTileM;
-    const unsigned col0 = blockIdx.x * kTileN;
+    const float* a_fragment =
+        a_tile + (wave_m * 64 + lane % 32) * kStride + 4 * (lane / 32);
+    const float* b_fragment =
+        b_tile + (wave_n * 64 + lane % 32) * kStride + 4 * (lane / 32);
 
     // Two-level accumulation: the matrix cores add into `acc` for
     // kFlushSteps steps (256 contraction values), then `acc` is folded into
@@ -218,28 +261,23 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
     unsigned steps_since_flush = 0;
 
     Staged staged;
-    load_activation_tile(staged, activations, shape, row0, 0);
+    load_activation_tile(staged, activations, shape, row0, k_begin);
     if constexpr (!kBackward) {
-        load_weight_tile_forward<kDoubleQuantized>(staged, weight, shape,
-                                                   col0, 0, block_shift);
+        load_weight_tile_forward<kDoubleQuantized>(
+            staged, weight, shape, col0, k_begin, block_shift);
     } else {
-        load_weight_tile_backward<kDoubleQuantized>(staged, weight, shape,
-                                                    col0, 0, block_shift);
+        load_weight_tile_backward<kDoubleQuantized>(
+            staged, weight, shape, col0, k_begin, block_shift);
     }
 
-    const float* a_fragment =
-        a_tile + (wave_m * 64 + lane % 32) * kStride + 4 * (lane / 32);
-    const float* b_fragment =
-        b_tile + (wave_n * 64 + lane % 32) * kStride + 4 * (lane / 32);
-
-    for (unsigned k0 = 0; k0 < shape.contraction; k0 += kTileK) {
+    for (unsigned k0 = k_begin; k0 < k_end; k0 += kTileK) {
         __syncthreads();  // previous step's fragment reads are done
         store_activation_tile(staged, a_tile);
         store_weight_tile<kBackward>(staged, table, b_tile);
         __syncthreads();
 
         const unsigned next = k0 + kTileK;
-        if (next < shape.contraction) {
+        if (next < k_end) {
             load_activation_tile(staged, activations, shape, row0, next);
             if constexpr (!kBackward) {
                 load_weight_tile_forward<kDoubleQuantized>(
@@ -307,6 +345,22 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
 
     // Accumulator element e of lane l is output row 8*(e/4) + 4*(l/32) + e%4,
     // column l%32 of its 32 x 32 block.
+    if (partial != nullptr) {  // uniform; layout [kTileM][kTileN]
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const unsigned column = wave_n * 64 + j * 32 + lane % 32;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const unsigned row = wave_m * 64 + i * 32 + 8 * (e / 4) +
+                                         4 * (lane / 32) + e % 4;
+                    partial[row * kTileN + column] = total[i][j][e];
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -358,8 +412,151 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
     }
 }
 
+template <bool kDoubleQuantized, bool kBackward>
+__global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
+    const float* __restrict__ activations, Nf4WeightView weight,
+    const float* __restrict__ bias, float* __restrict__ result,
+    float* __restrict__ workspace, GemmShape shape, GemmPlan plan,
+    unsigned block_shift, LoraEpilogue lora
+) {
+    __shared__ __attribute__((aligned(16))) float a_tile[kTileM * kStride];
+    __shared__ __attribute__((aligned(16))) float b_tile[kTileN * kStride];
+    __shared__ float table[16];
+    load_codebook_to_lds(table);
+
+    // A whole tile, or a run of (tile, step) units: one or two segments,
+    // each inside one tile.
+    const bool whole = blockIdx.x < plan.whole_tiles;
+    const unsigned group = whole ? 0U : blockIdx.x - plan.whole_tiles;
+    const unsigned first_tile = whole ? blockIdx.x : plan.whole_tiles;
+    unsigned unit = whole ? 0U : plan.begin(group);
+    const unsigned unit_end = whole ? plan.steps : plan.begin(group + 1);
+    for (unsigned segment = 0; unit < unit_end; ++segment) {
+        const unsigned tile_in_run = unit / plan.steps;
+        const unsigned first_step = unit - tile_in_run * plan.steps;
+        const unsigned segment_steps =
+            min(unit_end - unit, plan.steps - first_step);
+        const unsigned tile = first_tile + tile_in_run;
+        float* const partial =
+            segment_steps == plan.steps
+                ? nullptr
+                : workspace + static_cast<std::size_t>(
+                                  group * kSlotsPerGroup + segment) *
+                                  kTileM * kTileN;
+        gemm_segment<kDoubleQuantized, kBackward>(
+            activations, weight, bias, result, partial, shape, block_shift,
+            lora, a_tile, b_tile, table, (tile / plan.tiles_n) * kTileM,
+            (tile % plan.tiles_n) * kTileN, first_step * kTileK,
+            (first_step + segment_steps) * kTileK);
+        unit += segment_steps;
+    }
+}
+
+// Adds the parts of every unit-dealt tile that more than one workgroup worked
+// on, in ascending workgroup order, plus bias and adapter term.  One thread
+// per output element: blockIdx.x is the tile among the unit-dealt ones,
+// blockIdx.y a run of 256 elements of it.
+__global__ __launch_bounds__(256) void gemm_parts_kernel(
+    const float* __restrict__ workspace, const float* __restrict__ bias,
+    float* __restrict__ result, GemmShape shape, GemmPlan plan,
+    LoraEpilogue lora
+) {
+    const unsigned dealt_tile = blockIdx.x;
+    const unsigned first_unit = dealt_tile * plan.steps;
+    const unsigned first_group = plan.owner(first_unit);
+    const unsigned last_group = plan.owner(first_unit + plan.steps - 1);
+    if (first_group == last_group) {
+        return;  // written directly by its only workgroup
+    }
+    const unsigned tile = plan.whole_tiles + dealt_tile;
+    const unsigned index = blockIdx.y * blockDim.x + threadIdx.x;
+    const unsigned m = index / kTileN;
+    const unsigned c = index % kTileN;
+    const unsigned row = (tile / plan.tiles_n) * kTileM + m;
+    const unsigned column = (tile % plan.tiles_n) * kTileN + c;
+    if (row >= shape.rows || column >= shape.columns) {
+        return;
+    }
+    const float* source = workspace + m * kTileN + c;
+    float sum = 0.0F;
+    for (unsigned group = first_group; group <= last_group; ++group) {
+        // A workgroup's slot 0 holds the first tile of its run.
+        const unsigned slot =
+            group * kSlotsPerGroup +
+            (dealt_tile == plan.begin(group) / plan.steps ? 0U : 1U);
+        sum += source[static_cast<std::size_t>(slot) * kTileM * kTileN];
+    }
+    if (bias != nullptr) {
+        sum += bias[column];
+    }
+    if (lora.reduced != nullptr) {
+        sum += lora_term(lora, row, column);
+    }
+    result[static_cast<std::size_t>(row) * shape.columns + column] = sum;
+}
+
+// Workgroups the device holds at once: two per compute unit.
+constexpr unsigned kPlaces = 512;
+// A unit-dealt run is at least this many steps (a quarter of a kilobyte of
+// codes per weight row), and unit dealing is not worth a second kernel when
+// the leftover tiles nearly fill the device anyway.
+constexpr unsigned kMinimumRunSteps = 8;
+
+template <bool kDoubleQuantized, bool kBackward>
+hipError_t launch_encoding(const LinearProblem& p, const GemmShape& shape,
+                           hipStream_t stream) {
+    const auto kernel = mfma_gemm_kernel<kDoubleQuantized, kBackward>;
+    const unsigned tiles_m = (shape.rows + kTileM - 1) / kTileM;
+    const unsigned tiles_n = (shape.columns + kTileN - 1) / kTileN;
+    const unsigned tiles = tiles_m * tiles_n;
+    GemmPlan plan;
+    plan.tiles_n = tiles_n;
+    plan.steps = (shape.contraction + kTileK - 1) / kTileK;
+    const unsigned leftover = tiles % kPlaces;
+    const bool deal_units = leftover != 0 && leftover * 10 < kPlaces * 9 &&
+                            plan.steps >= 2 * kMinimumRunSteps &&
+                            // partial tiles fit the workspace
+                            static_cast<std::size_t>(kPlaces) *
+                                    kSlotsPerGroup * kTileM * kTileN *
+                                    sizeof(float) <=
+                                kStreamWorkspaceBytes;
+    plan.whole_tiles = deal_units ? tiles - leftover : tiles;
+    plan.quotient = 0;
+    plan.remainder = 0;
+    if (!deal_units) {
+        kernel<<<tiles, kThreads, 0, stream>>>(
+            p.activations, p.weight, p.bias, p.result, nullptr, shape, plan,
+            p.block_shift, p.lora);
+        return hipSuccess;
+    }
+    float* workspace = nullptr;
+    if (const hipError_t status = stream_workspace(stream, &workspace);
+        status != hipSuccess) {
+        return status;
+    }
+    const unsigned units = leftover * plan.steps;
+    unsigned groups = units / kMinimumRunSteps;
+    if (groups > kPlaces) {
+        groups = kPlaces;
+    }
+    if (groups < leftover) {
+        groups = leftover;  // a run never exceeds one tile
+    }
+    plan.quotient = units / groups;
+    plan.remainder = units % groups;
+    kernel<<<plan.whole_tiles + groups, kThreads, 0, stream>>>(
+        p.activations, p.weight, p.bias, p.result, workspace, shape, plan,
+        p.block_shift, p.lora);
+    if (groups != leftover) {  // some tile has parts
+        const dim3 grid(leftover, kTileM * kTileN / 256);
+        gemm_parts_kernel<<<grid, 256, 0, stream>>>(
+            workspace, p.bias, p.result, shape, plan, p.lora);
+    }
+    return hipSuccess;
+}
+
 template <bool kBackward>
-void launch(const LinearProblem& p, hipStream_t stream) {
+hipError_t launch(const LinearProblem& p, hipStream_t stream) {
     GemmShape shape;
     shape.rows = static_cast<unsigned>(p.rows);
     shape.input_width = static_cast<unsigned>(p.input_width);
@@ -370,24 +567,20 @@ void launch(const LinearProblem& p, hipStream_t stream) {
         shape.contraction = static_cast<unsigned>(p.output_width);
         shape.columns = static_cast<unsigned>(p.input_width);
     }
-    const dim3 grid((shape.columns + kTileN - 1) / kTileN,
-                    (shape.rows + kTileM - 1) / kTileM);
-    if (p.weight.encoding == 0) {
-        mfma_gemm_kernel<false, kBackward><<<grid, kThreads, 0, stream>>>(
-            p.activations, p.weight, p.bias, p.result, shape, p.block_shift,
-            p.lora);
-    } else {
-        mfma_gemm_kernel<true, kBackward><<<grid, kThreads, 0, stream>>>(
-            p.activations, p.weight, p.bias, p.result, shape, p.block_shift,
-            p.lora);
-    }
+    return p.weight.encoding == 0
+               ? launch_encoding<false, kBackward>(p, shape, stream)
+               : launch_encoding<true, kBackward>(p, shape, stream);
 }
 
 bool common_supports(const LinearProblem& p) {
     constexpr std::size_t kLimit = 1ULL << 31;
     return p.rows >= 1 && p.rows < kLimit && p.input_width < kLimit &&
            p.output_width < kLimit &&
-           (p.rows + kTileM - 1) / kTileM <= 65535 &&
+           // tile and (tile, step) unit counts stay 32-bit
+           ((p.rows + kTileM - 1) / kTileM) *
+                   ((std::max(p.input_width, p.output_width) + kTileN - 1) /
+                    kTileN) <
+               (1ULL << 24) &&
            reinterpret_cast<std::uintptr_t>(p.weight.codes) % 8 == 0 &&
            reinterpret_cast<std::uintptr_t>(p.activations) % 16 == 0;
 }
@@ -401,8 +594,8 @@ bool mfma_forward_supports(const LinearProblem& p) {
     return common_supports(p) && p.input_width % kTileK == 0;
 }
 
-void launch_mfma_forward(const LinearProblem& p, hipStream_t stream) {
-    launch<false>(p, stream);
+hipError_t launch_mfma_forward(const LinearProblem& p, hipStream_t stream) {
+    return launch<false>(p, stream);
 }
 
 bool mfma_input_backward_supports(const LinearProblem& p) {
@@ -412,8 +605,9 @@ bool mfma_input_backward_supports(const LinearProblem& p) {
            p.input_width % kChunk == 0;
 }
 
-void launch_mfma_input_backward(const LinearProblem& p, hipStream_t stream) {
-    launch<true>(p, stream);
+hipError_t launch_mfma_input_backward(const LinearProblem& p,
+                                      hipStream_t stream) {
+    return launch<true>(p, stream);
 }
 
 }  // namespace rthip

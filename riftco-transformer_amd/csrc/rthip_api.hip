@@ -430,7 +430,11 @@ rthip_status linear_forward_common(
                         "the MFMA family needs a row width that is a "
                         "multiple of 32 and aligned pointers");
         }
-        rthip::launch_mfma_forward(problem, hip_stream);
+        if (const hipError_t status =
+                rthip::launch_mfma_forward(problem, hip_stream);
+            status != hipSuccess) {
+            return from_hip(status, "GEMM workspace allocation");
+        }
         break;
     case RTHIP_NF4_ALGORITHM_SKINNY:
         if (!rthip::skinny_forward_supports(problem)) {
@@ -690,7 +694,11 @@ rthip_status rthip_nf4_linear_input_backward_with(
                         "multiple of 32, a row width that is a multiple of "
                         "16 and aligned pointers");
         }
-        rthip::launch_mfma_input_backward(problem, hip_stream);
+        if (const hipError_t status =
+                rthip::launch_mfma_input_backward(problem, hip_stream);
+            status != hipSuccess) {
+            return from_hip(status, "GEMM workspace allocation");
+        }
         break;
     case RTHIP_NF4_ALGORITHM_GEMV:
     case RTHIP_NF4_ALGORITHM_SKINNY:

@@ -341,6 +341,36 @@ def test_shared_output_tiles_are_added_in_a_fixed_order(gpu, package, library,
                 f"launch {launch}")
 
 
+@pytest.mark.parametrize("rows,out_w,in_w,double_quantized", [
+    (300, 1000, 1024, False),   # 24 tiles, each cut into four runs
+    (130, 260, 1056, True),     # 6 tiles, runs of 8 and 9 steps
+    (1280, 2560, 4096, True),   # 200 tiles dealt to 512 workgroups
+    (2200, 3700, 512, False),   # 522 tiles: 512 whole, 10 cut into runs
+    (200, 384, 256, False),     # too few steps: whole tiles only
+])
+def test_gemm_leftover_tiles_are_dealt_in_units(gpu, package, library, oracle,
+                                                rows, out_w, in_w,
+                                                double_quantized):
+    """Tile counts that do not fill the device evenly: the leftover tiles are
+    cut along the contraction, partial tiles are added by a second kernel.
+    Both directions, with bias, ragged edges in every dimension."""
+    weight = oracle.quantize(helpers.normal(95, (out_w, in_w), 0.02), 64,
+                             double_quantized, 256)
+    assert library.select_algorithm(package.FORWARD, rows, in_w, out_w,
+                                    64) == package.ALGORITHM_MFMA
+    x = helpers.normal(96, (rows, in_w), 1.0)
+    dy = helpers.normal(97, (rows, out_w), 1.0e-2)
+    bias = helpers.normal(98, (out_w,), 0.01)
+    check_layer(gpu, package, library, oracle, weight, x, dy, bias=bias,
+                oracle_rows=2)
+    # the same launch again gives the same bits
+    device_weight = upload(gpu, weight)
+    first = host(gpu.linear_forward(to_device(x), device_weight))
+    for _ in range(3):
+        helpers.assert_bit_equal(
+            host(gpu.linear_forward(to_device(x), device_weight)), first)
+
+
 def test_zero_scale_blocks_and_saturated_scales(gpu, package, library,
                                                 oracle):
     dense = helpers.normal(70, (64, 128), 0.02)
