@@ -23,8 +23,14 @@
 // single matrix with fewer than 128 tiles the contraction is therefore cut
 // into slices, one workgroup per (tile, slice) writes its partial tile to the
 // stream's workspace, and a second kernel adds the slices in ascending order.
+//
+// A large single matrix whose tile count does not fill the device evenly
+// (2048 x 11008 is 1376 tiles on 512 places) has its leftover tiles cut along
+// the contraction and dealt in equal runs to the workgroups that would
+// otherwise idle (tile_plan.hpp), as the packed GEMM does.
 
 #include "kernels.hpp"
+#include "tile_plan.hpp"
 
 namespace rthip {
 namespace {
@@ -117,32 +123,20 @@ __device__ __forceinline__ void store_tiles(const Staged& staged,
     }
 }
 
-__global__ __launch_bounds__(kThreads, 2) void dense_matmul_kernel(
+// Contraction values [k_begin, k_end) of the output tile at (row0, col0).
+// `partial` null: the result goes to `out` ([rows][columns]); otherwise the
+// 128 x 128 sums go to `partial` ([kTileM][kTileN]).
+__device__ __forceinline__ void matmul_segment(
     const float* __restrict__ left, const float* __restrict__ right,
-    float* __restrict__ out, MatmulShape shape
+    float* __restrict__ out, float* __restrict__ partial,
+    const MatmulShape& shape, float* __restrict__ left_tile,
+    float* __restrict__ right_tile, unsigned row0, unsigned col0,
+    unsigned k_begin, unsigned k_end
 ) {
-    __shared__ __attribute__((aligned(16))) float left_tile[kTileM * kStride];
-    __shared__ __attribute__((aligned(16))) float right_tile[kTileN * kStride];
-
     const unsigned lane = threadIdx.x % 64;
     const unsigned wave = threadIdx.x / 64;
     const unsigned wave_m = wave / 2;
     const unsigned wave_n = wave % 2;
-    const unsigned row0 = blockIdx.y * kTileM;
-    const unsigned col0 = blockIdx.x * kTileN;
-    unsigned k_begin = 0;
-    unsigned k_end = shape.shared;
-    if (shape.slice == 0) {
-        const std::size_t batch = blockIdx.z;
-        left += batch * shape.rows * shape.shared;
-        right += batch * shape.shared * shape.columns;
-        out += batch * shape.rows * shape.columns;
-    } else {
-        k_begin = blockIdx.z * shape.slice;
-        k_end = min(k_begin + shape.slice, shape.shared);
-        out += static_cast<std::size_t>(blockIdx.z) * shape.rows *
-               shape.columns;
-    }
 
     floatx16 acc[2][2];
     floatx16 total[2][2];
@@ -232,21 +226,118 @@ __global__ __launch_bounds__(kThreads, 2) void dense_matmul_kernel(
     for (int i = 0; i < 2; ++i) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const unsigned column = col0 + wave_n * 64 + j * 32 + lane % 32;
-            if (column >= shape.columns) {
+            const unsigned tile_column = wave_n * 64 + j * 32 + lane % 32;
+            const unsigned column = col0 + tile_column;
+            if (partial == nullptr && column >= shape.columns) {
                 continue;
             }
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const unsigned row = row0 + wave_m * 64 + i * 32 +
-                                     8 * (e / 4) + 4 * (lane / 32) + e % 4;
-                if (row < shape.rows) {
-                    out[static_cast<std::size_t>(row) * shape.columns +
-                        column] = total[i][j][e] + acc[i][j][e];
+                const unsigned tile_row = wave_m * 64 + i * 32 + 8 * (e / 4) +
+                                          4 * (lane / 32) + e % 4;
+                const float value = total[i][j][e] + acc[i][j][e];
+                if (partial != nullptr) {  // uniform
+                    partial[tile_row * kTileN + tile_column] = value;
+                } else if (row0 + tile_row < shape.rows) {
+                    out[static_cast<std::size_t>(row0 + tile_row) *
+                            shape.columns +
+                        column] = value;
                 }
             }
         }
     }
+}
+
+// One whole tile per workgroup; blockIdx.z is the batch or, for a sliced
+// contraction, the slice.
+__global__ __launch_bounds__(kThreads, 2) void dense_matmul_kernel(
+    const float* __restrict__ left, const float* __restrict__ right,
+    float* __restrict__ out, MatmulShape shape
+) {
+    __shared__ __attribute__((aligned(16))) float left_tile[kTileM * kStride];
+    __shared__ __attribute__((aligned(16))) float right_tile[kTileN * kStride];
+    unsigned k_begin = 0;
+    unsigned k_end = shape.shared;
+    if (shape.slice == 0) {
+        const std::size_t batch = blockIdx.z;
+        left += batch * shape.rows * shape.shared;
+        right += batch * shape.shared * shape.columns;
+        out += batch * shape.rows * shape.columns;
+    } else {
+        k_begin = blockIdx.z * shape.slice;
+        k_end = min(k_begin + shape.slice, shape.shared);
+        out += static_cast<std::size_t>(blockIdx.z) * shape.rows *
+               shape.columns;
+    }
+    matmul_segment(left, right, out, nullptr, shape, left_tile, right_tile,
+                   blockIdx.y * kTileM, blockIdx.x * kTileN, k_begin, k_end);
+}
+
+// A single matrix covered according to a TilePlan: whole tiles first, then
+// runs of (tile, step) units.
+__global__ __launch_bounds__(kThreads, 2) void dense_matmul_planned_kernel(
+    const float* __restrict__ left, const float* __restrict__ right,
+    float* __restrict__ out, float* __restrict__ workspace, MatmulShape shape,
+    TilePlan plan
+) {
+    __shared__ __attribute__((aligned(16))) float left_tile[kTileM * kStride];
+    __shared__ __attribute__((aligned(16))) float right_tile[kTileN * kStride];
+    const bool whole = blockIdx.x < plan.whole_tiles;
+    const unsigned group = whole ? 0U : blockIdx.x - plan.whole_tiles;
+    const unsigned first_tile = whole ? blockIdx.x : plan.whole_tiles;
+    unsigned unit = whole ? 0U : plan.begin(group);
+    const unsigned unit_end = whole ? plan.steps : plan.begin(group + 1);
+    for (unsigned segment = 0; unit < unit_end; ++segment) {
+        const unsigned tile_in_run = unit / plan.steps;
+        const unsigned first_step = unit - tile_in_run * plan.steps;
+        const unsigned segment_steps =
+            min(unit_end - unit, plan.steps - first_step);
+        const unsigned tile = first_tile + tile_in_run;
+        float* const partial =
+            segment_steps == plan.steps
+                ? nullptr
+                : workspace +
+                      static_cast<std::size_t>(group * 2 + segment) * kTileM *
+                          kTileN;
+        matmul_segment(left, right, out, partial, shape, left_tile,
+                       right_tile, (tile / plan.tiles_n) * kTileM,
+                       (tile % plan.tiles_n) * kTileN, first_step * kTileK,
+                       min((first_step + segment_steps) * kTileK,
+                           shape.shared));
+        unit += segment_steps;
+    }
+}
+
+// Adds the parts of every unit-dealt tile that more than one workgroup worked
+// on, in ascending workgroup order.  blockIdx.x is the tile among the
+// unit-dealt ones, blockIdx.y a run of 256 elements of it.
+__global__ __launch_bounds__(256) void matmul_parts_kernel(
+    const float* __restrict__ workspace, float* __restrict__ out,
+    MatmulShape shape, TilePlan plan
+) {
+    const unsigned dealt_tile = blockIdx.x;
+    const unsigned first_unit = dealt_tile * plan.steps;
+    const unsigned first_group = plan.owner(first_unit);
+    const unsigned last_group = plan.owner(first_unit + plan.steps - 1);
+    if (first_group == last_group) {
+        return;  // written directly by its only workgroup
+    }
+    const unsigned tile = plan.whole_tiles + dealt_tile;
+    const unsigned index = blockIdx.y * blockDim.x + threadIdx.x;
+    const unsigned m = index / kTileN;
+    const unsigned c = index % kTileN;
+    const unsigned row = (tile / plan.tiles_n) * kTileM + m;
+    const unsigned column = (tile % plan.tiles_n) * kTileN + c;
+    if (row >= shape.rows || column >= shape.columns) {
+        return;
+    }
+    const float* source = workspace + m * kTileN + c;
+    float sum = 0.0F;
+    for (unsigned group = first_group; group <= last_group; ++group) {
+        sum += source[static_cast<std::size_t>(plan.slot(group, dealt_tile)) *
+                      kTileM * kTileN];
+    }
+    out[static_cast<std::size_t>(row) * shape.columns + column] = sum;
 }
 
 // out[i] = sum over slices of partial[slice][i], ascending.
@@ -349,6 +440,31 @@ hipError_t launch_dense_matmul(const float* left, const float* right,
             add_slices_kernel<<<(count + 255) / 256, 256, 0, stream>>>(
                 workspace, out, count, static_cast<unsigned>(slices));
             return hipSuccess;
+        }
+        if (batch_count == 1 && tiles < (1ULL << 24)) {
+            TilePlan plan;
+            plan.tiles_n = static_cast<unsigned>(tiles_n);
+            plan.steps = static_cast<unsigned>(steps);
+            const unsigned groups = plan_tiles(
+                plan, static_cast<unsigned>(tiles),
+                kTileM * kTileN * sizeof(float), kStreamWorkspaceBytes);
+            if (groups != 0) {
+                float* workspace = nullptr;
+                if (const hipError_t status =
+                        stream_workspace(stream, &workspace);
+                    status != hipSuccess) {
+                    return status;
+                }
+                dense_matmul_planned_kernel<<<plan.whole_tiles + groups,
+                                              kThreads, 0, stream>>>(
+                    left, right, out, workspace, shape, plan);
+                const dim3 parts(static_cast<unsigned>(tiles) -
+                                     plan.whole_tiles,
+                                 kTileM * kTileN / 256);
+                matmul_parts_kernel<<<parts, 256, 0, stream>>>(workspace, out,
+                                                               shape, plan);
+                return hipSuccess;
+            }
         }
         const dim3 grid(static_cast<unsigned>(tiles_n),
                         static_cast<unsigned>(tiles_m),

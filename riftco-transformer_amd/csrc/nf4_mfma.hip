@@ -38,6 +38,7 @@
 
 #include "kernels.hpp"
 #include "nf4_decode.hpp"
+#include "tile_plan.hpp"
 
 #include <algorithm>
 
@@ -61,32 +62,6 @@ struct GemmShape {
     unsigned input_width;  // I: the weight's row length
 };
 
-// How a launch covers the tile grid.  Tiles are numbered row-major (tile /
-// tiles_n is the tile row).  The first `whole_tiles` workgroups take one whole
-// tile each.  The tiles after those are cut into (tile, step) units -- one
-// contraction step of one tile, tile-major -- which are dealt to the remaining
-// workgroups in contiguous runs: the first `remainder` of them take
-// quotient + 1 units, the others quotient.  A run never exceeds one tile's
-// worth of steps, so it touches at most two tiles.  Whole-tile workgroups
-// come first in the grid and the shorter runs last, which is also the order
-// in which the device starts them.
-struct GemmPlan {
-    unsigned tiles_n;      // output tiles per tile row
-    unsigned whole_tiles;  // tiles computed by one workgroup each
-    unsigned steps;        // contraction steps per tile
-    unsigned quotient;
-    unsigned remainder;
-
-    __host__ __device__ unsigned begin(unsigned group) const {
-        return group * quotient + (group < remainder ? group : remainder);
-    }
-    __host__ __device__ unsigned owner(unsigned unit) const {
-        const unsigned boundary = remainder * (quotient + 1);
-        return unit < boundary ? unit / (quotient + 1)
-                               : remainder + (unit - boundary) / quotient;
-    }
-};
-constexpr unsigned kSlotsPerGroup = 2;  // partial tiles a workgroup may write
 
 // Registers holding one step's global loads of a thread.
 struct Staged {
@@ -416,7 +391,7 @@ template <bool kDoubleQuantized, bool kBackward>
 __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
     const float* __restrict__ activations, Nf4WeightView weight,
     const float* __restrict__ bias, float* __restrict__ result,
-    float* __restrict__ workspace, GemmShape shape, GemmPlan plan,
+    float* __restrict__ workspace, GemmShape shape, TilePlan plan,
     unsigned block_shift, LoraEpilogue lora
 ) {
     __shared__ __attribute__((aligned(16))) float a_tile[kTileM * kStride];
@@ -440,9 +415,9 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
         float* const partial =
             segment_steps == plan.steps
                 ? nullptr
-                : workspace + static_cast<std::size_t>(
-                                  group * kSlotsPerGroup + segment) *
-                                  kTileM * kTileN;
+                : workspace +
+                      static_cast<std::size_t>(group * 2 + segment) * kTileM *
+                          kTileN;
         gemm_segment<kDoubleQuantized, kBackward>(
             activations, weight, bias, result, partial, shape, block_shift,
             lora, a_tile, b_tile, table, (tile / plan.tiles_n) * kTileM,
@@ -458,7 +433,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
 // blockIdx.y a run of 256 elements of it.
 __global__ __launch_bounds__(256) void gemm_parts_kernel(
     const float* __restrict__ workspace, const float* __restrict__ bias,
-    float* __restrict__ result, GemmShape shape, GemmPlan plan,
+    float* __restrict__ result, GemmShape shape, TilePlan plan,
     LoraEpilogue lora
 ) {
     const unsigned dealt_tile = blockIdx.x;
@@ -480,11 +455,8 @@ __global__ __launch_bounds__(256) void gemm_parts_kernel(
     const float* source = workspace + m * kTileN + c;
     float sum = 0.0F;
     for (unsigned group = first_group; group <= last_group; ++group) {
-        // A workgroup's slot 0 holds the first tile of its run.
-        const unsigned slot =
-            group * kSlotsPerGroup +
-            (dealt_tile == plan.begin(group) / plan.steps ? 0U : 1U);
-        sum += source[static_cast<std::size_t>(slot) * kTileM * kTileN];
+        sum += source[static_cast<std::size_t>(plan.slot(group, dealt_tile)) *
+                      kTileM * kTileN];
     }
     if (bias != nullptr) {
         sum += bias[column];
@@ -495,13 +467,6 @@ __global__ __launch_bounds__(256) void gemm_parts_kernel(
     result[static_cast<std::size_t>(row) * shape.columns + column] = sum;
 }
 
-// Workgroups the device holds at once: two per compute unit.
-constexpr unsigned kPlaces = 512;
-// A unit-dealt run is at least this many steps (a quarter of a kilobyte of
-// codes per weight row), and unit dealing is not worth a second kernel when
-// the leftover tiles nearly fill the device anyway.
-constexpr unsigned kMinimumRunSteps = 8;
-
 template <bool kDoubleQuantized, bool kBackward>
 hipError_t launch_encoding(const LinearProblem& p, const GemmShape& shape,
                            hipStream_t stream) {
@@ -509,46 +474,24 @@ hipError_t launch_encoding(const LinearProblem& p, const GemmShape& shape,
     const unsigned tiles_m = (shape.rows + kTileM - 1) / kTileM;
     const unsigned tiles_n = (shape.columns + kTileN - 1) / kTileN;
     const unsigned tiles = tiles_m * tiles_n;
-    GemmPlan plan;
+    TilePlan plan;
     plan.tiles_n = tiles_n;
     plan.steps = (shape.contraction + kTileK - 1) / kTileK;
-    const unsigned leftover = tiles % kPlaces;
-    const bool deal_units = leftover != 0 && leftover * 10 < kPlaces * 9 &&
-                            plan.steps >= 2 * kMinimumRunSteps &&
-                            // partial tiles fit the workspace
-                            static_cast<std::size_t>(kPlaces) *
-                                    kSlotsPerGroup * kTileM * kTileN *
-                                    sizeof(float) <=
-                                kStreamWorkspaceBytes;
-    plan.whole_tiles = deal_units ? tiles - leftover : tiles;
-    plan.quotient = 0;
-    plan.remainder = 0;
-    if (!deal_units) {
-        kernel<<<tiles, kThreads, 0, stream>>>(
-            p.activations, p.weight, p.bias, p.result, nullptr, shape, plan,
-            p.block_shift, p.lora);
-        return hipSuccess;
-    }
+    const unsigned groups =
+        plan_tiles(plan, tiles, kTileM * kTileN * sizeof(float),
+                   kStreamWorkspaceBytes);
     float* workspace = nullptr;
-    if (const hipError_t status = stream_workspace(stream, &workspace);
-        status != hipSuccess) {
-        return status;
+    if (groups != 0) {
+        if (const hipError_t status = stream_workspace(stream, &workspace);
+            status != hipSuccess) {
+            return status;
+        }
     }
-    const unsigned units = leftover * plan.steps;
-    unsigned groups = units / kMinimumRunSteps;
-    if (groups > kPlaces) {
-        groups = kPlaces;
-    }
-    if (groups < leftover) {
-        groups = leftover;  // a run never exceeds one tile
-    }
-    plan.quotient = units / groups;
-    plan.remainder = units % groups;
     kernel<<<plan.whole_tiles + groups, kThreads, 0, stream>>>(
         p.activations, p.weight, p.bias, p.result, workspace, shape, plan,
         p.block_shift, p.lora);
-    if (groups != leftover) {  // some tile has parts
-        const dim3 grid(leftover, kTileM * kTileN / 256);
+    if (groups != 0) {
+        const dim3 grid(tiles - plan.whole_tiles, kTileM * kTileN / 256);
         gemm_parts_kernel<<<grid, 256, 0, stream>>>(
             workspace, p.bias, p.result, shape, plan, p.lora);
     }

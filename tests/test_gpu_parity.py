@@ -573,6 +573,9 @@ def test_lora_with_zero_b_equals_the_plain_forward(gpu, package, library,
     (1, 512, 2048, 1024),
     (1, 200, 1000, 260),    # sliced contraction, last slice ends mid-step
     (1, 2048, 4096, 16),    # sliced contraction, many row tiles
+    (1, 1280, 1024, 2560),  # 200 tiles dealt in runs to 512 workgroups
+    (1, 2200, 520, 3700),   # 522 tiles: 512 whole, 10 dealt; ragged edges
+    (2, 1280, 256, 1300),   # batched: whole tiles only
 ])
 def test_dense_matmul(gpu, package, library, oracle, batch, rows, shared,
                       columns):
