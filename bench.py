@@ -14,9 +14,9 @@ everything resident in HBM before the timed region.
 The same JSON line carries
   roofline      HBM roofline of the GEMV kernel (bytes per launch / average
                 launch duration from HIP events on the launch stream)
-  gemm          M = 2048 forward and input-backward GEMMs of BASELINE configs 4
-                and 5 with their fp32-MFMA rooflines
-  small_batch   M in {4, 16, 64} on the three distinct shapes (config 3)
+  gemm          M = 2048 forward and input-backward GEMMs (prefill / training
+                shapes) with their fp32-MFMA rooflines
+  small_batch   M in {1, 4, 16, 64} on the three distinct shapes
   lora          the fused bias + rank-16 adapter forward beside the plain one
   matmul        dense fp32 matmul at layer and adapter shapes
   quantizer     the device quantizer on one 11008 x 4096 weight (wall clock,
@@ -173,7 +173,7 @@ DOMINANT_KERNEL_HBM_BYTES = int((7303.0 * 2.00 + 25.0) * 1024)
 
 
 def bench_gemm(package, device, torch, steps):
-    """BASELINE configs 4 and 5: M = 2048."""
+    """Prefill / training forward and the input backward: M = 2048."""
     rows = 2048
     results = []
     cases = [
@@ -214,7 +214,7 @@ def bench_gemm(package, device, torch, steps):
 
 
 def bench_small_batch(package, device, torch, steps):
-    """BASELINE config 3: M in {4, 16, 64}, fp32 scales; rotating weights."""
+    """Small-batch decode: M in {1, 4, 16, 64}, fp32 scales; rotating weights."""
     results = []
     copies = 12  # 12 x >= 9.4 MB per shape: beyond the last-level cache
     for name, out_w, in_w in (LAYER_SHAPES[0], LAYER_SHAPES[4],

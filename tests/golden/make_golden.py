@@ -67,7 +67,7 @@ def closed_form(reference) -> dict:
 
 
 def config1(reference):
-    """BASELINE config 1: x [16,256] ~N(0,1), W [768,256] ~N(0,0.02), block 64,
+    """The tiny parity configuration: x [16,256] ~N(0,1), W [768,256] ~N(0,0.02), block 64,
     bias [768] ~N(0,0.01); plus an upstream [16,768] ~N(0,1e-2) for backward."""
     x = helpers.normal(1, (16, 256), 1.0)
     dense = helpers.normal(2, (768, 256), 0.02)

@@ -154,7 +154,8 @@ def test_reference_fixtures(gpu, package, library, oracle, name,
 @pytest.mark.parametrize("double_quantized", [False, True])
 def test_config1_tiny_layer_with_bias(gpu, package, library, oracle,
                                       double_quantized):
-    """BASELINE config 1 against the compiled reference's stored outputs."""
+    """The tiny parity configuration (x [16, 256], W [768, 256], bias) against
+    the compiled reference's stored outputs."""
     golden = np.load(os.path.join(GOLDEN, "config1.npz"))
     x = helpers.normal(1, (16, 256), 1.0)
     dense = helpers.normal(2, (768, 256), 0.02)
@@ -390,7 +391,7 @@ def test_zero_scale_blocks_and_saturated_scales(gpu, package, library,
     (4096, 11008, True)])
 def test_prefill_shapes_at_full_size(gpu, package, library, oracle, out_w,
                                      in_w, double_quantized):
-    """M = 2048 at BASELINE's shapes.  Size-independent checks: every output
+    """M = 2048 at the Llama-7B layer shapes.  Size-independent checks: every output
     against an fp64 product over the bit-exact deq(W) (computed on the device
     by the vendor BLAS, an independent path), 32 seeded rows against the CPU
     oracle, and linearity y(a*x1 + x2) = a*y(x1) + y(x2) for a power of two."""

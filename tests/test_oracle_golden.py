@@ -128,7 +128,7 @@ def test_llama_rows(oracle, digests, name, out_w, in_w, seed,
 
 
 def test_payload_bytes_match_the_published_figures(oracle, digests):
-    # BASELINE: 9 437 184 / 25 362 432 B (fp32 scales), 8 654 852 /
+    # expected: 9 437 184 / 25 362 432 B (fp32 scales), 8 654 852 /
     # 23 259 908 B (double-quantised, C = 256).
     llama = digests["llama"]
     assert llama["q_proj"]["fp32"]["payload_bytes"] == 9437184
