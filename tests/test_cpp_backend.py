@@ -87,6 +87,18 @@ def test_packed_state_reader_fails_as_the_reference_reader_does(tmp_path):
         assert [kind, rest] == [want[0], str(want[1])], name
 
 
+def test_work_split_of_the_tiled_kernels():
+    """Host arithmetic of tile_plan.hpp: runs cover every unit once, never
+    exceed a tile, slots are unique (tests/cpp/test_tile_plan.cpp)."""
+    binary = os.path.join(BUILD, "test_tile_plan")
+    assert os.path.exists(binary), \
+        "tests/cpp/build/test_tile_plan is not built (make -C tests/cpp)"
+    result = subprocess.run([binary], capture_output=True, text=True,
+                            timeout=120)
+    assert result.returncode == 0, result.stdout + result.stderr
+    assert "tile plan tests passed" in result.stdout
+
+
 def test_unavailable_when_the_runtime_sees_no_device():
     result = run(["--expect-unavailable"],
                  RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE, FAKE_RTHIP_NO_DEVICE="1")
