@@ -362,12 +362,34 @@ def cpu_baseline(budget_seconds=12.0):
         seconds = time.perf_counter() - begin
         if seconds >= budget_seconds:
             break
+    # The M = 2048 products would take minutes per call on one core: time a
+    # few rows of the same shapes and scale linearly (the reference loops are
+    # linear in the row count).
+    gate, _ = layer[4]
+    prefill = {}
+    for name, rows, run in (
+            ("forward_11008x4096", 4,
+             lambda x: backend.forward(x, gate, faithful=True)),
+            ("input_backward_11008x4096", 2,
+             lambda dy: backend.input_backward(dy, gate, faithful=True))):
+        width = gate.input_width if name.startswith("forward") \
+            else gate.output_width
+        sample = rng.standard_normal((rows, width), dtype=np.float32)
+        start = time.perf_counter()
+        run(sample)
+        elapsed = time.perf_counter() - start
+        macs = rows * gate.output_width * gate.input_width
+        prefill[name] = {
+            "rows_timed": rows, "gmac_per_s": macs / elapsed / 1e9,
+            "seconds_for_2048_rows_extrapolated": elapsed * 2048 / rows,
+        }
     return {
         "value": total_bytes / seconds / 1e9, "unit": "GB/s", "cores": 1,
         "kind": backend.kind, "seconds": seconds,
         "sample": "%d passes over one Llama-7B layer (7 projections at M=1, "
                   "fp32 scales, %.1f MB packed per pass)"
                   % (passes, total_bytes / passes / 1e6),
+        "prefill": prefill,
     }
 
 
