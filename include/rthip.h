@@ -81,8 +81,9 @@ enum {
     /* small batches (forward, up to 64 rows): weights decoded straight into
      * MFMA operands, no LDS tile */
     RTHIP_NF4_ALGORITHM_SKINNY = 4,
-    /* up to 16 rows (forward) with a row width of 1024..4096: like SKINNY, but
-     * x stays in registers and the wavefronts split the contraction axis */
+    /* up to 64 rows (forward) with a row width of 1024..4096: like SKINNY, but
+     * x stays in registers, 16 rows per workgroup, and the wavefronts split
+     * the contraction axis */
     RTHIP_NF4_ALGORITHM_RESIDENT = 5
 };
 

@@ -54,8 +54,8 @@ hipError_t stream_workspace(hipStream_t stream, float** out);
 // operands.  Shapes whose output tiles are shared between workgroups use a
 // per-stream workspace that is allocated on first use, so the launcher can
 // fail.
-// nf4_resident.hip: up to 16 rows, x resident in registers
-constexpr std::size_t kResidentMaxRows = 16;
+// nf4_resident.hip: up to 64 rows in groups of 16, x resident in registers
+constexpr std::size_t kResidentMaxRows = 64;
 bool resident_forward_supports(const LinearProblem& problem);
 hipError_t launch_resident_forward(const LinearProblem& problem,
                                    hipStream_t stream);

@@ -1,4 +1,4 @@
-// Forward product for up to 16 rows when a row of the weight is short enough
+// Forward product for up to 64 rows when a row of the weight is short enough
 // for x to live in registers (row width 1024, 2048, 3072 or 4096):
 //     y[r, o] = sum_i x[r, i] * codebook[code(o, i)] * scale(o, i / B)
 // restating reference_quantized_linear_forward
@@ -31,10 +31,16 @@
 //     ones.
 //   * Tiles are dealt round-robin to one persistent workgroup per compute
 //     unit; the codes of tile t + 1 are requested before tile t is computed.
-//   * A wavefront parks its 16 x 16 partial tile in LDS; after the ONLY
-//     barrier, at the end of the kernel, the workgroup adds the eight partial
-//     tiles of each of its output tiles in wavefront order and writes y with
-//     bias and adapter term.  Nothing depends on scheduling.
+//   * More than 16 rows of x are handled as up to four row groups of 16: a
+//     workgroup holds ONE row group for its whole life, and the work items
+//     (tile, row group) are numbered so that the row groups of a tile go to
+//     workgroups eight apart in the grid -- the same XCD, in the same round of
+//     the dispatch -- which read the tile's weights at about the same time, so
+//     the weights come from HBM once and from that XCD's L2 for the others.
+//   * A wavefront parks its 16 x 16 partial tile in LDS; every four tiles
+//     (and at the end) the workgroup meets at a barrier, adds the eight
+//     partial tiles of each parked output tile in wavefront order and writes y
+//     with bias and adapter term.  Nothing depends on scheduling.
 
 #include "kernels.hpp"
 #include "nf4_decode.hpp"
@@ -52,7 +58,7 @@ constexpr int kTileRows = 16;        // weight rows per tile
 constexpr int kGroupWeights = 128;   // contraction values per wavefront group
 constexpr int kLaneWeights = 32;     // of which one lane owns this many
 constexpr unsigned kComputeUnits = 256;
-constexpr unsigned kMaxIterations = 8;  // tiles one workgroup may park
+constexpr unsigned kParkTiles = 4;  // tiles a workgroup parks between flushes
 // Per-wavefront LDS area that x passes through on its way into registers:
 // [16 rows][128 values], rows padded by four floats.
 constexpr unsigned kStagingStride = kGroupWeights + 4;
@@ -73,7 +79,7 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
     const float* __restrict__ x, Nf4WeightView weight,
     const float* __restrict__ bias, float* __restrict__ y, unsigned rows,
     unsigned output_width, unsigned block_shift, unsigned tile_count,
-    unsigned iterations, LoraEpilogue lora
+    unsigned row_groups, unsigned iterations, LoraEpilogue lora
 ) {
     constexpr unsigned kInputWidth = 1024U * kGroups;
     constexpr int kSubChunks = 2 * kGroups;  // 16 weights each
@@ -93,6 +99,15 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
     // first contraction value of this lane in group 0
     const unsigned k_base =
         wave * (kInputWidth / kWaves) + quarter * kLaneWeights;
+    // Work item w = blockIdx.x + i * gridDim.x of iteration i is tile
+    // 8 (w / (8 G)) + w % 8 and row group (w / 8) % G.  The grid is a multiple
+    // of 8 G, so the row group is the same in every iteration.
+    const unsigned row_base = (blockIdx.x / 8) % row_groups * kTileRows;
+    const unsigned rows_here = min(rows - row_base, 16U);
+    const auto tile_of = [&](unsigned iteration) {
+        const unsigned item = blockIdx.x + iteration * gridDim.x;
+        return item / (8 * row_groups) * 8 + item % 8;
+    };
 
     const std::size_t elements =
         static_cast<std::size_t>(output_width) * kInputWidth;  // < 2^32
@@ -152,10 +167,8 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
         }
     };
 
-    // Tiles are dealt round-robin: iteration i of workgroup b takes tile
-    // b + i * gridDim.x.
     Codes ring[2];
-    load_codes(ring[0], blockIdx.x);
+    load_codes(ring[0], tile_of(0));
 
     // This lane's slice of x: row lane % 16, resident for the whole kernel.
     // A lane's values are 128 contiguous bytes of one x row, and the 16 rows
@@ -180,8 +193,8 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
                     floatx4,
                     __builtin_amdgcn_raw_buffer_load_b128(
                         x_buffer,
-                        row < rows
-                            ? (row * kInputWidth +
+                        row < rows_here
+                            ? ((row_base + row) * kInputWidth +
                                wave * (kInputWidth / kWaves) +
                                kGroupWeights * g + piece_column) *
                                   static_cast<unsigned>(sizeof(float))
@@ -269,47 +282,62 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        parked[(iteration * kWaves + wave) * 64 + lane] = acc;
+        parked[((iteration % kParkTiles) * kWaves + wave) * 64 + lane] = acc;
+    };
+
+    // Adds the eight wavefront partials of the tiles parked since the last
+    // flush, in wavefront order, and writes y with bias and adapter term.
+    // Accumulator element r of lane l is x row 4 (l / 16) + r and weight row
+    // l % 16 of the tile.
+    const auto flush = [&](unsigned first_iteration, unsigned count) {
+        __syncthreads();  // every wavefront has parked these tiles
+        for (unsigned index = thread; index < count * 256;
+             index += kThreads) {
+            const unsigned iteration = first_iteration + index / 256;
+            const unsigned m = (index % 256) / 16;
+            const unsigned column = index % 16;
+            const unsigned tile = tile_of(iteration);
+            const unsigned n = tile * kTileRows + column;
+            if (tile >= tile_count || n >= output_width || m >= rows_here) {
+                continue;
+            }
+            const float* source =
+                reinterpret_cast<const float*>(
+                    parked + (iteration % kParkTiles) * kWaves * 64 +
+                    (m / 4) * 16 + column) +
+                m % 4;
+            float sum = 0.0F;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                sum += source[w * 64 * 4];  // wavefront order
+            }
+            if (bias != nullptr) {
+                sum += bias[n];
+            }
+            if (lora.reduced != nullptr) {
+                sum += lora_term(lora, row_base + m, n);
+            }
+            y[static_cast<std::size_t>(row_base + m) * output_width + n] =
+                sum;
+        }
+        __syncthreads();  // the parking slots are free again
     };
 
     issue_lookups(ring[0], 0);
     for (unsigned iteration = 0; iteration < iterations; iteration += 2) {
-        load_codes(ring[1], blockIdx.x + (iteration + 1) * gridDim.x);
+        load_codes(ring[1], tile_of(iteration + 1));
         compute(ring[0], ring[1], iteration);
         if (iteration + 1 < iterations) {  // uniform
-            load_codes(ring[0], blockIdx.x + (iteration + 2) * gridDim.x);
+            load_codes(ring[0], tile_of(iteration + 2));
             compute(ring[1], ring[0], iteration + 1);
         }
-    }
-
-    // The only barrier after the table build.  Accumulator element r of lane
-    // l is x row 4 (l / 16) + r and weight row l % 16 of the tile.
-    __syncthreads();
-    for (unsigned index = thread; index < iterations * 256; index += kThreads) {
-        const unsigned iteration = index / 256;
-        const unsigned m = (index % 256) / 16;
-        const unsigned column = index % 16;
-        const unsigned tile = blockIdx.x + iteration * gridDim.x;
-        const unsigned n = tile * kTileRows + column;
-        if (tile >= tile_count || n >= output_width || m >= rows) {
-            continue;
+        // The only barriers after the table build: one pair per kParkTiles
+        // tiles.
+        const unsigned done = min(iteration + 2, iterations);
+        if (done % kParkTiles == 0 || done == iterations) {  // uniform
+            const unsigned first = (done - 1) / kParkTiles * kParkTiles;
+            flush(first, done - first);
         }
-        const float* source = reinterpret_cast<const float*>(
-                                  parked + iteration * kWaves * 64 +
-                                  (m / 4) * 16 + column) +
-                              m % 4;
-        float sum = 0.0F;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            sum += source[w * 64 * 4];  // wavefront order
-        }
-        if (bias != nullptr) {
-            sum += bias[n];
-        }
-        if (lora.reduced != nullptr) {
-            sum += lora_term(lora, m, n);
-        }
-        y[static_cast<std::size_t>(m) * output_width + n] = sum;
     }
 }
 
@@ -317,18 +345,19 @@ template <int kGroups, bool kDoubleQuantized>
 hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     const unsigned tiles = static_cast<unsigned>(
         (p.output_width + kTileRows - 1) / kTileRows);
-    // One workgroup per compute unit, more only if a workgroup would
-    // otherwise have to park more tiles than it has room for.
-    unsigned groups = tiles < kComputeUnits ? tiles : kComputeUnits;
-    unsigned iterations = (tiles + groups - 1) / groups;
-    if (iterations > kMaxIterations) {
-        iterations = kMaxIterations;
-        groups = (tiles + iterations - 1) / iterations;
+    const unsigned row_groups =
+        static_cast<unsigned>((p.rows + kTileRows - 1) / kTileRows);
+    // Work items (tile, row group), tiles padded to a multiple of eight.  One
+    // workgroup per compute unit, rounded down to a multiple of 8 x row
+    // groups so that a workgroup keeps its row group.
+    const unsigned items = (tiles + 7) / 8 * 8 * row_groups;
+    const unsigned granule = 8 * row_groups;
+    unsigned groups = kComputeUnits / granule * granule;
+    if (groups > items) {
+        groups = items;
     }
-    const std::size_t parked_bytes =
-        static_cast<std::size_t>(iterations) * kWaves * 64 * sizeof(floatx4);
-    const std::size_t shared_bytes =
-        parked_bytes > kStagingBytes ? parked_bytes : kStagingBytes;
+    const unsigned iterations = (items + groups - 1) / groups;
+    const std::size_t shared_bytes = kStagingBytes;
     const auto kernel = resident_forward_kernel<kGroups, kDoubleQuantized>;
     // More than the default 64 KB of LDS.
     static const hipError_t configured = hipFuncSetAttribute(
@@ -336,14 +365,14 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
         hipFuncAttributeMaxDynamicSharedMemorySize,
         static_cast<int>(kStagingBytes));
     static_assert(kStagingBytes >=
-                  kMaxIterations * kWaves * 64 * sizeof(floatx4));
+                  kParkTiles * kWaves * 64 * sizeof(floatx4));
     if (configured != hipSuccess) {
         return configured;
     }
     kernel<<<groups, kThreads, shared_bytes, stream>>>(
         p.activations, p.weight, p.bias, p.result,
         static_cast<unsigned>(p.rows), static_cast<unsigned>(p.output_width),
-        p.block_shift, tiles, iterations, p.lora);
+        p.block_shift, tiles, row_groups, iterations, p.lora);
     return hipSuccess;
 }
 

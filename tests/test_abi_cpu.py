@@ -48,14 +48,16 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(fwd, 2048, 4096, 11008, 64) == package.ALGORITHM_MFMA
     # small batches -> weights decoded straight into MFMA operands
     assert select(fwd, 16, 256, 768, 64) == package.ALGORITHM_SKINNY
-    assert select(fwd, 64, 4096, 11008, 64) == package.ALGORITHM_SKINNY
+    assert select(fwd, 64, 11008, 4096, 64) == package.ALGORITHM_SKINNY
     assert select(fwd, 65, 4096, 11008, 64) == package.ALGORITHM_MFMA
     assert select(fwd, 16, 128, 768, 32) == package.ALGORITHM_SKINNY
-    # up to 16 rows and a row width of 1024..4096 -> x resident in registers
+    # up to 64 rows and a row width of 1024..4096 -> x resident in registers
     assert select(fwd, 16, 4096, 11008, 64) == package.ALGORITHM_RESIDENT
     assert select(fwd, 5, 4096, 4096, 64) == package.ALGORITHM_RESIDENT
     assert select(fwd, 8, 3072, 1000, 32) == package.ALGORITHM_RESIDENT
-    assert select(fwd, 17, 4096, 4096, 64) == package.ALGORITHM_SKINNY
+    assert select(fwd, 17, 4096, 4096, 64) == package.ALGORITHM_RESIDENT
+    assert select(fwd, 64, 4096, 11008, 64) == package.ALGORITHM_RESIDENT
+    assert select(fwd, 65, 4096, 11008, 64) == package.ALGORITHM_MFMA
     assert select(fwd, 16, 11008, 4096, 64) == package.ALGORITHM_SKINNY
     assert select(fwd, 16, 5120, 4096, 64) == package.ALGORITHM_SKINNY
     # (row width a multiple of 32 but not of 64 -> tiled GEMM)

@@ -281,16 +281,17 @@ def test_small_batch_work_split(gpu, package, library, oracle, out_w, in_w,
 ])
 def test_resident_small_batch_family(gpu, package, library, oracle, out_w,
                                      in_w, block, second, double_quantized):
-    """Up to 16 rows with x resident in registers: every row count from the
-    GEMV's to the family's limit, with bias, against the oracle, fp64 and the
-    other families (check_layer runs each that accepts the shape)."""
+    """Up to 64 rows, in row groups of 16, with x resident in registers: row
+    counts from the GEMV's to the family's limit (one to four row groups, full
+    and partly empty), with bias, against the oracle, fp64 and the other
+    families (check_layer runs each that accepts the shape)."""
     dense = helpers.normal(73, (out_w, in_w), 0.02)
     dense[1] = 0.0
     weight = oracle.quantize(dense, block, double_quantized, second)
-    assert library.select_algorithm(package.FORWARD, 16, in_w, out_w,
+    assert library.select_algorithm(package.FORWARD, 64, in_w, out_w,
                                     block) == package.ALGORITHM_RESIDENT
     bias = helpers.normal(74, (out_w,), 0.01)
-    for rows in (1, 5, 11, 16):
+    for rows in (1, 5, 16, 17, 33, 48, 64):
         x = helpers.normal(75 + rows, (rows, in_w), 1.0)
         dy = helpers.normal(76 + rows, (rows, out_w), 1.0e-2)
         check_layer(gpu, package, library, oracle, weight, x, dy, bias=bias,
@@ -880,16 +881,21 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
     bias = to_device(helpers.normal(161, (1000,), 0.01))
     lora_a = to_device(helpers.normal(162, (8, 2048), 0.05))
     lora_b = to_device(helpers.normal(163, (1000, 8), 0.05))
-    row_counts = {"gemv": 2, "resident": 9, "skinny": 40, "mfma": 130}
+    # name -> (rows, pinned family or None for the automatic choice)
+    launches = {"gemv": (2, None), "resident": (9, None),
+                "resident, three row groups": (40, None),
+                "skinny": (40, package.ALGORITHM_SKINNY), "mfma": (130, None)}
     inputs = {name: torch.zeros((rows, 2048), device="cuda")
-              for name, rows in row_counts.items()}
+              for name, (rows, _) in launches.items()}
     upstream = torch.zeros((130, 1000), device="cuda")
-    for name, rows in row_counts.items():
-        assert package.ALGORITHM_NAMES[library.select_algorithm(
-            package.FORWARD, rows, 2048, 1000, 64)] == name
+    for name, (rows, family) in launches.items():
+        if family is None:
+            assert package.ALGORITHM_NAMES[library.select_algorithm(
+                package.FORWARD, rows, 2048, 1000, 64)] == name.split(",")[0]
 
     def launch_all():
-        outputs = {name: gpu.linear_forward(x, device_weight, bias)
+        outputs = {name: gpu.linear_forward(x, device_weight, bias,
+                                            algorithm=launches[name][1])
                    for name, x in inputs.items()}
         outputs["adapter"], _ = gpu.lora_linear_forward(
             inputs["resident"], device_weight, lora_a, lora_b, 0.5, bias)
