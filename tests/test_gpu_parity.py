@@ -373,6 +373,24 @@ def test_gemm_leftover_tiles_are_dealt_in_units(gpu, package, library, oracle,
             host(gpu.linear_forward(to_device(x), device_weight)), first)
 
 
+@pytest.mark.parametrize("out_w,in_w", [(4096, 4096), (11008, 4096),
+                                        (4096, 11008)])
+@pytest.mark.parametrize("double_quantized", [False, True])
+def test_small_batches_at_the_llama_shapes(gpu, package, library, oracle,
+                                           out_w, in_w, double_quantized):
+    """The small-batch decode configuration at full size: M in {4, 16, 64} on
+    the three distinct Llama-7B projection shapes, both scale encodings; every
+    family that takes the shape, every output against fp64, two rows against
+    the CPU oracle."""
+    weight = oracle.quantize(helpers.normal(99, (out_w, in_w), 0.02), 64,
+                             double_quantized, 256)
+    for rows in (4, 16, 64):
+        x = helpers.normal(100 + rows, (rows, in_w), 1.0)
+        dy = helpers.normal(101 + rows, (rows, out_w), 1.0e-2)
+        check_layer(gpu, package, library, oracle, weight, x, dy,
+                    oracle_rows=2)
+
+
 def test_zero_scale_blocks_and_saturated_scales(gpu, package, library,
                                                 oracle):
     dense = helpers.normal(70, (64, 128), 0.02)
