@@ -14,6 +14,8 @@ everything resident in HBM before the timed region.
 The same JSON line carries
   roofline      HBM roofline of the GEMV kernel (bytes per launch / average
                 launch duration from HIP events on the launch stream)
+  decode_double_quantized_scales
+                the decode step again with the nested scale encoding
   gemm          M = 2048 forward and input-backward GEMMs (prefill / training
                 shapes) with their fp32-MFMA rooflines
   small_batch   M in {1, 4, 16, 64} on the three distinct shapes
@@ -98,13 +100,15 @@ def time_region(torch, body, repeats):
     return start.elapsed_time(stop)
 
 
-def bench_decode(package, device, torch, layers, steps, warmup, use_graph):
+def bench_decode(package, device, torch, layers, steps, warmup, use_graph,
+                 double_quantized=False):
     library = package.load_library()
     weights = []
     for layer in range(layers):
         for index, (_, out_w, in_w) in enumerate(LAYER_SHAPES):
             weights.append(synthetic_weight(package, torch, out_w, in_w,
-                                            False, 1000 * layer + index))
+                                            double_quantized,
+                                            1000 * layer + index))
     x = {width: torch.randn(1, width, device="cuda")
          for width in (4096, 11008)}
     y = {width: torch.empty(1, width, device="cuda")
@@ -477,6 +481,18 @@ def main():
         "roofline": decode["roofline"],
     }
     if not arguments.skip_extras:
+        del decode
+        # The same decode step with the reference's double-quantised scale
+        # encoding (3.36 GB of packed payload per step instead of 3.64).
+        nested = bench_decode(package, device, torch, arguments.layers,
+                              max(3, arguments.steps // 2), arguments.warmup,
+                              not arguments.no_graph, double_quantized=True)
+        line["decode_double_quantized_scales"] = {
+            "value": nested["value"], "unit": "GB/s",
+            "ms_per_step": nested["ms_per_step"],
+            "bytes_per_step": nested["bytes_per_step"],
+        }
+        del nested
         line["gemm"] = bench_gemm(package, device, torch,
                                   max(3, arguments.steps // 4))
         line["small_batch"] = bench_small_batch(package, device, torch,

@@ -143,10 +143,18 @@ __device__ __forceinline__ unsigned slot_of_lane(unsigned lane) {
 
 typedef unsigned uint2_vec __attribute__((ext_vector_type(2)));
 
-template <int kRows, int kSegments>
+// Shared scale loads per batch (nested scale encoding): one covers every
+// (row, block) of the batch that a wavefront touches, except for block size
+// 32, which needs two.
+constexpr int kScaleLoads = 2;
+
+// kShared false: the scale of this lane's weights of every row.  kShared true:
+// the scale of ONE (row, block) pair per lane and load; the lanes that need it
+// fetch it from this lane (see scale_of below).
+template <int kRows, int kSegments, bool kShared>
 struct RowBatch {
     uint2_vec codes[kRows][kSegments];
-    float scales[kRows][kSegments];
+    float scales[kShared ? kScaleLoads : kRows][kSegments];
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base,
@@ -156,6 +164,8 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base,
                                              static_cast<int>(bytes),
                                              0x00020000);
 }
+
+static_assert(RTHIP_GEMV_ROWS <= 4, "one scale load covers four rows");
 
 // kX: x rows held per thread (1, 2 or 4; a 3-row call runs as 4 with a zero
 // row).  kSegments: segments per thread.  kRows: weight rows per batch.
@@ -194,8 +204,33 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
     const unsigned row_blocks = input_width >> block_shift;
     const __amdgpu_buffer_rsrc_t secondary_buffer =
         make_buffer(weight.secondary_scales, secondary_bytes);
-    const std::uint8_t* const primary_bytes =
-        static_cast<const std::uint8_t*>(weight.primary_scales);
+    // Plain fp32 scales are loaded by the lane that uses them, one per row
+    // and stripe.  For the nested encoding that would mean two loads and a
+    // decode (with a division) per row, which nearly doubles the kernel's
+    // work, so those are shared: a wavefront's 64 segments of a row span 1024
+    // weights = P = max(1, 1024 / B) quantisation blocks, the kRows rows of a
+    // batch need only kRows x P scales per wavefront, lane l of load q fetches
+    // and decodes the scale of row q x (64 / P) + l / P, block l % P of the
+    // wavefront's range, and the lanes that own weights of that block read it
+    // from lane l with one ds_bpermute: one decode per lane and batch instead
+    // of kRows.  (Sharing plain fp32 scales the same way measured 2-4 %
+    // slower than loading them: the ds_bpermute costs more than the load it
+    // replaces.)  The range check of the whole-array descriptor rejects rows
+    // past the output width.
+    const unsigned block_total =
+        (output_width * input_width) >> block_shift;  // < 2^32 / 32
+    const __amdgpu_buffer_rsrc_t primary_buffer = make_buffer(
+        weight.primary_scales, kDoubleQuantized ? block_total : 0U);
+    // lanes per block (log2), blocks per wavefront-row (log2), rows per load
+    const unsigned lanes_shift = block_shift - 4;
+    const unsigned p_shift = lanes_shift < 6 ? 6 - lanes_shift : 0;
+    const unsigned rows_per_load = 64U >> p_shift;
+    const unsigned my_row = lane >> p_shift;          // within a load
+    const unsigned my_block = lane & ((1U << p_shift) - 1);
+    // lane that holds the scale of MY weights of row r of a load
+    const unsigned my_source =
+        (lanes_shift < 6 ? (lane >> lanes_shift) : 0U) * 4;  // byte address
+    const unsigned wave_in_team = thread / kWave;
 
     // Per-lane constants: where this thread's segments sit inside a row.  The
     // row width is a multiple of the block size, so a row starts on a block
@@ -206,50 +241,86 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
         segment_weights[j] = (thread + kTeamThreads * j) * kSegment;
     }
 
-    const auto load_batch = [&](RowBatch<kRows, kSegments>& batch,
-                                unsigned batch_index) {
+    using Batch = RowBatch<kRows, kSegments, kDoubleQuantized>;
+    const auto load_batch = [&](Batch& batch, unsigned batch_index) {
 #pragma unroll
         for (int row = 0; row < kRows; ++row) {
             const unsigned o = batch_index * kRows + row;  // scalar
             const bool row_valid = o < output_width;
             const std::size_t row_start =
                 static_cast<std::size_t>(o) * input_width;
-            const std::size_t row_block = row_start >> block_shift;
             const __amdgpu_buffer_rsrc_t code_row = make_buffer(
                 weight.codes + (row_start >> 1),
                 row_valid ? row_code_bytes : 0U);
-            constexpr unsigned kScaleBytes = kDoubleQuantized ? 1 : 4;
-            const __amdgpu_buffer_rsrc_t primary_row = make_buffer(
-                primary_bytes + row_block * kScaleBytes,
-                row_valid ? row_blocks * kScaleBytes : 0U);
+            const __amdgpu_buffer_rsrc_t scale_row = make_buffer(
+                static_cast<const float*>(weight.primary_scales) +
+                    (row_start >> block_shift),
+                row_valid && !kDoubleQuantized ? row_blocks * 4 : 0U);
 #pragma unroll
             for (int j = 0; j < kSegments; ++j) {
                 batch.codes[row][j] = __builtin_amdgcn_raw_buffer_load_b64(
                     code_row, segment_weights[j] >> 1, 0, 0);
-                const unsigned segment_block =
-                    segment_weights[j] >> block_shift;
                 if constexpr (!kDoubleQuantized) {
                     batch.scales[row][j] = __builtin_bit_cast(
-                        float, __builtin_amdgcn_raw_buffer_load_b32(
-                                   primary_row, segment_block * 4, 0, 0));
-                } else {
+                        float,
+                        __builtin_amdgcn_raw_buffer_load_b32(
+                            scale_row,
+                            (segment_weights[j] >> block_shift) * 4, 0, 0));
+                }
+            }
+        }
+        if constexpr (!kDoubleQuantized) {
+            return;
+        }
+#pragma unroll
+        for (int q = 0; q < kScaleLoads; ++q) {
+            if (q * rows_per_load >= static_cast<unsigned>(kRows)) {
+                break;  // uniform: only block size 32 needs the second load
+            }
+            const unsigned row_in_batch = q * rows_per_load + my_row;
+            const unsigned o = batch_index * kRows + row_in_batch;
+            const bool mine = row_in_batch < static_cast<unsigned>(kRows) &&
+                              o < output_width;
+#pragma unroll
+            for (int j = 0; j < kSegments; ++j) {
+                // first weight of this wavefront's segments of stripe j
+                const unsigned wave_first =
+                    (wave_in_team * kWave + kTeamThreads * j) * kSegment;
+                const unsigned block =
+                    o * row_blocks + (wave_first >> block_shift) + my_block;
+                const unsigned offset = mine ? block : 0x80000000U;
+                {
                     const std::uint8_t scale_code =
-                        __builtin_amdgcn_raw_buffer_load_b8(
-                            primary_row, segment_block, 0, 0);
-                    // Rows past the output width get an index past the end
-                    // of the table, which reads as zero.
-                    const unsigned group =
-                        row_valid ? static_cast<unsigned>(
-                                        (row_block + segment_block) >>
-                                        weight.second_level_shift)
-                                  : 0x3FFFFFFFU;
+                        __builtin_amdgcn_raw_buffer_load_b8(primary_buffer,
+                                                            offset, 0, 0);
                     const float second = __builtin_bit_cast(
-                        float, __builtin_amdgcn_raw_buffer_load_b32(
-                                   secondary_buffer, group * 4, 0, 0));
-                    batch.scales[row][j] = decode_double_quantized_scale(
+                        float,
+                        __builtin_amdgcn_raw_buffer_load_b32(
+                            secondary_buffer,
+                            mine ? (block >> weight.second_level_shift) * 4
+                                 : 0x80000000U,
+                            0, 0));
+                    batch.scales[q][j] = decode_double_quantized_scale(
                         scale_code, second, weight.offset);
                 }
             }
+        }
+    };
+    // The scale of this lane's weights of row `row` (of the batch), stripe j.
+    const auto scale_of = [&](const Batch& batch, int row, int j) {
+        if constexpr (!kDoubleQuantized) {
+            return batch.scales[row][j];
+        } else {
+            const unsigned q = static_cast<unsigned>(row) / rows_per_load;
+            const unsigned row_in_load =
+                static_cast<unsigned>(row) % rows_per_load;
+            const float held =
+                q == 0 ? batch.scales[0][j] : batch.scales[1][j];
+            return __builtin_bit_cast(
+                float, __builtin_amdgcn_ds_bpermute(
+                           static_cast<int>(((row_in_load << p_shift) * 4) +
+                                            my_source),
+                           __builtin_bit_cast(int, held)));
         }
     };
 
@@ -261,7 +332,7 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
     // A ring of register batches: batch i lives in slot i % kDepth and is
     // requested kDepth - 1 batches before it is used.  (Loads past the last
     // batch are range-checked to zero by the buffer descriptor.)
-    RowBatch<kRows, kSegments> ring[kDepth];
+    Batch ring[kDepth];
 #pragma unroll
     for (int d = 0; d < kDepth - 1; ++d) {
         load_batch(ring[d], first_batch + d * stride);
@@ -315,8 +386,8 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
 
     // One batch: refill the slot freed by the previous batch, compute
     // `current`, reduce, park.
-    const auto step = [&](const RowBatch<kRows, kSegments>& current,
-                          RowBatch<kRows, kSegments>& refill,
+    const auto step = [&](const Batch& current,
+                          Batch& refill,
                           unsigned iteration) {
         const unsigned batch_index = first_batch + iteration * stride;
         if (iteration + kDepth - 1 < iterations) {
@@ -357,6 +428,11 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
             for (int r = 0; r < kX; ++r) {
                 row_acc[r] = 0.0F;
             }
+            float row_scale[kSegments];
+#pragma unroll
+            for (int j = 0; j < kSegments; ++j) {
+                row_scale[j] = scale_of(current, row, j);
+            }
 #pragma unroll
             for (int j = 0; j < kSegments; ++j) {
                 float even[kX];
@@ -377,7 +453,7 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
                 }
 #pragma unroll
                 for (int r = 0; r < kX; ++r) {
-                    row_acc[r] += (even[r] + odd[r]) * current.scales[row][j];
+                    row_acc[r] += (even[r] + odd[r]) * row_scale[j];
                 }
             }
 #pragma unroll
