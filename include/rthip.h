@@ -41,7 +41,7 @@ extern "C" {
 #endif
 
 #define RTHIP_ABI_VERSION_MAJOR 1u
-#define RTHIP_ABI_VERSION_MINOR 2u
+#define RTHIP_ABI_VERSION_MINOR 3u
 
 typedef int32_t rthip_status;
 
@@ -167,6 +167,35 @@ rthip_status rthip_nf4_linear_input_backward(
     uint64_t second_level_block, float offset, float* dx, uint64_t rows,
     uint64_t input_width, uint64_t output_width, uint64_t block_size,
     void* stream);
+
+/*
+ * y_m = x.deq(W_m)^T (+ bias_m) for m < member_count: several packed weights
+ * applied to the SAME x, as the query, key and value projections of an
+ * attention block are (src/model/decoder_only_transformer.cpp:406-419 calls
+ * query_, key_ and value_.forward on one normalised input; a gated feed-forward
+ * does the same with its gate and up projections).  The result is, bit for
+ * bit, that of member_count calls of rthip_nf4_linear_forward; the point is
+ * the launch count: for rows <= 4 up to four members run as ONE streaming
+ * launch, which removes the fixed cost between decode-sized kernels.  Other
+ * row counts, or members the streaming kernel cannot take, are launched one
+ * by one.  The members share input_width, block_size, encoding and
+ * second_level_block; each has its own output_width, offset, bias and y.
+ * `members` is a HOST array, read before the call returns.
+ */
+typedef struct rthip_nf4_member {
+    const uint8_t* codes;
+    const void* primary_scales;
+    const float* secondary_scales; /* NULL for fp32 scales */
+    float offset;
+    const float* bias_or_null;
+    float* y;                      /* [rows, output_width] */
+    uint64_t output_width;
+} rthip_nf4_member;
+
+rthip_status rthip_nf4_linear_forward_group(
+    const float* x, const rthip_nf4_member* members, uint64_t member_count,
+    int32_t encoding, uint64_t second_level_block, uint64_t rows,
+    uint64_t input_width, uint64_t block_size, void* stream);
 
 /*
  * y = x.deq(W)^T + bias + lora_scale * ((x.A^T).B^T)

@@ -82,6 +82,16 @@ _size = ctypes.c_size_t
 # The six values that describe a packed weight, in ABI order.
 _WEIGHT = [_ptr, _ptr, _ptr, _i32, _u64, _f32]
 
+
+
+class Member(ctypes.Structure):
+    """rthip_nf4_member: one weight of a group that shares its input."""
+
+    _fields_ = [("codes", _ptr), ("primary_scales", _ptr),
+                ("secondary_scales", _ptr), ("offset", _f32),
+                ("bias_or_null", _ptr), ("y", _ptr), ("output_width", _u64)]
+
+
 _PROTOTYPES = {
     "rthip_abi_version": (ctypes.c_uint32, []),
     "rthip_last_error": (ctypes.c_char_p, []),
@@ -103,6 +113,9 @@ _PROTOTYPES = {
         [_i32, _ptr] + _WEIGHT + [_ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
     "rthip_nf4_linear_input_backward_with": (
         _i32, [_i32, _ptr] + _WEIGHT + [_ptr, _u64, _u64, _u64, _u64, _ptr]),
+    "rthip_nf4_linear_forward_group": (
+        _i32, [_ptr, ctypes.POINTER(Member), _u64, _i32, _u64, _u64, _u64,
+               _u64, _ptr]),
     "rthip_matmul": (
         _i32, [_ptr, _ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
     "rthip_lora_reduce": (_i32, [_ptr, _ptr, _ptr, _u64, _u64, _u64, _ptr]),
@@ -259,6 +272,33 @@ class Library:
             status = self._lib.rthip_nf4_linear_forward_with(
                 algorithm, x_ptr, *weight.abi_arguments(), *tail)
         self._check(status)
+
+    def linear_forward_group(self, x_ptr: int, members, rows: int,
+                             stream: int = 0) -> None:
+        """members: (weight, bias_ptr or None, y_ptr) triples whose weights
+        share input width, block size and scale encoding."""
+        first = members[0][0]
+        array = (Member * len(members))()
+        for slot, (weight, bias_ptr, y_ptr) in zip(array, members):
+            if (weight.input_width, weight.block_size, weight.encoding,
+                    weight.second_level_block) != (
+                    first.input_width, first.block_size, first.encoding,
+                    first.second_level_block):
+                raise ValueError("the weights of a group must share input "
+                                 "width, block size and scale encoding")
+            slot.codes = weight.codes.data_ptr()
+            slot.primary_scales = weight.primary_scales.data_ptr()
+            slot.secondary_scales = (
+                None if weight.secondary_scales is None
+                else weight.secondary_scales.data_ptr())
+            slot.offset = weight.offset
+            slot.bias_or_null = bias_ptr
+            slot.y = y_ptr
+            slot.output_width = weight.output_width
+        self._check(self._lib.rthip_nf4_linear_forward_group(
+            x_ptr, array, len(members), first.encoding,
+            first.second_level_block, rows, first.input_width,
+            first.block_size, stream))
 
     def matmul(self, left_ptr: int, right_ptr: int, out_ptr: int,
                batch_count: int, rows: int, shared: int, columns: int,

@@ -44,6 +44,13 @@ void launch_fill(float* out, float value, std::size_t count,
 constexpr std::size_t kGemvMaxRows = 4;
 bool gemv_forward_supports(const LinearProblem& problem);
 void launch_gemv_forward(const LinearProblem& problem, hipStream_t stream);
+// Up to kGemvGroupMax weights applied to the same activations in ONE launch
+// (the projections of a layer that share their input).  Every output equals,
+// bit for bit, what launch_gemv_forward writes for that member alone.
+constexpr std::size_t kGemvGroupMax = 4;
+bool gemv_group_supports(const LinearProblem* problems, std::size_t count);
+void launch_gemv_group(const LinearProblem* problems, std::size_t count,
+                       hipStream_t stream);
 
 // workspace.hip -- scratch memory shared by the kernels that pass partial
 // results between workgroups; one fixed-size buffer per (device, stream).

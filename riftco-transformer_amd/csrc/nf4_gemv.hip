@@ -17,7 +17,19 @@
 //     one scale per segment:  acc += scale * sum_i x_i * codebook[c_i].
 // The loads of batch b + 1 are issued before batch b is computed, and the
 // wavefronts never wait for each other inside the loop, so HBM requests are in
-// flight for the whole life of the workgroup.
+// flight for the whole life of the workgroup.  Nothing may branch around
+// those loads or sit between them and the work they overlap with: the
+// compiler's wait counts are exact only along straight-line code, and a
+// uniform `if` around the loads makes every wait for the CURRENT batch wait
+// for the just-issued loads as well.  Hence the two compiled copies of the
+// step (with and without a batch left to request) and the deferred decode of
+// nested scales.
+//
+// Groups.  One launch can cover up to kGemvGroupMax weights that share x (the
+// query/key/value or gate/up projections of a layer): their batches are
+// numbered one weight after the other and dealt exactly like the batches of a
+// single weight, so every output is computed by the same lanes in the same
+// order as in a launch of its own, and the launch's fixed cost is paid once.
 //
 // Decode.  Nibble -> fp32 is a table lookup in LDS, 4 bytes of table per
 // weight.  Nibbles are decoded two at a time -- a code BYTE indexes a table of
@@ -47,6 +59,8 @@
 #include "nf4_decode.hpp"
 #include "nf4_pair_table.hpp"
 
+#include <type_traits>
+
 namespace rthip {
 namespace {
 
@@ -56,7 +70,7 @@ constexpr int kSegment = 16;       // weights per thread per row visit
 constexpr int kRowLanes = 16;      // lanes of one DPP row
 constexpr unsigned kComputeUnits = 256;
 // Row totals a team may park in LDS before the final barrier, per wavefront.
-constexpr unsigned kParkedValues = 128;
+constexpr unsigned kParkedValues = 512;
 #ifndef RTHIP_GEMV_TEAMS
 #define RTHIP_GEMV_TEAMS 2
 #endif
@@ -143,18 +157,53 @@ __device__ __forceinline__ unsigned slot_of_lane(unsigned lane) {
 
 typedef unsigned uint2_vec __attribute__((ext_vector_type(2)));
 
-// Shared scale loads per batch (nested scale encoding): one covers every
-// (row, block) of the batch that a wavefront touches, except for block size
-// 32, which needs two.
-constexpr int kScaleLoads = 2;
+// One weight of a launch.  A launch covers up to kGemvGroupMax weights that
+// are applied to the same x (the q/k/v or gate/up projections of a layer):
+// their row batches are numbered one member after the other, and member m owns
+// batches first_batch .. first_batch + ceil(output_width / kRows) - 1.  Unused
+// members carry first_batch = 0xFFFFFFFF.
+struct GemvMember {
+    const std::uint8_t* codes;
+    const void* primary_scales;
+    const float* secondary_scales;
+    const float* bias;
+    float* y;
+    unsigned output_width;
+    unsigned first_batch;
+    unsigned secondary_bytes;  // extent of the second-level scale table
+    float offset;
+};
+struct GemvGroup {
+    GemvMember member[kGemvGroupMax];
+};
+static_assert(kGemvGroupMax == 4, "member selection is written for four");
 
-// kShared false: the scale of this lane's weights of every row.  kShared true:
-// the scale of ONE (row, block) pair per lane and load; the lanes that need it
-// fetch it from this lane (see scale_of below).
+// Field `field` of member m, m per lane (the epilogue): a chain of selects
+// over kernel arguments.
+#define RTHIP_MEMBER(m, field)                                              \
+    (!kGrouped || (m) == 0                                                  \
+         ? group.member[0].field                                            \
+         : ((m) == 1 ? group.member[1].field                                \
+                     : ((m) == 2 ? group.member[2].field                    \
+                                 : group.member[3].field)))
+
+// Shared scale loads per batch (nested scale encoding): a load covers 64
+// (row, block) pairs and a wavefront's part of a row spans at most 32 blocks
+// (block size 32), so two-row batches need one load and four-row batches two.
+constexpr int scale_loads(int rows) { return rows * 32 > 64 ? 2 : 1; }
+
+// kShared false: scales[row][j] is the scale of this lane's weights of row
+// `row`.  kShared true: scale_codes[q][j] / scales[q][j] are the scale code
+// and the second-level scale of ONE (row, block) pair per lane and load, as
+// loaded; the step that consumes the batch decodes them, and the lanes that
+// need a scale fetch it from the lane that holds it (see scale_of below).
 template <int kRows, int kSegments, bool kShared>
 struct RowBatch {
     uint2_vec codes[kRows][kSegments];
-    float scales[kShared ? kScaleLoads : kRows][kSegments];
+    float scales[kShared ? scale_loads(kRows) : kRows][kSegments];
+    unsigned scale_codes[kShared ? scale_loads(kRows) : 1]
+                        [kShared ? kSegments : 1];
+    float offset;  // of the member the batch belongs to (uniform)
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base,
@@ -165,18 +214,19 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base,
                                              0x00020000);
 }
 
-static_assert(RTHIP_GEMV_ROWS <= 4, "one scale load covers four rows");
+static_assert(RTHIP_GEMV_ROWS <= 4, "two scale loads cover four rows");
 
 // kX: x rows held per thread (1, 2 or 4; a 3-row call runs as 4 with a zero
 // row).  kSegments: segments per thread.  kRows: weight rows per batch.
 // kTeams: teams per workgroup (2 teams of four wavefronts, or 1 team of eight
 // for rows so wide that four wavefronts' threads could not hold their x).
+// kGrouped: more than one member (a single weight compiles to the same code as
+// before: every member selection folds to member 0).
 template <int kX, int kSegments, int kRows, int kTeams, int kDepth,
-          bool kDoubleQuantized>
+          bool kDoubleQuantized, bool kGrouped>
 __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
-    const float* __restrict__ x, Nf4WeightView weight, unsigned secondary_bytes,
-    const float* __restrict__ bias, float* __restrict__ y, unsigned x_rows,
-    unsigned input_width, unsigned output_width, unsigned block_shift,
+    const float* __restrict__ x, GemvGroup group, unsigned second_level_shift,
+    unsigned x_rows, unsigned input_width, unsigned block_shift,
     unsigned batch_count, unsigned iterations, LoraEpilogue lora
 ) {
     constexpr int kThreads = kWorkgroupThreads;
@@ -202,8 +252,27 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
     // beyond the payload.
     const unsigned row_code_bytes = input_width / 2;
     const unsigned row_blocks = input_width >> block_shift;
-    const __amdgpu_buffer_rsrc_t secondary_buffer =
-        make_buffer(weight.secondary_scales, secondary_bytes);
+    // The member that the batches being REQUESTED belong to.  A team's batch
+    // numbers only grow, so the member only moves forward: its fields live in
+    // scalar registers and are re-read from the kernel arguments in the rare
+    // step that crosses into the next member (a uniform branch without any
+    // vector memory access in it, so the wait counts around it stay exact).
+    // Batches past the last one stay with the last member, where their rows
+    // lie past its output width.
+    unsigned member_index = 0;
+    GemvMember member = group.member[0];
+    unsigned member_end = kGrouped ? group.member[1].first_batch : 0xFFFFFFFFU;
+    const auto seek_member = [&](unsigned batch_index) {
+        if constexpr (kGrouped) {
+            while (batch_index >= member_end) {
+                ++member_index;
+                member = group.member[member_index];
+                member_end = member_index + 1 < kGemvGroupMax
+                                 ? group.member[member_index + 1].first_batch
+                                 : 0xFFFFFFFFU;
+            }
+        }
+    };
     // Plain fp32 scales are loaded by the lane that uses them, one per row
     // and stripe.  For the nested encoding that would mean two loads and a
     // decode (with a division) per row, which nearly doubles the kernel's
@@ -215,12 +284,8 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
     // from lane l with one ds_bpermute: one decode per lane and batch instead
     // of kRows.  (Sharing plain fp32 scales the same way measured 2-4 %
     // slower than loading them: the ds_bpermute costs more than the load it
-    // replaces.)  The range check of the whole-array descriptor rejects rows
-    // past the output width.
-    const unsigned block_total =
-        (output_width * input_width) >> block_shift;  // < 2^32 / 32
-    const __amdgpu_buffer_rsrc_t primary_buffer = make_buffer(
-        weight.primary_scales, kDoubleQuantized ? block_total : 0U);
+    // replaces.)  These loads go through a descriptor of the member's whole
+    // scale array.
     // lanes per block (log2), blocks per wavefront-row (log2), rows per load
     const unsigned lanes_shift = block_shift - 4;
     const unsigned p_shift = lanes_shift < 6 ? 6 - lanes_shift : 0;
@@ -242,18 +307,24 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
     }
 
     using Batch = RowBatch<kRows, kSegments, kDoubleQuantized>;
+    constexpr int kScaleLoads = scale_loads(kRows);
     const auto load_batch = [&](Batch& batch, unsigned batch_index) {
+        seek_member(batch_index);
+        const unsigned output_width = member.output_width;
+        const std::uint8_t* const codes = member.codes;
+        const void* const primary_scales = member.primary_scales;
+        const unsigned first_row = (batch_index - member.first_batch) * kRows;
+        batch.offset = member.offset;
 #pragma unroll
         for (int row = 0; row < kRows; ++row) {
-            const unsigned o = batch_index * kRows + row;  // scalar
+            const unsigned o = first_row + row;  // scalar
             const bool row_valid = o < output_width;
             const std::size_t row_start =
                 static_cast<std::size_t>(o) * input_width;
             const __amdgpu_buffer_rsrc_t code_row = make_buffer(
-                weight.codes + (row_start >> 1),
-                row_valid ? row_code_bytes : 0U);
+                codes + (row_start >> 1), row_valid ? row_code_bytes : 0U);
             const __amdgpu_buffer_rsrc_t scale_row = make_buffer(
-                static_cast<const float*>(weight.primary_scales) +
+                static_cast<const float*>(primary_scales) +
                     (row_start >> block_shift),
                 row_valid && !kDoubleQuantized ? row_blocks * 4 : 0U);
 #pragma unroll
@@ -272,13 +343,20 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
         if constexpr (!kDoubleQuantized) {
             return;
         }
+        const unsigned block_total =
+            (output_width * input_width) >> block_shift;  // < 2^32 / 32
+        const __amdgpu_buffer_rsrc_t primary_buffer =
+            make_buffer(primary_scales, block_total);
+        const __amdgpu_buffer_rsrc_t secondary_buffer =
+            make_buffer(member.secondary_scales, member.secondary_bytes);
+        // Every load is always issued (a second one is needed for block size
+        // 32 only; otherwise every lane's offset is the rejected one and no
+        // memory is touched): a branch here would sit between these loads
+        // and the waits of the step that issued them.
 #pragma unroll
         for (int q = 0; q < kScaleLoads; ++q) {
-            if (q * rows_per_load >= static_cast<unsigned>(kRows)) {
-                break;  // uniform: only block size 32 needs the second load
-            }
             const unsigned row_in_batch = q * rows_per_load + my_row;
-            const unsigned o = batch_index * kRows + row_in_batch;
+            const unsigned o = first_row + row_in_batch;
             const bool mine = row_in_batch < static_cast<unsigned>(kRows) &&
                               o < output_width;
 #pragma unroll
@@ -288,39 +366,35 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
                     (wave_in_team * kWave + kTeamThreads * j) * kSegment;
                 const unsigned block =
                     o * row_blocks + (wave_first >> block_shift) + my_block;
-                const unsigned offset = mine ? block : 0x80000000U;
-                {
-                    const std::uint8_t scale_code =
-                        __builtin_amdgcn_raw_buffer_load_b8(primary_buffer,
-                                                            offset, 0, 0);
-                    const float second = __builtin_bit_cast(
-                        float,
-                        __builtin_amdgcn_raw_buffer_load_b32(
-                            secondary_buffer,
-                            mine ? (block >> weight.second_level_shift) * 4
-                                 : 0x80000000U,
-                            0, 0));
-                    batch.scales[q][j] = decode_double_quantized_scale(
-                        scale_code, second, weight.offset);
-                }
+                batch.scale_codes[q][j] = __builtin_amdgcn_raw_buffer_load_b8(
+                    primary_buffer, mine ? block : 0x80000000U, 0, 0);
+                batch.scales[q][j] = __builtin_bit_cast(
+                    float, __builtin_amdgcn_raw_buffer_load_b32(
+                               secondary_buffer,
+                               mine ? (block >> second_level_shift) * 4
+                                    : 0x80000000U,
+                               0, 0));
             }
         }
     };
     // The scale of this lane's weights of row `row` (of the batch), stripe j.
-    const auto scale_of = [&](const Batch& batch, int row, int j) {
+    // held: this lane's decoded (row, block) scales of the batch.
+    const auto scale_of = [&](const Batch& batch,
+                              const float (&held)[kScaleLoads][kSegments],
+                              int row, int j) {
         if constexpr (!kDoubleQuantized) {
             return batch.scales[row][j];
         } else {
             const unsigned q = static_cast<unsigned>(row) / rows_per_load;
             const unsigned row_in_load =
                 static_cast<unsigned>(row) % rows_per_load;
-            const float held =
-                q == 0 ? batch.scales[0][j] : batch.scales[1][j];
             return __builtin_bit_cast(
                 float, __builtin_amdgcn_ds_bpermute(
                            static_cast<int>(((row_in_load << p_shift) * 4) +
                                             my_source),
-                           __builtin_bit_cast(int, held)));
+                           __builtin_bit_cast(
+                               int, q == 0 ? held[0][j]
+                                           : held[kScaleLoads - 1][j])));
         }
     };
 
@@ -386,12 +460,23 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
 
     // One batch: refill the slot freed by the previous batch, compute
     // `current`, reduce, park.
-    const auto step = [&](const Batch& current,
-                          Batch& refill,
-                          unsigned iteration) {
+    // kRefill: whether a batch kDepth - 1 steps ahead exists.  It is a
+    // compile-time property of the call, not a branch around the loads: with
+    // a branch, the compiler's wait counts must assume the path WITHOUT the
+    // new loads, so every wait for the current batch would also wait for the
+    // loads just issued and nothing would be prefetched.
+    const auto step = [&](const Batch& current, Batch& refill,
+                          unsigned iteration, auto refill_exists) {
+        constexpr bool kRefill = decltype(refill_exists)::value;
         const unsigned batch_index = first_batch + iteration * stride;
-        if (iteration + kDepth - 1 < iterations) {
+        // The table address bits pass through an empty asm in the copy that
+        // loads: the lookups' address arithmetic is otherwise identical in
+        // both copies, gets hoisted above the branch between them, and drags
+        // the wait for the current codes in front of the new loads.
+        unsigned step_lane_bits = lane_bits;
+        if constexpr (kRefill) {
             load_batch(refill, batch_index + (kDepth - 1) * stride);
+            asm volatile("" : "+v"(step_lane_bits)::"memory");
         }
 
         // Table lookups run one weight row ahead of the multiply-adds that
@@ -409,11 +494,27 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
 #pragma unroll
                     for (int b = 0; b < 4; ++b) {
                         out[j][4 * w + b] =
-                            pair_table_lookup(table, words[w], b, lane_bits);
+                            pair_table_lookup(table, words[w], b,
+                                              step_lane_bits);
                     }
                 }
             }
         };
+
+        // Nested scales are decoded here, a step after they were requested.
+        float held[kScaleLoads][kSegments];
+        if constexpr (kDoubleQuantized) {
+            const float scale_offset = current.offset;
+#pragma unroll
+            for (int q = 0; q < kScaleLoads; ++q) {
+#pragma unroll
+                for (int j = 0; j < kSegments; ++j) {
+                    held[q][j] = decode_double_quantized_scale(
+                        static_cast<std::uint8_t>(current.scale_codes[q][j]),
+                        current.scales[q][j], scale_offset);
+                }
+            }
+        }
 
         float acc[kValues];
         look_up(0, levels[0]);
@@ -431,7 +532,7 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
             float row_scale[kSegments];
 #pragma unroll
             for (int j = 0; j < kSegments; ++j) {
-                row_scale[j] = scale_of(current, row, j);
+                row_scale[j] = scale_of(current, held, row, j);
             }
 #pragma unroll
             for (int j = 0; j < kSegments; ++j) {
@@ -474,13 +575,20 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
         }
     };
 
-    // Walk the ring with static slot numbers (no register copies).
+    // Walk the ring with static slot numbers (no register copies).  The last
+    // kDepth - 1 steps have nothing left to request; they run the copy of the
+    // step that issues no loads.
     for (unsigned iteration = 0; iteration < iterations;
          iteration += kDepth) {
 #pragma unroll
         for (int d = 0; d < kDepth; ++d) {
             if (iteration + d < iterations) {
-                step(ring[d], ring[(d + kDepth - 1) % kDepth], iteration + d);
+                Batch& refill = ring[(d + kDepth - 1) % kDepth];
+                if (iteration + d + kDepth - 1 < iterations) {
+                    step(ring[d], refill, iteration + d, std::true_type{});
+                } else {
+                    step(ring[d], refill, iteration + d, std::false_type{});
+                }
             }
         }
     }
@@ -494,7 +602,16 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
         const unsigned iteration = index / kValues;
         const unsigned value = index % kValues;
         const unsigned batch_index = first_batch + iteration * stride;
-        const unsigned o = batch_index * kRows + value / kX;
+        // which member the batch belongs to: per lane here
+        const unsigned m =
+            !kGrouped
+                ? 0U
+                : (batch_index >= group.member[1].first_batch ? 1U : 0U) +
+                      (batch_index >= group.member[2].first_batch ? 1U : 0U) +
+                      (batch_index >= group.member[3].first_batch ? 1U : 0U);
+        const unsigned output_width = RTHIP_MEMBER(m, output_width);
+        const unsigned o =
+            (batch_index - RTHIP_MEMBER(m, first_batch)) * kRows + value / kX;
         const unsigned r = value % kX;
         if (batch_index < batch_count && o < output_width && r < x_rows) {
             float sum = 0.0F;
@@ -502,12 +619,14 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
             for (int wave = 0; wave < kTeamWaves; ++wave) {
                 sum += partial[team][iteration][wave][value];
             }
+            const float* const bias = RTHIP_MEMBER(m, bias);
             if (bias != nullptr) {
                 sum += bias[o];
             }
-            if (lora.reduced != nullptr) {
+            if (!kGrouped && lora.reduced != nullptr) {
                 sum += lora_term(lora, r, o);
             }
+            float* const y = RTHIP_MEMBER(m, y);
             y[r * output_width + o] = sum;
         }
     }
@@ -531,27 +650,58 @@ bool wide_team(const LinearProblem& p) {
     return held_rows(p) * segments_per_thread(p, 256) > kMaxHeldSegments;
 }
 
-template <int kX, int kSegments, bool kDoubleQuantized, bool kWide = false>
-void launch_instance(const LinearProblem& p, hipStream_t stream) {
+// The weights of one launch: `count` problems that share activations, row
+// count, row width, block size and scale encoding.
+struct Launch {
+    const LinearProblem* problems;
+    std::size_t count;
+};
+
+template <int kX, int kSegments, bool kDoubleQuantized, bool kGrouped,
+          bool kWide = false>
+void launch_instance(const Launch& launch, hipStream_t stream) {
     // Two teams (eight wavefronts) per workgroup measured best on MI355X; a
     // thread that carries more x rows or segments takes fewer weight rows per
     // batch so that its registers fit.
     constexpr bool kLight = kX * kSegments == 1;
     constexpr int kTeams = kWide ? 1 : (kLight ? RTHIP_GEMV_TEAMS : 2);
+    // (nested scales keep two more registers per segment and ring slot)
     constexpr int kRows =
-        kLight ? RTHIP_GEMV_ROWS : (kX * kSegments <= 4 ? 4 : 2);
+        kLight ? RTHIP_GEMV_ROWS
+               : (kX * kSegments <= 4 && !(kDoubleQuantized && kSegments >= 3)
+                      ? 4
+                      : 2);
     constexpr int kDepth = kLight ? RTHIP_GEMV_DEPTH : 2;
     constexpr unsigned kMaxIterations = kParkedValues / (kRows * kX);
-    const std::size_t elements = p.output_width * p.input_width;
-    const std::size_t block_count = elements >> p.block_shift;
-    // extent of the second-level scale table (double-quantised scales only)
-    const unsigned secondary_bytes =
-        kDoubleQuantized
-            ? static_cast<unsigned>(
-                  (((block_count - 1) >> p.weight.second_level_shift) + 1) * 4)
-            : 0U;
-    const unsigned batch_count =
-        static_cast<unsigned>((p.output_width + kRows - 1) / kRows);
+    const LinearProblem& first = launch.problems[0];
+    GemvGroup group{};
+    unsigned batch_count = 0;
+    for (std::size_t m = 0; m < kGemvGroupMax; ++m) {
+        GemvMember& member = group.member[m];
+        if (m >= launch.count) {
+            member.first_batch = 0xFFFFFFFFU;
+            continue;
+        }
+        const LinearProblem& p = launch.problems[m];
+        const std::size_t block_count =
+            (p.output_width * p.input_width) >> p.block_shift;
+        member.codes = p.weight.codes;
+        member.primary_scales = p.weight.primary_scales;
+        member.secondary_scales = p.weight.secondary_scales;
+        member.bias = p.bias;
+        member.y = p.result;
+        member.output_width = static_cast<unsigned>(p.output_width);
+        member.first_batch = batch_count;
+        member.secondary_bytes =
+            kDoubleQuantized
+                ? static_cast<unsigned>(
+                      (((block_count - 1) >> p.weight.second_level_shift) + 1) *
+                      4)
+                : 0U;
+        member.offset = p.weight.offset;
+        batch_count +=
+            static_cast<unsigned>((p.output_width + kRows - 1) / kRows);
+    }
     const unsigned team_groups = (batch_count + kTeams - 1) / kTeams;
     // One workgroup per CU; more when a team would otherwise need more
     // batches than its LDS parking space holds.
@@ -560,39 +710,57 @@ void launch_instance(const LinearProblem& p, hipStream_t stream) {
         blocks = (team_groups + kMaxIterations - 1) / kMaxIterations;
     }
     const unsigned iterations = (team_groups + blocks - 1) / blocks;
-    gemv_forward_kernel<kX, kSegments, kRows, kTeams, kDepth, kDoubleQuantized>
-        <<<blocks, kWorkgroupThreads, 0, stream>>>(
-            p.activations, p.weight, secondary_bytes, p.bias, p.result,
-            static_cast<unsigned>(p.rows),
-            static_cast<unsigned>(p.input_width),
-            static_cast<unsigned>(p.output_width), p.block_shift, batch_count,
-            iterations, p.lora);
+    gemv_forward_kernel<kX, kSegments, kRows, kTeams, kDepth, kDoubleQuantized,
+                        kGrouped><<<blocks, kWorkgroupThreads, 0, stream>>>(
+        first.activations, group, first.weight.second_level_shift,
+        static_cast<unsigned>(first.rows),
+        static_cast<unsigned>(first.input_width), first.block_shift,
+        batch_count, iterations, first.lora);
 }
 
-template <int kX, bool kDoubleQuantized>
-void launch_segments(const LinearProblem& p, hipStream_t stream) {
+template <int kX, bool kDoubleQuantized, bool kGrouped>
+void launch_segments(const Launch& launch, hipStream_t stream) {
+    const LinearProblem& p = launch.problems[0];
     if (wide_team(p)) {
         // four x rows and a row wider than 8192: two segments per thread of a
         // 512-thread team
         if constexpr (kX == 4) {
-            launch_instance<kX, 2, kDoubleQuantized, true>(p, stream);
+            launch_instance<kX, 2, kDoubleQuantized, kGrouped, true>(launch,
+                                                                     stream);
         }
         return;
     }
     switch (segments_per_thread(p, 256)) {
-    case 1: launch_instance<kX, 1, kDoubleQuantized>(p, stream); break;
-    case 2: launch_instance<kX, 2, kDoubleQuantized>(p, stream); break;
-    case 3: launch_instance<kX, 3, kDoubleQuantized>(p, stream); break;
-    default: launch_instance<kX, 4, kDoubleQuantized>(p, stream); break;
+    case 1:
+        launch_instance<kX, 1, kDoubleQuantized, kGrouped>(launch, stream);
+        break;
+    case 2:
+        launch_instance<kX, 2, kDoubleQuantized, kGrouped>(launch, stream);
+        break;
+    case 3:
+        launch_instance<kX, 3, kDoubleQuantized, kGrouped>(launch, stream);
+        break;
+    default:
+        launch_instance<kX, 4, kDoubleQuantized, kGrouped>(launch, stream);
+        break;
     }
 }
 
-template <bool kDoubleQuantized>
-void launch_rows(const LinearProblem& p, hipStream_t stream) {
-    switch (p.rows) {
-    case 1: launch_segments<1, kDoubleQuantized>(p, stream); break;
-    case 2: launch_segments<2, kDoubleQuantized>(p, stream); break;
-    default: launch_segments<4, kDoubleQuantized>(p, stream); break;
+template <bool kDoubleQuantized, bool kGrouped>
+void launch_rows(const Launch& launch, hipStream_t stream) {
+    switch (launch.problems[0].rows) {
+    case 1: launch_segments<1, kDoubleQuantized, kGrouped>(launch, stream); break;
+    case 2: launch_segments<2, kDoubleQuantized, kGrouped>(launch, stream); break;
+    default: launch_segments<4, kDoubleQuantized, kGrouped>(launch, stream); break;
+    }
+}
+
+template <bool kGrouped>
+void launch_encoding(const Launch& launch, hipStream_t stream) {
+    if (launch.problems[0].weight.encoding == 0) {
+        launch_rows<false, kGrouped>(launch, stream);
+    } else {
+        launch_rows<true, kGrouped>(launch, stream);
     }
 }
 
@@ -618,10 +786,36 @@ bool gemv_forward_supports(const LinearProblem& p) {
 }
 
 void launch_gemv_forward(const LinearProblem& p, hipStream_t stream) {
-    if (p.weight.encoding == 0) {
-        launch_rows<false>(p, stream);
+    launch_encoding<false>(Launch{&p, 1}, stream);
+}
+
+bool gemv_group_supports(const LinearProblem* problems, std::size_t count) {
+    if (count < 1 || count > kGemvGroupMax) {
+        return false;
+    }
+    const LinearProblem& first = problems[0];
+    std::size_t batches = 0;
+    for (std::size_t m = 0; m < count; ++m) {
+        const LinearProblem& p = problems[m];
+        if (!gemv_forward_supports(p) || p.activations != first.activations ||
+            p.rows != first.rows || p.input_width != first.input_width ||
+            p.block_shift != first.block_shift ||
+            p.weight.encoding != first.weight.encoding ||
+            p.weight.second_level_shift != first.weight.second_level_shift ||
+            p.lora.reduced != nullptr) {
+            return false;
+        }
+        batches += (p.output_width + 1) / 2;  // at least two rows per batch
+    }
+    return batches < (1ULL << 31);
+}
+
+void launch_gemv_group(const LinearProblem* problems, std::size_t count,
+                       hipStream_t stream) {
+    if (count == 1) {
+        launch_gemv_forward(problems[0], stream);
     } else {
-        launch_rows<true>(p, stream);
+        launch_encoding<true>(Launch{problems, count}, stream);
     }
 }
 

@@ -640,6 +640,101 @@ rthip_status rthip_nf4_linear_forward(
         input_width, output_width, block_size, stream);
 }
 
+rthip_status rthip_nf4_linear_forward_group(
+    const float* x, const rthip_nf4_member* members, uint64_t member_count,
+    int32_t encoding, uint64_t second_level_block, uint64_t rows,
+    uint64_t input_width, uint64_t block_size, void* stream
+) {
+    constexpr uint64_t kMaxMembers = 64;
+    if (x == nullptr || members == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "input and members must not be null");
+    }
+    if (member_count == 0 || member_count > kMaxMembers) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "a group holds between 1 and %llu weights",
+                    static_cast<unsigned long long>(kMaxMembers));
+    }
+    rthip::LinearProblem problems[kMaxMembers];
+    for (uint64_t m = 0; m < member_count; ++m) {
+        const rthip_nf4_member& member = members[m];
+        rthip::LinearProblem& problem = problems[m];
+        problem = rthip::LinearProblem{};
+        if (member.y == nullptr) {
+            return fail(RTHIP_INVALID_ARGUMENT,
+                        "input and output must not be null");
+        }
+        if (static_cast<const void*>(x) == static_cast<const void*>(member.y)) {
+            return fail(RTHIP_INVALID_ARGUMENT,
+                        "quantized linear input and output must not alias");
+        }
+        for (uint64_t other = 0; other < m; ++other) {
+            if (members[other].y == member.y) {
+                return fail(RTHIP_INVALID_ARGUMENT,
+                            "two members of a group write the same output");
+            }
+        }
+        if (const rthip_status status = check_dimensions(
+                rows, input_width, member.output_width, block_size,
+                &problem.block_shift);
+            status != RTHIP_OK) {
+            return status;
+        }
+        if (const rthip_status status = make_weight_view(
+                member.codes, member.primary_scales, member.secondary_scales,
+                encoding, second_level_block, member.offset, &problem.weight);
+            status != RTHIP_OK) {
+            return status;
+        }
+        problem.activations = x;
+        problem.bias = member.bias_or_null;
+        problem.result = member.y;
+        problem.rows = rows;
+        problem.input_width = input_width;
+        problem.output_width = member.output_width;
+    }
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+    uint64_t next = 0;
+    while (next < member_count) {
+        // the longest run of members from here that one streaming launch takes
+        uint64_t run = 0;
+        if (rows <= rthip::kGemvMaxRows) {
+            run = member_count - next < rthip::kGemvGroupMax
+                      ? member_count - next
+                      : rthip::kGemvGroupMax;
+            while (run > 0 &&
+                   !rthip::gemv_group_supports(problems + next, run)) {
+                --run;
+            }
+        }
+        if (run > 0) {
+            rthip::launch_gemv_group(problems + next, run, hip_stream);
+            if (const rthip_status status =
+                    finish_launch("NF4 linear forward launch");
+                status != RTHIP_OK) {
+                return status;
+            }
+            next += run;
+            continue;
+        }
+        const rthip_nf4_member& member = members[next];
+        if (const rthip_status status = linear_forward_common(
+                RTHIP_NF4_ALGORITHM_AUTO, x, member.codes,
+                member.primary_scales, member.secondary_scales, encoding,
+                second_level_block, member.offset, member.bias_or_null,
+                LoraArguments{nullptr, nullptr, 0, 0.0F, nullptr}, member.y,
+                rows, input_width, member.output_width, block_size, stream);
+            status != RTHIP_OK) {
+            return status;
+        }
+        ++next;
+    }
+    return ok();
+}
+
 rthip_status rthip_nf4_linear_input_backward_with(
     int32_t algorithm, const float* dy, const uint8_t* codes,
     const void* primary_scales, const float* secondary_scales,

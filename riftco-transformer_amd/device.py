@@ -90,6 +90,23 @@ def linear_forward(x: torch.Tensor, weight: DeviceWeight,
     return out
 
 
+def linear_forward_group(x: torch.Tensor, weights, biases=None):
+    """[x . deq(W_m)^T (+ bias_m) for every m] for weights that share x,
+    through rthip_nf4_linear_forward_group (one launch for decode-sized x)."""
+    assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous()
+    rows = x.numel() // weights[0].input_width
+    if biases is None:
+        biases = [None] * len(weights)
+    outs = [torch.empty((rows, weight.output_width), dtype=torch.float32,
+                        device=x.device) for weight in weights]
+    load_library().linear_forward_group(
+        x.data_ptr(),
+        [(weight, None if bias is None else bias.data_ptr(), out.data_ptr())
+         for weight, bias, out in zip(weights, biases, outs)],
+        rows, _stream())
+    return outs
+
+
 def lora_linear_forward(x: torch.Tensor, weight: DeviceWeight,
                         lora_a: torch.Tensor, lora_b: torch.Tensor,
                         lora_scale: float,

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol(package, library):
 
 
 def test_abi_version(package, library):
-    assert library.abi_version() == (1, 2)
+    assert library.abi_version() == (1, 3)
 
 
 def test_select_algorithm_is_pure_host_logic(package, library):
@@ -116,6 +116,30 @@ def test_lora_arguments_are_checked_before_any_device_work(package, library):
         library.lora_reduce(0x3000, 0, 0x7000, 1, 64, 8)
     with pytest.raises(package.InvalidArgument):
         library.lora_reduce(0x3000, 0x5000, 0x7000, 1, 64, 0)
+
+
+def test_group_arguments_are_checked_before_any_device_work(package, library):
+    weight = package.DeviceWeight(
+        64, 64, 64, package.SCALE_FLOAT32, _Fake(0x1000), _Fake(0x2000), None)
+    call = library.linear_forward_group
+    with pytest.raises(package.InvalidArgument):  # one output for two members
+        call(0x3000, [(weight, None, 0x4000), (weight, None, 0x4000)], 1)
+    assert "same output" in library.last_error()
+    with pytest.raises(package.InvalidArgument):  # output aliases the input
+        call(0x3000, [(weight, None, 0x3000)], 1)
+    with pytest.raises(package.InvalidArgument):  # no output
+        call(0x3000, [(weight, None, 0)], 1)
+    with pytest.raises(package.InvalidArgument):  # no rows
+        call(0x3000, [(weight, None, 0x4000)], 0)
+    with pytest.raises(package.InvalidArgument):  # too many members
+        call(0x3000, [(weight, None, 0x4000 + 256 * m) for m in range(65)], 1)
+    other = package.DeviceWeight(
+        64, 128, 64, package.SCALE_FLOAT32, _Fake(0x1000), _Fake(0x2000), None)
+    with pytest.raises(ValueError):  # different input widths
+        call(0x3000, [(weight, None, 0x4000), (other, None, 0x5000)], 1)
+    if not library.is_available():
+        with pytest.raises(package.Unavailable):
+            call(0x3000, [(weight, None, 0x4000)], 1)
 
 
 def test_matmul_arguments_are_checked_before_any_device_work(package,

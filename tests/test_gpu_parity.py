@@ -319,6 +319,66 @@ def test_wide_rows_at_three_and_four_rows(gpu, package, library, oracle, out_w,
                     oracle_rows=2)
 
 
+@pytest.mark.parametrize("widths,in_w,block,double_quantized", [
+    ((4096, 4096, 4096), 4096, 64, False),     # q/k/v
+    ((11008, 11008), 4096, 64, True),          # gate/up
+    ((77, 5, 1026, 33), 1040, 32, True),       # widths that end inside a batch
+    ((64, 300), 8192 + 256, 128, False),       # one 512-thread team per row
+    ((48, 50, 52, 54, 56, 58), 256, 64, True),  # more members than one launch
+    ((130,), 512, 64, False),                  # a group of one
+])
+def test_group_of_weights_that_share_an_input(gpu, package, library, oracle,
+                                              widths, in_w, block,
+                                              double_quantized):
+    """rthip_nf4_linear_forward_group against one call per member (bit for
+    bit) and against the CPU oracle."""
+    weights = [oracle.quantize(helpers.normal(300 + m, (out_w, in_w), 0.02),
+                               block, double_quantized, 256)
+               for m, out_w in enumerate(widths)]
+    device_weights = [upload(gpu, weight) for weight in weights]
+    biases = [None if m % 2 else helpers.normal(320 + m, (out_w,), 0.01)
+              for m, out_w in enumerate(widths)]
+    device_biases = [None if bias is None else to_device(bias)
+                     for bias in biases]
+    for rows in (1, 2, 3, 4, 7):
+        x = helpers.normal(340 + rows, (rows, in_w), 1.0)
+        x_device = to_device(x)
+        together = gpu.linear_forward_group(x_device, device_weights,
+                                            device_biases)
+        for m, weight in enumerate(weights):
+            alone = host(gpu.linear_forward(x_device, device_weights[m],
+                                            device_biases[m]))
+            helpers.assert_bit_equal(host(together[m]), alone,
+                                     f"member {m} at {rows} rows")
+        if rows in (1, 4):
+            for m in (0, len(weights) - 1):
+                dense = oracle.dequantize(weights[m])
+                cpu = oracle.forward(x, weights[m], biases[m])
+                drift = helpers.normalized_error(
+                    host(together[m]), cpu, in_w, helpers.rms(x),
+                    helpers.rms(dense))
+                assert drift <= 2 * TOLERANCE, \
+                    f"member {m} at {rows} rows vs CPU oracle: {drift:.3g}"
+
+
+def test_group_arguments_are_checked(gpu, package, library, oracle):
+    weight = upload(gpu, oracle.quantize(helpers.normal(1, (64, 64), 0.02),
+                                         64, False, 256))
+    x = to_device(helpers.normal(2, (1, 64), 1.0))
+    y = to_device(np.zeros((1, 64), np.float32))
+    call = library.linear_forward_group
+    with pytest.raises(package.InvalidArgument):  # two members, one output
+        call(x.data_ptr(), [(weight, None, y.data_ptr())] * 2, 1)
+    with pytest.raises(package.InvalidArgument):  # output aliases the input
+        call(x.data_ptr(), [(weight, None, x.data_ptr())], 1)
+    with pytest.raises(package.InvalidArgument):
+        call(x.data_ptr(), [(weight, None, 0)], 1)
+    with pytest.raises(package.InvalidArgument):
+        call(0, [(weight, None, y.data_ptr())], 1)
+    with pytest.raises(package.InvalidArgument):
+        call(x.data_ptr(), [(weight, None, y.data_ptr())], 0)
+
+
 def test_shared_output_tiles_are_added_in_a_fixed_order(gpu, package, library,
                                                         oracle):
     """When several workgroups hold parts of an output tile, the parts are
