@@ -16,6 +16,9 @@ The same JSON line carries
                 launch duration from HIP events on the launch stream)
   decode_double_quantized_scales
                 the decode step again with the nested scale encoding
+  decode_shared_input_groups
+                the decode step with q/k/v and gate/up launched together
+                through rthip_nf4_linear_forward_group
   gemm          M = 2048 forward and input-backward GEMMs (prefill / training
                 shapes) with their fp32-MFMA rooflines
   small_batch   M in {1, 4, 16, 64} on the three distinct shapes
@@ -100,26 +103,52 @@ def time_region(torch, body, repeats):
     return start.elapsed_time(stop)
 
 
+# Projections of a layer that read the same activations (one launch each when
+# the step is run through rthip_nf4_linear_forward_group).
+SHARED_INPUT_GROUPS = [("q_proj", "k_proj", "v_proj"), ("o_proj",),
+                       ("gate_proj", "up_proj"), ("down_proj",)]
+
+
 def bench_decode(package, device, torch, layers, steps, warmup, use_graph,
-                 double_quantized=False):
+                 double_quantized=False, grouped=False):
+    """One token through all 7 projections of `layers` layers.  grouped:
+    projections that share their input go through ONE call of the group entry
+    point (4 launches per layer instead of 7); otherwise one call each."""
     library = package.load_library()
-    weights = []
-    for layer in range(layers):
-        for index, (_, out_w, in_w) in enumerate(LAYER_SHAPES):
-            weights.append(synthetic_weight(package, torch, out_w, in_w,
-                                            double_quantized,
-                                            1000 * layer + index))
+    names = [name for name, _, _ in LAYER_SHAPES]
     x = {width: torch.randn(1, width, device="cuda")
          for width in (4096, 11008)}
-    y = {width: torch.empty(1, width, device="cuda")
-         for width in (4096, 11008)}
-    launches = [(x[w.input_width].data_ptr(), w, y[w.output_width].data_ptr())
-                for w in weights]
+    weights = []
+    launches = []  # (x pointer, [(weight, bias pointer, y pointer), ...])
+    outputs = []
+    for layer in range(layers):
+        of_layer = {}
+        for index, (name, out_w, in_w) in enumerate(LAYER_SHAPES):
+            of_layer[name] = synthetic_weight(package, torch, out_w, in_w,
+                                              double_quantized,
+                                              1000 * layer + index)
+            weights.append(of_layer[name])
+        groups = SHARED_INPUT_GROUPS if grouped else [(n,) for n in names]
+        for group in groups:
+            members = []
+            for slot, name in enumerate(group):
+                weight = of_layer[name]
+                if layer == 0:
+                    outputs.append(torch.empty(1, weight.output_width,
+                                               device="cuda"))
+                y = [t for t in outputs
+                     if t.shape[1] == weight.output_width][slot]
+                members.append((weight, None, y.data_ptr()))
+            launches.append((x[members[0][0].input_width].data_ptr(), members))
 
     def launch_all(items):
         stream = torch.cuda.current_stream().cuda_stream
-        for x_ptr, weight, y_ptr in items:
-            library.linear_forward(x_ptr, weight, None, y_ptr, 1, stream)
+        for x_ptr, members in items:
+            if len(members) == 1:
+                weight, _, y_ptr = members[0]
+                library.linear_forward(x_ptr, weight, None, y_ptr, 1, stream)
+            else:
+                library.linear_forward_group(x_ptr, members, 1, stream)
 
     launch_all(launches)  # first use outside any capture
     torch.cuda.synchronize()
@@ -133,19 +162,21 @@ def bench_decode(package, device, torch, layers, steps, warmup, use_graph,
     milliseconds = time_region(torch, step, steps)
     wall = time.perf_counter() - wall
     bytes_per_step = sum(w.payload_bytes for w in weights)
-    launches_per_step = len(weights)
+    launches_per_step = len(launches)
     seconds = milliseconds / 1e3
     gbs = bytes_per_step * steps / seconds / 1e9
 
     # The dominant kernel: the K = 4096 instantiation (6 of 7 projections).
-    dominant = [item for item in launches if item[1].input_width == 4096]
+    dominant = [item for item in launches
+                if item[1][0][0].input_width == 4096]
 
     dominant_pass = lambda: launch_all(dominant)
     if use_graph:
         dominant_pass = capture(torch, dominant_pass)
     dominant_pass()
     dominant_ms = time_region(torch, dominant_pass, steps)
-    dominant_bytes = sum(item[1].payload_bytes for item in dominant)
+    dominant_bytes = sum(member[0].payload_bytes
+                         for item in dominant for member in item[1])
     average_us = dominant_ms * 1e3 / (steps * len(dominant))
     achieved = dominant_bytes * steps / (dominant_ms / 1e3) / 1e9
     return {
@@ -157,11 +188,13 @@ def bench_decode(package, device, torch, layers, steps, warmup, use_graph,
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": DOMINANT_KERNEL_HBM_BYTES,
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+            "traffic": None if grouped else DOMINANT_KERNEL_HBM_BYTES,
+            "traffic_source": None if grouped else
+                              "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                               "scaled by a copy of known size "
                               "(profiles/decode_gemv_hbm_traffic_pmc.txt)",
-            "kernel": "gemv_forward_kernel<rows=1, K=4096>",
+            "kernel": "gemv_forward_kernel<rows=1, K=4096%s>" % (
+                ", grouped" if grouped else ""),
             "bytes_per_launch": dominant_bytes / len(dominant),
             "avg_launch_us": average_us,
         },
@@ -493,6 +526,19 @@ def main():
             "bytes_per_step": nested["bytes_per_step"],
         }
         del nested
+        # The same step with projections that share their input launched
+        # together (q/k/v and gate/up): 4 launches per layer instead of 7.
+        together = bench_decode(package, device, torch, arguments.layers,
+                                max(3, arguments.steps // 2),
+                                arguments.warmup, not arguments.no_graph,
+                                grouped=True)
+        line["decode_shared_input_groups"] = {
+            "value": together["value"], "unit": "GB/s",
+            "ms_per_step": together["ms_per_step"],
+            "launches_per_step": together["launches_per_step"],
+            "roofline": together["roofline"],
+        }
+        del together
         line["gemm"] = bench_gemm(package, device, torch,
                                   max(3, arguments.steps // 4))
         line["small_batch"] = bench_small_batch(package, device, torch,
