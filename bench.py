@@ -166,9 +166,11 @@ def bench_decode(package, device, torch, layers, steps, warmup, use_graph,
     seconds = milliseconds / 1e3
     gbs = bytes_per_step * steps / seconds / 1e9
 
-    # The dominant kernel: the K = 4096 instantiation (6 of 7 projections).
+    # The dominant kernel: the K = 4096 instantiation (6 of 7 projections);
+    # in a grouped step, its launches that cover more than one weight.
     dominant = [item for item in launches
-                if item[1][0][0].input_width == 4096]
+                if item[1][0][0].input_width == 4096 and
+                (not grouped or len(item[1]) > 1)]
 
     dominant_pass = lambda: launch_all(dominant)
     if use_graph:
@@ -188,9 +190,9 @@ def bench_decode(package, device, torch, layers, steps, warmup, use_graph,
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None if grouped else DOMINANT_KERNEL_HBM_BYTES,
-            "traffic_source": None if grouped else
-                              "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+            "traffic": (GROUPED_KERNEL_HBM_BYTES if grouped
+                        else DOMINANT_KERNEL_HBM_BYTES),
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                               "scaled by a copy of known size "
                               "(profiles/decode_gemv_hbm_traffic_pmc.txt)",
             "kernel": "gemv_forward_kernel<rows=1, K=4096%s>" % (
@@ -204,9 +206,12 @@ def bench_decode(package, device, torch, layers, steps, warmup, use_graph,
 # HBM bytes per launch of the dominant kernel (average over its 4:2 mix of
 # 4096x4096 and 11008x4096 weights), measured with rocprofv3 counters in runs
 # of their own -- a counter run cannot be nested inside this timing run:
-# FETCH_SIZE 7303.0 x 2.00 KiB (the factor a copy kernel of known size gives)
+# FETCH_SIZE 7329.2 x 2.00 KiB (the factor a copy kernel of known size gives)
 # plus WRITE_SIZE 25.0 x 1.00 KiB.  Algorithmic bytes: 14 745 600.
-DOMINANT_KERNEL_HBM_BYTES = int((7303.0 * 2.00 + 25.0) * 1024)
+DOMINANT_KERNEL_HBM_BYTES = int((7329.2 * 2.00 + 25.0) * 1024)
+# The same for the grouped launches (q/k/v and gate/up, 1:1): FETCH_SIZE
+# 19424.1 x 2.00 KiB plus WRITE_SIZE 67.0 KiB.  Algorithmic: 39 518 208.
+GROUPED_KERNEL_HBM_BYTES = int((19424.1 * 2.00 + 67.0) * 1024)
 
 
 def bench_gemm(package, device, torch, steps):
@@ -449,6 +454,10 @@ def main():
                         help="for rocprofv3 --pmc runs: a 1 GiB elementwise "
                              "copy of known traffic, then one decode step "
                              "launched kernel by kernel, nothing else")
+    parser.add_argument("--shared-input-groups", action="store_true",
+                        help="headline decode step (and the traffic "
+                             "calibration) with q/k/v and gate/up launched "
+                             "together: 4 launches per layer instead of 7")
     parser.add_argument("--no-graph", action="store_true",
                         help="launch the decode kernels one by one from "
                              "Python instead of replaying a HIP graph")
@@ -472,7 +481,8 @@ def main():
         for _ in range(3):
             torch.add(source, 1.0, out=target)
         torch.cuda.synchronize()
-        bench_decode(package, device, torch, arguments.layers, 1, 0, False)
+        bench_decode(package, device, torch, arguments.layers, 1, 0, False,
+                     grouped=arguments.shared_input_groups)
         print(json.dumps({"traffic_calibration": "done",
                           "copy_bytes_read": 2 ** 30,
                           "copy_bytes_written": 2 ** 30}))
@@ -491,7 +501,8 @@ def main():
 
     decode = bench_decode(package, device, torch, arguments.layers,
                           arguments.steps, arguments.warmup,
-                          not arguments.no_graph)
+                          not arguments.no_graph,
+                          grouped=arguments.shared_input_groups)
     line = {
         "metric": "NF4 linear: HBM GB/s at M=1, TFLOP/s at M=2048, % of "
                   "MI355X roofline",
@@ -504,7 +515,11 @@ def main():
             "workload": "decode GEMV M=1, Llama-7B layer shapes "
                         "(q/k/v/o 4096x4096, gate/up 11008x4096, down "
                         "4096x11008), NF4 block 64, fp32 absmax scales, "
-                        "%d layers x 7 projections per step" % arguments.layers,
+                        "%d layers x 7 projections per step%s" % (
+                            arguments.layers,
+                            ", projections that share their input launched "
+                            "together" if arguments.shared_input_groups
+                            else ", one launch per projection"),
             "layers": arguments.layers,
             "bytes_per_step": decode["bytes_per_step"],
             "launches_per_step": decode["launches_per_step"],
