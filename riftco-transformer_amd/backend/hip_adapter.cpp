@@ -818,6 +818,63 @@ const BackendAdapter& hip_backend_adapter() noexcept {
     return adapter;
 }
 
+void hip_quantized_linear_forward_group(
+    std::span<const QuantizedLinearForwardRequest> requests
+) {
+    constexpr std::string_view operation = "quantized-linear forward group";
+    if (requests.empty()) {
+        throw std::invalid_argument(
+            "a quantized-linear group needs at least one request");
+    }
+    const HipRuntime& runtime = require_runtime();
+    const QuantizedLinearForwardRequest& first = requests.front();
+    const auto& input = require_hip_tensor(first.input, operation);
+    const auto& first_weight = require_hip_weight(first.weight, operation);
+    std::vector<rthip_nf4_member> members;
+    members.reserve(requests.size());
+    for (const QuantizedLinearForwardRequest& request : requests) {
+        const auto& weight = require_hip_weight(request.weight, operation);
+        if (&request.input != &first.input ||
+            request.dimensions.rows != first.dimensions.rows ||
+            request.dimensions.input_width != first.dimensions.input_width ||
+            request.dimensions.block_size != first.dimensions.block_size ||
+            weight.encoding() != first_weight.encoding() ||
+            weight.second_level_block_size() !=
+                first_weight.second_level_block_size()) {
+            throw std::invalid_argument(
+                "the requests of a quantized-linear group must share their "
+                "input, row count, input width, block size and scale "
+                "encoding");
+        }
+    }
+    const float* source = input.device_for_read();
+    for (const QuantizedLinearForwardRequest& request : requests) {
+        const auto& weight = require_hip_weight(request.weight, operation);
+        auto& output = require_hip_tensor(request.output, operation);
+        rthip_nf4_member member{};
+        member.codes = static_cast<const std::uint8_t*>(
+            weight.packed_codes_native_handle());
+        member.primary_scales = weight.primary_scales_native_handle();
+        member.secondary_scales = static_cast<const float*>(
+            weight.secondary_scales_native_handle());
+        member.offset = weight.offset();
+        member.bias_or_null = nullptr;
+        member.y = output.device_for_overwrite();
+        member.output_width = request.dimensions.output_width;
+        members.push_back(member);
+    }
+    check(runtime,
+          runtime.nf4_linear_forward_group(
+              source, members.data(), members.size(),
+              static_cast<int32_t>(first_weight.encoding()),
+              first_weight.second_level_block_size(), first.dimensions.rows,
+              first.dimensions.input_width, first.dimensions.block_size,
+              nullptr),
+          operation);
+    finish_operation(runtime,
+                     "quantized-linear forward group synchronisation");
+}
+
 std::vector<HipPackedWeight> hip_load_packed_model_state(
     std::span<const std::uint8_t> state
 ) {

@@ -57,6 +57,18 @@ struct HipPackedWeightSource {
 [[nodiscard]] std::vector<std::uint8_t> hip_packed_model_state_bytes(
     std::span<const HipPackedWeightSource> weights);
 
+// Several packed linears applied to ONE input -- the query, key and value
+// projections of an attention block
+// (src/model/decoder_only_transformer.cpp:406-419) -- in one call: every
+// request must name the same input storage and agree in rows, input width,
+// block size and scale encoding; outputs are what one
+// quantized_linear_forward per request writes, bit for bit, but decode-sized
+// inputs go out as one kernel launch per four weights.  Like the capability
+// call it stands in for, it expects requests that the dispatcher has already
+// validated (dispatch_quantized_linear_forward's checks, once per request).
+void hip_quantized_linear_forward_group(
+    std::span<const QuantizedLinearForwardRequest> requests);
+
 // Optional extension implemented by hip weight storage: the O(#blocks) scale
 // validation that the dispatcher runs before every launch
 // (src/core/backend/nn/quantized_linear/dispatch.cpp:98-151) only has to run

@@ -80,6 +80,8 @@ void load(HipRuntime& runtime) {
               reason) ||
         !bind(library, "rthip_nf4_linear_forward", runtime.nf4_linear_forward,
               reason) ||
+        !bind(library, "rthip_nf4_linear_forward_group",
+              runtime.nf4_linear_forward_group, reason) ||
         !bind(library, "rthip_nf4_linear_input_backward",
               runtime.nf4_linear_input_backward, reason) ||
         !bind(library, "rthip_nf4_dequantize", runtime.nf4_dequantize,

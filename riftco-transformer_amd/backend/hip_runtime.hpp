@@ -35,6 +35,8 @@ struct HipRuntime {
     decltype(&rthip_fill_f32) fill_f32 = nullptr;
     decltype(&rthip_stream_synchronize) stream_synchronize = nullptr;
     decltype(&rthip_nf4_linear_forward) nf4_linear_forward = nullptr;
+    decltype(&rthip_nf4_linear_forward_group) nf4_linear_forward_group =
+        nullptr;
     decltype(&rthip_nf4_linear_input_backward) nf4_linear_input_backward =
         nullptr;
     decltype(&rthip_nf4_dequantize) nf4_dequantize = nullptr;

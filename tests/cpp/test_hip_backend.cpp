@@ -469,6 +469,63 @@ void test_transformer_sized_layer() {
     }
 }
 
+void test_forward_group() {
+    // Three projections of one input (the query/key/value pattern), through
+    // hip_quantized_linear_forward_group: bit for bit what one dispatch per
+    // projection writes.
+    namespace detail = riftco_transformer::backend_detail;
+    const std::size_t widths[] = {96, 64, 130};
+    for (const bool double_quantized : {false, true}) {
+        std::vector<HostWeight> weights;
+        std::vector<std::unique_ptr<backend::QuantizedWeightStorage>> storages;
+        for (std::size_t m = 0; m < 3; ++m) {
+            weights.push_back(quantize(
+                pseudo_normal(widths[m] * 256, 0.02F, 40 + m), widths[m], 256,
+                64, double_quantized, 256));
+            storages.push_back(to_hip(weights.back()));
+        }
+        for (const std::size_t rows : {std::size_t{1}, std::size_t{3},
+                                       std::size_t{9}}) {
+            const auto input = pseudo_normal(rows * 256, 1.0F, 50 + rows);
+            auto source = backend::make_tensor_storage(kHip, input);
+            std::vector<std::unique_ptr<backend::TensorStorage>> targets;
+            std::vector<backend::QuantizedLinearForwardRequest> requests;
+            for (std::size_t m = 0; m < 3; ++m) {
+                targets.push_back(backend::make_tensor_storage(
+                    kHip, rows * widths[m], 0.0F));
+                requests.push_back({*source, *storages[m], *targets[m],
+                                    {rows, 256, widths[m], 64}});
+            }
+            detail::hip_quantized_linear_forward_group(requests);
+            for (std::size_t m = 0; m < 3; ++m) {
+                const auto data = std::as_const(*targets[m]).data();
+                const std::vector<float> together(data.begin(), data.end());
+                const std::vector<float> alone =
+                    hip_forward(input, *storages[m], weights[m]);
+                require(together.size() == alone.size() &&
+                            std::memcmp(together.data(), alone.data(),
+                                        alone.size() * sizeof(float)) == 0,
+                        "a grouped forward must equal the separate one");
+            }
+        }
+        // requests that do not belong together are refused
+        const auto input = pseudo_normal(256, 1.0F, 60);
+        auto source = backend::make_tensor_storage(kHip, input);
+        auto other_source = backend::make_tensor_storage(kHip, input);
+        auto target_a = backend::make_tensor_storage(kHip, widths[0], 0.0F);
+        auto target_b = backend::make_tensor_storage(kHip, widths[1], 0.0F);
+        const std::vector<backend::QuantizedLinearForwardRequest> mixed = {
+            {*source, *storages[0], *target_a, {1, 256, widths[0], 64}},
+            {*other_source, *storages[1], *target_b, {1, 256, widths[1], 64}}};
+        require_throws<std::invalid_argument>(
+            [&] { detail::hip_quantized_linear_forward_group(mixed); },
+            "a group over two inputs", "share their input");
+        require_throws<std::invalid_argument>(
+            [&] { detail::hip_quantized_linear_forward_group({}); },
+            "an empty group", "at least one request");
+    }
+}
+
 void test_tensor_storage() {
     auto filled = backend::make_tensor_storage(kHip, 5, 1.5F);
     require(filled->backend() == kHip && filled->size() == 5 &&
@@ -947,6 +1004,7 @@ int main(int argc, char** argv) {
         }
         test_accelerator_oracle();
         test_transformer_sized_layer();
+        test_forward_group();
         test_tensor_storage();
         test_dispatch_validation();
         test_packed_model_state();

@@ -193,6 +193,27 @@ rthip_status rthip_nf4_linear_forward(
     return RTHIP_OK;
 }
 
+rthip_status rthip_nf4_linear_forward_group(
+    const float* x, const rthip_nf4_member* members, uint64_t member_count,
+    int32_t encoding, uint64_t second_level_block, uint64_t rows,
+    uint64_t input_width, uint64_t block_size, void* stream) {
+    if (members == nullptr || member_count == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT, "a group needs members");
+    }
+    for (uint64_t m = 0; m < member_count; ++m) {
+        const rthip_nf4_member& member = members[m];
+        if (const rthip_status status = rthip_nf4_linear_forward(
+                x, member.codes, member.primary_scales,
+                member.secondary_scales, encoding, second_level_block,
+                member.offset, member.bias_or_null, member.y, rows,
+                input_width, member.output_width, block_size, stream);
+            status != RTHIP_OK) {
+            return status;
+        }
+    }
+    return RTHIP_OK;
+}
+
 rthip_status rthip_nf4_linear_input_backward(
     const float* dy, const uint8_t* codes, const void* primary_scales,
     const float* secondary_scales, int32_t encoding,
