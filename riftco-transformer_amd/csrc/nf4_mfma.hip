@@ -54,6 +54,9 @@ constexpr int kTileK = 32;        // contraction per step
 constexpr int kStride = 36;       // padded LDS row stride in floats
 constexpr int kChunk = 16;        // weights decoded per thread per step
 constexpr unsigned kFlushSteps = 8;  // steps per first-level accumulation
+// LDS of a workgroup: two buffers x (activation tile + weight tile)
+constexpr std::size_t kTileBytes =
+    std::size_t{2} * (kTileM + kTileN) * kStride * sizeof(float);
 
 struct GemmShape {
     unsigned rows;         // M
@@ -201,19 +204,24 @@ __device__ __forceinline__ void gemm_segment(
     const float* __restrict__ activations, const Nf4WeightView& weight,
     const float* __restrict__ bias, float* __restrict__ result,
     float* __restrict__ partial, const GemmShape& shape, unsigned block_shift,
-    const LoraEpilogue& lora, float* __restrict__ a_tile,
-    float* __restrict__ b_tile, const float* __restrict__ table,
-    unsigned row0, unsigned col0, unsigned k_begin, unsigned k_end
+    const LoraEpilogue& lora, float* __restrict__ tiles,
+    const float* __restrict__ table, unsigned row0, unsigned col0,
+    unsigned k_begin, unsigned k_end
 ) {
     const unsigned thread = threadIdx.x;
     const unsigned lane = thread % 64;
     const unsigned wave = thread / 64;
     const unsigned wave_m = wave / 2;
     const unsigned wave_n = wave % 2;
-    const float* a_fragment =
-        a_tile + (wave_m * 64 + lane % 32) * kStride + 4 * (lane / 32);
-    const float* b_fragment =
-        b_tile + (wave_n * 64 + lane % 32) * kStride + 4 * (lane / 32);
+    // tiles: [buffer][activations | weights][row or column][k], two buffers.
+    // A step computes from one buffer while the next step's tiles are written
+    // into the other, so the writes need no barrier of their own.
+    constexpr unsigned kTileFloats = kTileM * kStride;
+    constexpr unsigned kBufferFloats = 2 * kTileFloats;
+    const unsigned a_offset =
+        (wave_m * 64 + lane % 32) * kStride + 4 * (lane / 32);
+    const unsigned b_offset = kTileFloats +
+        (wave_n * 64 + lane % 32) * kStride + 4 * (lane / 32);
 
     // Two-level accumulation: the matrix cores add into `acc` for
     // kFlushSteps steps (256 contraction values), then `acc` is folded into
@@ -236,61 +244,81 @@ __device__ __forceinline__ void gemm_segment(
     unsigned steps_since_flush = 0;
 
     Staged staged;
-    load_activation_tile(staged, activations, shape, row0, k_begin);
-    if constexpr (!kBackward) {
-        load_weight_tile_forward<kDoubleQuantized>(
-            staged, weight, shape, col0, k_begin, block_shift);
-    } else {
-        load_weight_tile_backward<kDoubleQuantized>(
-            staged, weight, shape, col0, k_begin, block_shift);
-    }
-
-    for (unsigned k0 = k_begin; k0 < k_end; k0 += kTileK) {
-        __syncthreads();  // previous step's fragment reads are done
-        store_activation_tile(staged, a_tile);
-        store_weight_tile<kBackward>(staged, table, b_tile);
-        __syncthreads();
-
-        const unsigned next = k0 + kTileK;
-        if (next < k_end) {
-            load_activation_tile(staged, activations, shape, row0, next);
-            if constexpr (!kBackward) {
-                load_weight_tile_forward<kDoubleQuantized>(
-                    staged, weight, shape, col0, next, block_shift);
-            } else {
-                load_weight_tile_backward<kDoubleQuantized>(
-                    staged, weight, shape, col0, next, block_shift);
-            }
+    const auto load_step = [&](unsigned k) {
+        load_activation_tile(staged, activations, shape, row0, k);
+        if constexpr (!kBackward) {
+            load_weight_tile_forward<kDoubleQuantized>(
+                staged, weight, shape, col0, k, block_shift);
+        } else {
+            load_weight_tile_backward<kDoubleQuantized>(
+                staged, weight, shape, col0, k, block_shift);
         }
-
+    };
+    const auto store_step = [&](unsigned buffer) {
+        float* const target = tiles + buffer * kBufferFloats;
+        store_activation_tile(staged, target);
+        store_weight_tile<kBackward>(staged, table, target + kTileFloats);
+    };
+    // Matrix instructions of contraction values [kk, kk + 8) of the step.
+    const auto multiply = [&](const float* a_fragment,
+                              const float* b_fragment, int kk) {
+        float4 a[2];
+        float4 b[2];
 #pragma unroll
-        for (int kk = 0; kk < kTileK; kk += 8) {
-            float4 a[2];
-            float4 b[2];
+        for (int i = 0; i < 2; ++i) {
+            a[i] = *reinterpret_cast<const float4*>(
+                a_fragment + i * 32 * kStride + kk);
+            b[i] = *reinterpret_cast<const float4*>(
+                b_fragment + i * 32 * kStride + kk);
+        }
+        const float a_values[2][4] = {{a[0].x, a[0].y, a[0].z, a[0].w},
+                                      {a[1].x, a[1].y, a[1].z, a[1].w}};
+        const float b_values[2][4] = {{b[0].x, b[0].y, b[0].z, b[0].w},
+                                      {b[1].x, b[1].y, b[1].z, b[1].w}};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                a[i] = *reinterpret_cast<const float4*>(
-                    a_fragment + i * 32 * kStride + kk);
-                b[i] = *reinterpret_cast<const float4*>(
-                    b_fragment + i * 32 * kStride + kk);
-            }
-            const float a_values[2][4] = {{a[0].x, a[0].y, a[0].z, a[0].w},
-                                          {a[1].x, a[1].y, a[1].z, a[1].w}};
-            const float b_values[2][4] = {{b[0].x, b[0].y, b[0].z, b[0].w},
-                                          {b[1].x, b[1].y, b[1].z, b[1].w}};
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                            a_values[i][s], b_values[j][s], acc[i][j], 0, 0,
-                            0);
-                    }
+                for (int j = 0; j < 2; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                        a_values[i][s], b_values[j][s], acc[i][j], 0, 0, 0);
                 }
             }
         }
+    };
+
+    load_step(k_begin);
+    __syncthreads();  // nobody still reads the tiles of an earlier segment
+    store_step(0);
+    if (k_begin + kTileK < k_end) {
+        load_step(k_begin + kTileK);
+    }
+    __syncthreads();
+
+    unsigned buffer = 0;
+    for (unsigned k0 = k_begin; k0 < k_end; k0 += kTileK) {
+        const float* const a_fragment =
+            tiles + buffer * kBufferFloats + a_offset;
+        const float* const b_fragment =
+            tiles + buffer * kBufferFloats + b_offset;
+        multiply(a_fragment, b_fragment, 0);
+        multiply(a_fragment, b_fragment, 8);
+
+        // The next step's tiles go into the other buffer while this step's
+        // matrix instructions run, and once the staging registers are free
+        // they take the loads of the step after that, which then have a
+        // whole step to arrive.
+        const unsigned next = k0 + kTileK;
+        if (next < k_end) {  // uniform
+            store_step(buffer ^ 1U);
+            if (next + kTileK < k_end) {
+                load_step(next + kTileK);
+            }
+        }
+
+        multiply(a_fragment, b_fragment, 16);
+        multiply(a_fragment, b_fragment, 24);
 
         if (++steps_since_flush == kFlushSteps) {
             steps_since_flush = 0;
@@ -306,6 +334,10 @@ __device__ __forceinline__ void gemm_segment(
                 }
             }
         }
+        // One barrier per step: the other buffer is complete, and this one
+        // may be overwritten.
+        __syncthreads();
+        buffer ^= 1U;
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -394,8 +426,9 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
     float* __restrict__ workspace, GemmShape shape, TilePlan plan,
     unsigned block_shift, LoraEpilogue lora
 ) {
-    __shared__ __attribute__((aligned(16))) float a_tile[kTileM * kStride];
-    __shared__ __attribute__((aligned(16))) float b_tile[kTileN * kStride];
+    // two buffers of an activation and a weight tile each: more than the 64
+    // KB a static array may have, so sized at launch
+    extern __shared__ __attribute__((aligned(16))) float tiles[];
     __shared__ float table[16];
     load_codebook_to_lds(table);
 
@@ -420,7 +453,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
                           kTileN;
         gemm_segment<kDoubleQuantized, kBackward>(
             activations, weight, bias, result, partial, shape, block_shift,
-            lora, a_tile, b_tile, table, (tile / plan.tiles_n) * kTileM,
+            lora, tiles, table, (tile / plan.tiles_n) * kTileM,
             (tile % plan.tiles_n) * kTileN, first_step * kTileK,
             (first_step + segment_steps) * kTileK);
         unit += segment_steps;
@@ -487,7 +520,14 @@ hipError_t launch_encoding(const LinearProblem& p, const GemmShape& shape,
             return status;
         }
     }
-    kernel<<<plan.whole_tiles + groups, kThreads, 0, stream>>>(
+    static const hipError_t configured = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel),
+        hipFuncAttributeMaxDynamicSharedMemorySize,
+        static_cast<int>(kTileBytes));
+    if (configured != hipSuccess) {
+        return configured;
+    }
+    kernel<<<plan.whole_tiles + groups, kThreads, kTileBytes, stream>>>(
         p.activations, p.weight, p.bias, p.result, workspace, shape, plan,
         p.block_shift, p.lora);
     if (groups != 0) {
