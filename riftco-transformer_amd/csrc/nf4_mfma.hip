@@ -19,8 +19,12 @@
 // ds_read_b128 per lane fetches four consecutive contraction values; lanes
 // 0-31 take offsets 0..3 and lanes 32-63 offsets 4..7 of each group of eight,
 // which the four MFMAs of the group consume as (k, k+4) pairs -- any pairing is
-// valid because both operands use the same one.  Global loads for step t+1 are
-// issued before the MFMAs of step t.
+// valid because both operands use the same one.  There are two such pairs of
+// tiles: step t multiplies from one pair, writes the tiles of step t + 1 --
+// whose operands are in registers by then -- into the other between its two
+// halves of matrix instructions, and then requests the operands of step t + 2
+// into the freed registers, so a step has one barrier and its loads have a
+// whole step to arrive.
 //
 // Work split.  Output tiles are dealt to workgroups whole while they fill the
 // device evenly (two workgroups per compute unit).  What is left over -- 1376
