@@ -78,8 +78,10 @@ enum {
     RTHIP_NF4_ALGORITHM_GEMV = 2,
     /* LDS-tiled fp32 MFMA GEMM with dequantisation fused into the tile load */
     RTHIP_NF4_ALGORITHM_MFMA = 3,
-    /* small batches (forward, up to 64 rows): weights decoded straight into
-     * MFMA operands, no LDS tile */
+    /* small batches (up to 64 rows): weights decoded straight into MFMA
+     * operands, no LDS tile.  Forward: a slab kernel over the contraction;
+     * input backward: the packed weight is walked row by row as it lies in
+     * memory, a lane owning eight of its columns */
     RTHIP_NF4_ALGORITHM_SKINNY = 4,
     /* up to 64 rows (forward) with a row width of 1024..4096: like SKINNY, but
      * x stays in registers, 16 rows per workgroup, and the wavefronts split

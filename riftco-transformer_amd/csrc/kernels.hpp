@@ -72,6 +72,14 @@ bool skinny_forward_supports(const LinearProblem& problem);
 hipError_t launch_skinny_forward(const LinearProblem& problem,
                                  hipStream_t stream);
 
+// nf4_small_backward.hip -- input backward for up to 64 rows: the weight is
+// walked as it lies in memory, a lane owning eight columns of a weight row.
+// Uses the stream workspace when the weight rows are cut into chunks.
+constexpr std::size_t kSmallBackwardMaxRows = 64;
+bool small_input_backward_supports(const LinearProblem& problem);
+hipError_t launch_small_input_backward(const LinearProblem& problem,
+                                       hipStream_t stream);
+
 // lora.hip -- reduced[rows, rank] = x A^T, the input of the adapter epilogue.
 void launch_lora_reduce(const float* x, const float* a, float* reduced,
                         std::size_t rows, std::size_t input_width,

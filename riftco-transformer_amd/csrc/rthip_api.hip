@@ -195,6 +195,10 @@ int32_t select_forward(const rthip::LinearProblem& problem) {
 }
 
 int32_t select_input_backward(const rthip::LinearProblem& problem) {
+    if (problem.rows <= rthip::kSmallBackwardMaxRows &&
+        rthip::small_input_backward_supports(problem)) {
+        return RTHIP_NF4_ALGORITHM_SKINNY;
+    }
     if (rthip::mfma_input_backward_supports(problem)) {
         return RTHIP_NF4_ALGORITHM_MFMA;
     }
@@ -795,8 +799,21 @@ rthip_status rthip_nf4_linear_input_backward_with(
             return from_hip(status, "GEMM workspace allocation");
         }
         break;
-    case RTHIP_NF4_ALGORITHM_GEMV:
     case RTHIP_NF4_ALGORITHM_SKINNY:
+        if (!rthip::small_input_backward_supports(problem)) {
+            return fail(RTHIP_UNSUPPORTED,
+                        "the small-batch family needs rows <= %zu, a row "
+                        "width that is a multiple of 8, an output width that "
+                        "is a multiple of 4 and aligned pointers",
+                        rthip::kSmallBackwardMaxRows);
+        }
+        if (const hipError_t status =
+                rthip::launch_small_input_backward(problem, hip_stream);
+            status != hipSuccess) {
+            return from_hip(status, "small-batch workspace allocation");
+        }
+        break;
+    case RTHIP_NF4_ALGORITHM_GEMV:
     case RTHIP_NF4_ALGORITHM_RESIDENT:
         return fail(RTHIP_UNSUPPORTED,
                     "this family implements the forward product only");

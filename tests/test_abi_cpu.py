@@ -65,6 +65,13 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(fwd, 16, 40, 768, 32) == package.ALGORITHM_GENERIC
     assert select(bwd, 2048, 4096, 11008, 64) == package.ALGORITHM_MFMA
     assert select(bwd, 2048, 11008, 4096, 64) == package.ALGORITHM_MFMA
+    # up to 64 rows and a row width that is a multiple of 8 -> the backward
+    # kernel that walks the weight as it lies in memory
+    assert select(bwd, 1, 4096, 11008, 64) == package.ALGORITHM_SKINNY
+    assert select(bwd, 64, 11008, 4096, 64) == package.ALGORITHM_SKINNY
+    assert select(bwd, 16, 40, 768, 32) == package.ALGORITHM_SKINNY
+    assert select(bwd, 65, 11008, 4096, 64) == package.ALGORITHM_MFMA
+    assert select(bwd, 16, 36, 768, 32) == package.ALGORITHM_GENERIC
     # the reference's edge layout -> shape-agnostic kernels
     assert select(fwd, 2, 33, 33, 32) == package.ALGORITHM_GENERIC
     assert select(bwd, 2, 33, 33, 32) == package.ALGORITHM_GENERIC

@@ -379,6 +379,44 @@ def test_group_arguments_are_checked(gpu, package, library, oracle):
         call(x.data_ptr(), [(weight, None, y.data_ptr())], 0)
 
 
+@pytest.mark.parametrize("out_w,in_w,block,second,double_quantized", [
+    (4096, 4096, 64, 256, False),    # 32 column tiles x 8 chunks of rows
+    (4096, 11008, 64, 256, True),    # 86 column tiles, more units than CUs
+    (11008, 4096, 64, 256, True),    # chunks that end inside a 128-row walk
+    (132, 1040, 32, 32, True),       # one chunk; columns end inside a tile
+    (1028, 40, 4096, 32, False),     # one narrow tile, blocks span rows
+    (20, 8, 32, 32, False),          # a single lane's run of columns
+])
+def test_small_batch_input_backward(gpu, package, library, oracle, out_w, in_w,
+                                    block, second, double_quantized):
+    """Up to 64 rows of dy against the packed weight walked as it lies in
+    memory: one to four row groups, full and partly empty, against the oracle,
+    fp64 and the other families (check_layer runs each that accepts the
+    shape); and the same launch repeated, bit for bit (partial sums of row
+    chunks are added in a fixed order)."""
+    dense = helpers.normal(83, (out_w, in_w), 0.02)
+    dense[out_w // 2] = 0.0
+    weight = oracle.quantize(dense, block, double_quantized, second)
+    device_weight = upload(gpu, weight)
+    for rows in (1, 7, 16, 17, 40, 64):
+        assert library.select_algorithm(
+            package.INPUT_BACKWARD, rows, in_w, out_w,
+            block) == package.ALGORITHM_SKINNY
+        x = helpers.normal(84 + rows, (rows, in_w), 1.0)
+        dy = helpers.normal(85 + rows, (rows, out_w), 1.0e-2)
+        check_layer(gpu, package, library, oracle, weight, x, dy,
+                    oracle_rows=min(rows, 3))
+        dy_device = to_device(dy)
+        first = host(gpu.linear_input_backward(dy_device, device_weight))
+        for launch in range(3):
+            helpers.assert_bit_equal(
+                host(gpu.linear_input_backward(dy_device, device_weight)),
+                first, f"{rows} rows, launch {launch}")
+    assert library.select_algorithm(
+        package.INPUT_BACKWARD, 65, in_w, out_w,
+        block) != package.ALGORITHM_SKINNY
+
+
 def test_shared_output_tiles_are_added_in_a_fixed_order(gpu, package, library,
                                                         oracle):
     """When several workgroups hold parts of an output tile, the parts are
