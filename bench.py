@@ -22,6 +22,8 @@ The same JSON line carries
   gemm          M = 2048 forward and input-backward GEMMs (prefill / training
                 shapes) with their fp32-MFMA rooflines
   small_batch   M in {1, 4, 16, 64} on the three distinct shapes
+  small_batch_input_backward
+                the input backward at M in {1, 16, 64}, nested scales
   lora          the fused bias + rank-16 adapter forward beside the plain one
   matmul        dense fp32 matmul at layer and adapter shapes
   quantizer     the device quantizer on one 11008 x 4096 weight (wall clock,
@@ -270,6 +272,35 @@ def bench_small_batch(package, device, torch, steps):
             def body():
                 for weight in weights:
                     device.linear_forward(source, weight, out=target)
+
+            body()
+            torch.cuda.synchronize()
+            body = capture(torch, body)
+            body()
+            milliseconds = time_region(torch, body, steps) / (
+                steps * len(weights))
+            results.append({
+                "shape": name, "rows": rows, "us": milliseconds * 1e3,
+                "gb_per_s": weights[0].payload_bytes / milliseconds / 1e6,
+                "tflop_per_s": 2.0 * rows * out_w * in_w / milliseconds / 1e9,
+            })
+        del weights
+    return results
+
+
+def bench_small_batch_backward(package, device, torch, steps):
+    """Input backward at M in {1, 16, 64}, nested scales; rotating weights."""
+    results = []
+    for name, out_w, in_w in (LAYER_SHAPES[4], LAYER_SHAPES[6]):
+        weights = [synthetic_weight(package, torch, out_w, in_w, True, 700 + i)
+                   for i in range(12)]
+        for rows in (1, 16, 64):
+            upstream = torch.randn(rows, out_w, device="cuda") * 1.0e-2
+            target = torch.empty(rows, in_w, device="cuda")
+
+            def body():
+                for weight in weights:
+                    device.linear_input_backward(upstream, weight, out=target)
 
             body()
             torch.cuda.synchronize()
@@ -558,6 +589,8 @@ def main():
                                   max(3, arguments.steps // 4))
         line["small_batch"] = bench_small_batch(package, device, torch,
                                                 max(3, arguments.steps // 4))
+        line["small_batch_input_backward"] = bench_small_batch_backward(
+            package, device, torch, max(3, arguments.steps // 4))
         line["lora"] = bench_lora(package, device, torch,
                                   max(3, arguments.steps // 4))
         line["matmul"] = bench_matmul(package, device, torch,
