@@ -1008,6 +1008,8 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
         if family is None:
             assert package.ALGORITHM_NAMES[library.select_algorithm(
                 package.FORWARD, rows, 2048, 1000, 64)] == name.split(",")[0]
+    assert library.select_algorithm(package.INPUT_BACKWARD, 40, 2048, 1000,
+                                    64) == package.ALGORITHM_SKINNY
 
     def launch_all():
         outputs = {name: gpu.linear_forward(x, device_weight, bias,
@@ -1017,6 +1019,10 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
             inputs["resident"], device_weight, lora_a, lora_b, 0.5, bias)
         outputs["backward"] = gpu.linear_input_backward(upstream,
                                                         device_weight)
+        # up to 64 rows: the kernel that walks the weight row by row, here
+        # with its row chunks summed through the workspace
+        outputs["small backward"] = gpu.linear_input_backward(
+            upstream[:40].contiguous(), device_weight)
         return outputs
 
     def refill(seed):
