@@ -22,6 +22,9 @@ The same JSON line carries
   gemm          M = 2048 forward and input-backward GEMMs (prefill / training
                 shapes) with their fp32-MFMA rooflines
   small_batch   M in {1, 4, 16, 64} on the three distinct shapes
+  large_launches
+                M = 1 launches of 74 and 101 MB (lm_head; four gate/up weights
+                in one grouped launch)
   small_batch_input_backward
                 the input backward at M in {1, 16, 64}, nested scales
   lora          the fused bias + rank-16 adapter forward beside the plain one
@@ -285,6 +288,50 @@ def bench_small_batch(package, device, torch, steps):
                 "tflop_per_s": 2.0 * rows * out_w * in_w / milliseconds / 1e9,
             })
         del weights
+    return results
+
+
+def bench_large_launches(package, device, torch, steps):
+    """M = 1 launches that move more bytes than one projection: the lm_head of
+    the same model (32000 x 4096) and gate/up of two layers in one grouped
+    launch.  They show the rate the GEMV streams at once a launch's fixed cost
+    (about 3 us) is spread over enough bytes."""
+    library = package.load_library()
+    results = []
+    x = torch.randn(1, 4096, device="cuda")
+    cases = [("lm_head 32000x4096", [(32000, 4096)]),
+             ("4 x 11008x4096 in one launch", [(11008, 4096)] * 4)]
+    for name, shapes in cases:
+        copies = 6  # 6 x >= 74 MB: beyond the last-level cache
+        groups = [[synthetic_weight(package, torch, out_w, in_w, False,
+                                    900 + 10 * copy + index)
+                   for index, (out_w, in_w) in enumerate(shapes)]
+                  for copy in range(copies)]
+        outputs = [torch.empty(1, out_w, device="cuda")
+                   for out_w, _ in shapes]
+
+        def body():
+            stream = torch.cuda.current_stream().cuda_stream
+            for group in groups:
+                library.linear_forward_group(
+                    x.data_ptr(),
+                    [(weight, None, y.data_ptr())
+                     for weight, y in zip(group, outputs)], 1, stream)
+
+        body()
+        torch.cuda.synchronize()
+        body = capture(torch, body)
+        body()
+        milliseconds = time_region(torch, body, steps) / (steps * copies)
+        payload = sum(weight.payload_bytes for weight in groups[0])
+        gbs = payload / milliseconds / 1e6
+        results.append({
+            "launch": name, "bytes": payload, "us": milliseconds * 1e3,
+            "roofline": {"bound": "hbm", "achieved": gbs,
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": gbs / HBM_PEAK_GBS, "traffic": None},
+        })
+        del groups
     return results
 
 
@@ -589,6 +636,8 @@ def main():
                                   max(3, arguments.steps // 4))
         line["small_batch"] = bench_small_batch(package, device, torch,
                                                 max(3, arguments.steps // 4))
+        line["large_launches"] = bench_large_launches(
+            package, device, torch, max(3, arguments.steps // 2))
         line["small_batch_input_backward"] = bench_small_batch_backward(
             package, device, torch, max(3, arguments.steps // 4))
         line["lora"] = bench_lora(package, device, torch,
