@@ -43,6 +43,7 @@
 
 #include "kernels.hpp"
 #include "nf4_decode.hpp"
+#include "backward_split.hpp"
 #include "nf4_pair_table.hpp"
 
 namespace rthip {
@@ -52,14 +53,10 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 512;
 constexpr int kWaves = 8;
-constexpr int kTileColumns = 128;  // output columns of a workgroup
 constexpr int kLaneColumns = 8;    // of which a lane owns this many
 constexpr int kStepRows = 4;       // weight rows per matrix instruction
 constexpr int kSubSteps = 4;       // matrix-instruction steps per walk step
-// weight rows a workgroup covers per walk step
-constexpr unsigned kWalkRows = kWaves * kStepRows * kSubSteps;
-constexpr unsigned kComputeUnits = 256;
-constexpr unsigned kMaxChunks = 16;
+static_assert(kWalkRows == kWaves * kStepRows * kSubSteps);
 // Register slots for walk steps (steps in flight + 1): fewer when there are
 // more row groups, which is when a step lasts longer and registers are scarce.
 constexpr int ring_depth(int blocks) { return blocks <= 2 ? 3 : 2; }
@@ -73,13 +70,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_buffer(const void* base,
     return __builtin_amdgcn_make_buffer_rsrc(
         const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
 }
-
-struct BackwardSplit {
-    unsigned column_tiles;   // ceil(I / 128)
-    unsigned chunks;         // pieces of the weight rows
-    unsigned chunk_rows;     // rows per piece, a multiple of 128
-    unsigned units_per_xcd;  // ceil(column_tiles * chunks / 8)
-};
 
 // kBlocks: groups of 16 dy rows (1..4).
 template <int kBlocks, bool kDoubleQuantized>
@@ -347,48 +337,10 @@ __global__ __launch_bounds__(256) void small_backward_sum_kernel(
     dx[element] = sum;
 }
 
-// How the weight rows are cut: one workgroup fits per compute unit, so the
-// kernel takes ceil(units / 256) rounds of a chunk's length each; among the
-// chunk counts whose partial sums fit the workspace the one with the least
-// rounds x chunk length wins (ties: fewer chunks).
-BackwardSplit split_rows(const LinearProblem& p) {
-    BackwardSplit best{};
-    const unsigned column_tiles = static_cast<unsigned>(
-        (p.input_width + kTileColumns - 1) / kTileColumns);
-    double best_cost = 0.0;
-    for (unsigned chunks = 1; chunks <= kMaxChunks; ++chunks) {
-        const unsigned chunk_rows = static_cast<unsigned>(
-            ((p.output_width + chunks - 1) / chunks + kWalkRows - 1) /
-            kWalkRows * kWalkRows);
-        const unsigned actual = static_cast<unsigned>(
-            (p.output_width + chunk_rows - 1) / chunk_rows);
-        if (actual != chunks) {
-            continue;  // the same split as a smaller count
-        }
-        if (chunks > 1 && static_cast<std::size_t>(chunks) * p.rows *
-                                  p.input_width * sizeof(float) >
-                              kStreamWorkspaceBytes) {
-            break;
-        }
-        const unsigned units = column_tiles * chunks;
-        const unsigned rounds = (units + kComputeUnits - 1) / kComputeUnits;
-        // (+ the cost of writing and adding one more partial sum)
-        const double cost =
-            static_cast<double>(rounds) * chunk_rows + 8.0 * (chunks - 1);
-        if (best.chunks == 0 || cost < best_cost) {
-            best_cost = cost;
-            best.column_tiles = column_tiles;
-            best.chunks = chunks;
-            best.chunk_rows = chunk_rows;
-            best.units_per_xcd = (units + 7) / 8;
-        }
-    }
-    return best;
-}
-
 template <int kBlocks, bool kDoubleQuantized>
 hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
-    const BackwardSplit split = split_rows(p);
+    const BackwardSplit split = split_weight_rows(
+        p.rows, p.input_width, p.output_width, kStreamWorkspaceBytes);
     float* target = p.result;
     if (split.chunks > 1) {
         if (const hipError_t status = stream_workspace(stream, &target);

@@ -99,6 +99,19 @@ def test_work_split_of_the_tiled_kernels():
     assert "tile plan tests passed" in result.stdout
 
 
+def test_work_split_of_the_small_batch_input_backward():
+    """Host arithmetic of backward_split.hpp: chunks are whole walk steps and
+    cover every weight row once, partial sums fit the workspace, no cheaper
+    split exists (tests/cpp/test_backward_split.cpp)."""
+    binary = os.path.join(BUILD, "test_backward_split")
+    assert os.path.exists(binary), \
+        "tests/cpp/build/test_backward_split is not built (make -C tests/cpp)"
+    result = subprocess.run([binary], capture_output=True, text=True,
+                            timeout=120)
+    assert result.returncode == 0, result.stdout + result.stderr
+    assert "backward split tests passed" in result.stdout
+
+
 def test_unavailable_when_the_runtime_sees_no_device():
     result = run(["--expect-unavailable"],
                  RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE, FAKE_RTHIP_NO_DEVICE="1")
