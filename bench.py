@@ -526,8 +526,8 @@ def main():
                         help="run only the M = 2048 GEMM section (for "
                              "rocprofv3 counter runs)")
     parser.add_argument("--small-batch-only", action="store_true",
-                        help="run only the M in {1, 4, 16, 64} launches "
-                             "(for counter runs)")
+                        help="run only the launches of up to 64 rows, "
+                             "forward and input backward (for counter runs)")
     parser.add_argument("--traffic-calibration", action="store_true",
                         help="for rocprofv3 --pmc runs: a 1 GiB elementwise "
                              "copy of known traffic, then one decode step "
@@ -573,8 +573,11 @@ def main():
         return
 
     if arguments.small_batch_only:
-        print(json.dumps({"small_batch": bench_small_batch(
-            package, device, torch, arguments.steps)}))
+        print(json.dumps({
+            "small_batch": bench_small_batch(package, device, torch,
+                                             arguments.steps),
+            "small_batch_input_backward": bench_small_batch_backward(
+                package, device, torch, arguments.steps)}))
         return
 
     decode = bench_decode(package, device, torch, arguments.layers,
