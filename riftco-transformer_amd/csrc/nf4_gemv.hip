@@ -58,16 +58,15 @@
 #include "kernels.hpp"
 #include "nf4_decode.hpp"
 #include "nf4_pair_table.hpp"
+#include "gemv_shared.hpp"
 
 #include <type_traits>
 
 namespace rthip {
 namespace {
 
-constexpr int kWave = 64;
 constexpr int kWorkgroupThreads = 512;
 constexpr int kSegment = 16;       // weights per thread per row visit
-constexpr int kRowLanes = 16;      // lanes of one DPP row
 constexpr unsigned kComputeUnits = 256;
 // Row totals a team may park in LDS before the final barrier, per wavefront.
 constexpr unsigned kParkedValues = 512;
@@ -80,27 +79,6 @@ constexpr unsigned kParkedValues = 512;
 #ifndef RTHIP_GEMV_DEPTH
 #define RTHIP_GEMV_DEPTH 2
 #endif
-
-// value of lane (l ^ kXor) within the 16-lane DPP row, vector ALU only.
-template <int kXor>
-__device__ __forceinline__ float dpp_xor(float value) {
-    const int bits = __builtin_bit_cast(int, value);
-    int moved;
-    if constexpr (kXor == 1) {
-        moved = __builtin_amdgcn_update_dpp(0, bits, 0xB1, 0xF, 0xF, false);
-    } else if constexpr (kXor == 2) {
-        moved = __builtin_amdgcn_update_dpp(0, bits, 0x4E, 0xF, 0xF, false);
-    } else if constexpr (kXor == 4) {
-        // lanes 0-3 and 8-11 read four lanes up, the others four lanes down
-        moved = __builtin_amdgcn_update_dpp(0, bits, 0x104, 0xF, 0x5, false);
-        moved =
-            __builtin_amdgcn_update_dpp(moved, bits, 0x114, 0xF, 0xA, false);
-    } else {
-        static_assert(kXor == 8);
-        moved = __builtin_amdgcn_update_dpp(0, bits, 0x128, 0xF, 0xF, false);
-    }
-    return __builtin_bit_cast(float, moved);
-}
 
 template <int kXor, int kHalf, int kValues>
 __device__ __forceinline__ void transposed_step(float (&values)[kValues],
@@ -155,37 +133,6 @@ __device__ __forceinline__ unsigned slot_of_lane(unsigned lane) {
     return slot;
 }
 
-typedef unsigned uint2_vec __attribute__((ext_vector_type(2)));
-
-// One weight of a launch.  A launch covers up to kGemvGroupMax weights that
-// are applied to the same x (the q/k/v or gate/up projections of a layer):
-// their row batches are numbered one member after the other, and member m owns
-// batches first_batch .. first_batch + ceil(output_width / kRows) - 1.  Unused
-// members carry first_batch = 0xFFFFFFFF.
-struct GemvMember {
-    const std::uint8_t* codes;
-    const void* primary_scales;
-    const float* secondary_scales;
-    const float* bias;
-    float* y;
-    unsigned output_width;
-    unsigned first_batch;
-    unsigned secondary_bytes;  // extent of the second-level scale table
-    float offset;
-};
-struct GemvGroup {
-    GemvMember member[kGemvGroupMax];
-};
-static_assert(kGemvGroupMax == 4, "member selection is written for four");
-
-// Field `field` of member m, m per lane (the epilogue): a chain of selects
-// over kernel arguments.
-#define RTHIP_MEMBER(m, field)                                              \
-    (!kGrouped || (m) == 0                                                  \
-         ? group.member[0].field                                            \
-         : ((m) == 1 ? group.member[1].field                                \
-                     : ((m) == 2 ? group.member[2].field                    \
-                                 : group.member[3].field)))
 
 // Shared scale loads per batch (nested scale encoding): a load covers 64
 // (row, block) pairs and a wavefront's part of a row spans at most 32 blocks
@@ -205,14 +152,6 @@ struct RowBatch {
                         [kShared ? kSegments : 1];
     float offset;  // of the member the batch belongs to (uniform)
 };
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base,
-                                                             unsigned bytes) {
-    // Raw (untyped, stride 0) buffer with range checking on `bytes`.
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0,
-                                             static_cast<int>(bytes),
-                                             0x00020000);
-}
 
 static_assert(RTHIP_GEMV_ROWS <= 4, "two scale loads cover four rows");
 
@@ -567,8 +506,7 @@ __global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
         // Totals of each 16-lane DPP row, then of the wavefront's four rows;
         // the wavefront parks them and nobody waits here.
         float total = transposed_row_sum<kValues>(acc, lane);
-        total += __shfl_xor(total, 16, kWave);
-        total += __shfl_xor(total, 32, kWave);
+        total = sum_over_rows(total);
         if (lane < kValues) {
             partial[team][iteration][thread / kWave]
                    [slot_of_lane<kValues>(lane)] = total;
