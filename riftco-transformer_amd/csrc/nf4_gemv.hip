@@ -603,12 +603,12 @@ void launch_instance(const Launch& launch, hipStream_t stream) {
     // batch so that its registers fit.
     constexpr bool kLight = kX * kSegments == 1;
     constexpr int kTeams = kWide ? 1 : (kLight ? RTHIP_GEMV_TEAMS : 2);
-    // (nested scales keep two more registers per segment and ring slot)
+    // Rows of three and more segments per thread (wider than 8192 weights)
+    // also take two: a 4096 x 11008 weight has only two four-row batches per
+    // team, and the multiply of the last one is exposed (9.3 -> 8.6 us).
     constexpr int kRows =
         kLight ? RTHIP_GEMV_ROWS
-               : (kX * kSegments <= 4 && !(kDoubleQuantized && kSegments >= 3)
-                      ? 4
-                      : 2);
+               : (kX * kSegments <= 4 && kSegments < 3 ? 4 : 2);
     constexpr int kDepth = kLight ? RTHIP_GEMV_DEPTH : 2;
     constexpr unsigned kMaxIterations = kParkedValues / (kRows * kX);
     const LinearProblem& first = launch.problems[0];
