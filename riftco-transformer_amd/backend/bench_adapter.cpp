@@ -173,5 +173,55 @@ int main(int argc, char** argv) {
             }
         }
     }
+    // The decoder's pattern (src/model/decoder_only_transformer.cpp:406-419):
+    // three projections of one input per step, outputs alive together.
+    {
+        constexpr std::size_t width = 4096;
+        std::vector<std::unique_ptr<backend::QuantizedWeightStorage>> weights;
+        for (int m = 0; m < 3; ++m) {
+            std::vector<std::uint8_t> codes(width * width / 2);
+            for (auto& byte : codes) {
+                byte = static_cast<std::uint8_t>(random() & 0xFFU);
+            }
+            backend::Nf4ScaleStorageData scales;
+            scales.fp32_scales.assign(width * width / 64, 0.05F);
+            weights.push_back(backend::make_nf4_weight_storage(
+                kHip, std::move(codes), std::move(scales)));
+        }
+        std::vector<float> x(width);
+        for (auto& value : x) {
+            value = static_cast<float>(random() % 2001) / 1000.0F - 1.0F;
+        }
+        const auto input = backend::make_tensor_storage(kHip, x);
+        const backend::QuantizedLinearDimensions dimensions{1, width, width,
+                                                            64};
+        double checksum = 0.0;
+        for (int phase = 0; phase < 2; ++phase) {  // 0: warm-up
+            const int repeats = phase == 0 ? 20 : calls;
+            const auto begin = std::chrono::steady_clock::now();
+            std::unique_ptr<backend::TensorStorage> outputs[3];
+            for (int call = 0; call < repeats; ++call) {
+                for (auto& output : outputs) {
+                    output = backend::make_tensor_storage(kHip, width, 0.0F);
+                }
+                for (int m = 0; m < 3; ++m) {
+                    backend::dispatch_quantized_linear_forward(
+                        kHip, {*input, *weights[m], *outputs[m], dimensions});
+                }
+            }
+            checksum += std::as_const(*outputs[2]).data()[0];
+            if (phase == 1) {
+                const auto merged =
+                    backend::hip_forward_merge_statistics();
+                std::printf("q/k/v 3 x 4096x4096    %8.2f us per projection "
+                            "(%d steps, checksum %.6g; merged %llu requests "
+                            "into %llu launches)\n",
+                            seconds_since(begin) / (3.0 * repeats) * 1e6,
+                            repeats, checksum,
+                            static_cast<unsigned long long>(merged.requests),
+                            static_cast<unsigned long long>(merged.launches));
+            }
+        }
+    }
     return 0;
 }

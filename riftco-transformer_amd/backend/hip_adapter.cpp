@@ -34,6 +34,8 @@
 #include "core/backend/optim/adam/reference/update.hpp"
 #endif
 
+#include <array>
+#include <cstdint>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -89,6 +91,12 @@ bool environment_flag(const char* name) noexcept {
     const char* value = std::getenv(name);
     return value != nullptr && std::strcmp(value, "1") == 0;
 }
+
+// Decode-sized forwards that RIFTCO_TRANSFORMER_HIP_MERGE=1 holds back (see
+// PendingForwards below) name device memory by address, so they have to be
+// launched before any of that memory changes hands or is looked at.
+void launch_pending_forwards();
+void launch_pending_forwards_or_abort() noexcept;
 
 // Activation buffers come and go with every operation
 // (src/nn/quantized_linear.cpp:41 allocates the output of each forward), and
@@ -247,6 +255,7 @@ private:
         if (pointer_ == nullptr) {
             return;
         }
+        launch_pending_forwards_or_abort();
         if (kind_ == Kind::Pooled) {
             BufferPool::instance().release(pointer_, capacity_);
         } else {
@@ -269,11 +278,118 @@ private:
 // operation is not needed for correctness; RIFTCO_TRANSFORMER_HIP_ASYNC=1
 // drops it, and operations then queue behind each other on the device.
 // (Errors of a queued kernel surface at the next synchronising call.)
+bool merge_requested() noexcept {
+    static const bool merge = environment_flag("RIFTCO_TRANSFORMER_HIP_MERGE");
+    return merge;
+}
+
 void finish_operation(const HipRuntime& runtime, std::string_view operation) {
     static const bool deferred =
-        environment_flag("RIFTCO_TRANSFORMER_HIP_ASYNC");
+        environment_flag("RIFTCO_TRANSFORMER_HIP_ASYNC") || merge_requested();
     if (!deferred) {
         check(runtime, runtime.stream_synchronize(nullptr), operation);
+    }
+}
+
+// RIFTCO_TRANSFORMER_HIP_MERGE=1 (which implies the queued execution of
+// RIFTCO_TRANSFORMER_HIP_ASYNC=1).  A decoder calls the query, key and value
+// projections -- and gate and up -- one after the other on the same input
+// (src/model/decoder_only_transformer.cpp:406-419), each through
+// quantized_linear_forward.  At one to four rows a launch costs about as much
+// as the bytes it reads, so consecutive forwards that share their input are
+// held back here and go out together through rthip_nf4_linear_forward_group,
+// whose outputs are bit for bit those of separate launches.
+//
+// What is held back is a list of device addresses, so it is launched
+//   - when a forward arrives that does not fit the list (other input, shape,
+//     encoding; an output already in the list) or the list is full,
+//   - before any other operation of the adapter,
+//   - before host code sees a tensor (data()), and
+//   - before any device buffer is released.
+// An error of a held-back launch is reported by the call that launches it.
+class PendingForwards final {
+public:
+    static constexpr std::size_t kMaximumRows = 4;  // the decode kernel's range
+    static constexpr std::size_t kCapacity = 4;     // weights per launch
+
+    struct Shape {
+        const float* input = nullptr;
+        std::int32_t encoding = 0;
+        std::size_t second_level_block = 0;
+        std::size_t rows = 0;
+        std::size_t input_width = 0;
+        std::size_t block_size = 0;
+        [[nodiscard]] bool operator==(const Shape&) const noexcept = default;
+    };
+
+    static PendingForwards& instance() {
+        static PendingForwards pending;
+        return pending;
+    }
+
+    void add(const Shape& shape, const rthip_nf4_member& member) {
+        const std::lock_guard<std::mutex> lock(mutex_);
+        ++statistics_.requests;
+        bool fits = count_ != 0 && count_ < kCapacity && shape == shape_;
+        for (std::size_t m = 0; fits && m < count_; ++m) {
+            fits = members_[m].y != member.y;
+        }
+        if (!fits) {
+            launch_locked();
+        }
+        shape_ = shape;
+        members_[count_++] = member;
+        if (count_ == kCapacity) {
+            launch_locked();
+        }
+    }
+
+    void launch() {
+        const std::lock_guard<std::mutex> lock(mutex_);
+        launch_locked();
+    }
+
+    [[nodiscard]] HipForwardMergeStatistics statistics() noexcept {
+        const std::lock_guard<std::mutex> lock(mutex_);
+        return statistics_;
+    }
+
+private:
+    void launch_locked() {
+        if (count_ == 0) {
+            return;
+        }
+        const std::size_t count = std::exchange(count_, 0);
+        ++statistics_.launches;
+        const HipRuntime& runtime = require_runtime();
+        check(runtime,
+              runtime.nf4_linear_forward_group(
+                  shape_.input, members_.data(), count, shape_.encoding,
+                  shape_.second_level_block, shape_.rows, shape_.input_width,
+                  shape_.block_size, nullptr),
+              "quantized-linear forward (merged launch)");
+    }
+
+    std::mutex mutex_;
+    Shape shape_;
+    std::array<rthip_nf4_member, kCapacity> members_{};
+    std::size_t count_ = 0;
+    HipForwardMergeStatistics statistics_{};
+};
+
+void launch_pending_forwards() {
+    if (merge_requested()) {
+        PendingForwards::instance().launch();
+    }
+}
+
+// For destructors and the noexcept accessors: a launch that fails there ends
+// the process, as a failing read-back does (refresh_host).
+void launch_pending_forwards_or_abort() noexcept {
+    try {
+        launch_pending_forwards();
+    } catch (...) {
+        std::abort();
     }
 }
 
@@ -365,6 +481,7 @@ private:
     // noexcept by contract: a failing device read-back ends the process, as a
     // failing access to a managed CUDA allocation would.
     void refresh_host() const noexcept {
+        launch_pending_forwards_or_abort();
         if (freshest_ != Freshest::Device) {
             return;
         }
@@ -636,6 +753,27 @@ public:
         const auto& weight = require_hip_weight(request.weight, operation);
         auto& output = require_hip_tensor(request.output, operation);
         const float* source = input.device_for_read();
+        if (merge_requested() &&
+            request.dimensions.rows <= PendingForwards::kMaximumRows) {
+            rthip_nf4_member member{};
+            member.codes = static_cast<const std::uint8_t*>(
+                weight.packed_codes_native_handle());
+            member.primary_scales = weight.primary_scales_native_handle();
+            member.secondary_scales = static_cast<const float*>(
+                weight.secondary_scales_native_handle());
+            member.offset = weight.offset();
+            member.bias_or_null = nullptr;
+            member.y = output.device_for_overwrite();
+            member.output_width = request.dimensions.output_width;
+            PendingForwards::instance().add(
+                {source, static_cast<std::int32_t>(weight.encoding()),
+                 weight.second_level_block_size(), request.dimensions.rows,
+                 request.dimensions.input_width,
+                 request.dimensions.block_size},
+                member);
+            return;
+        }
+        launch_pending_forwards();
         check(runtime,
               runtime.nf4_linear_forward(
                   source,
@@ -664,6 +802,7 @@ public:
         const auto& upstream = require_hip_tensor(request.upstream, operation);
         const auto& weight = require_hip_weight(request.weight, operation);
         auto& gradient = require_hip_tensor(request.input_gradient, operation);
+        launch_pending_forwards();
         const float* source = upstream.device_for_read();
         check(runtime,
               runtime.nf4_linear_input_backward(
@@ -695,6 +834,7 @@ public:
     void matmul(const MatmulRequest& request) const override {
         constexpr std::string_view operation = "matmul";
         const HipRuntime& runtime = require_runtime();
+        launch_pending_forwards();
         const auto& left = require_hip_tensor(request.left, operation);
         const auto& right = require_hip_tensor(request.right, operation);
         auto& output = require_hip_tensor(request.output, operation);
@@ -818,6 +958,10 @@ const BackendAdapter& hip_backend_adapter() noexcept {
     return adapter;
 }
 
+HipForwardMergeStatistics hip_forward_merge_statistics() noexcept {
+    return PendingForwards::instance().statistics();
+}
+
 void hip_quantized_linear_forward_group(
     std::span<const QuantizedLinearForwardRequest> requests
 ) {
@@ -827,6 +971,7 @@ void hip_quantized_linear_forward_group(
             "a quantized-linear group needs at least one request");
     }
     const HipRuntime& runtime = require_runtime();
+    launch_pending_forwards();
     const QuantizedLinearForwardRequest& first = requests.front();
     const auto& input = require_hip_tensor(first.input, operation);
     const auto& first_weight = require_hip_weight(first.weight, operation);

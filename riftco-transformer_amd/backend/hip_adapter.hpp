@@ -69,6 +69,20 @@ struct HipPackedWeightSource {
 void hip_quantized_linear_forward_group(
     std::span<const QuantizedLinearForwardRequest> requests);
 
+// RIFTCO_TRANSFORMER_HIP_MERGE=1 gives callers that were NOT changed the same
+// launches: quantized_linear_forward calls of one to four rows that follow
+// each other on the same input are held back and launched together (at most
+// four weights per launch) as soon as a call arrives that does not belong to
+// them, another operation of the adapter runs, host code reads a tensor, or a
+// device buffer is released.  It implies RIFTCO_TRANSFORMER_HIP_ASYNC=1.
+// requests: forwards that went through the merge; launches: kernel launches
+// they became.  Both stay zero while the option is off.
+struct HipForwardMergeStatistics {
+    std::uint64_t requests = 0;
+    std::uint64_t launches = 0;
+};
+[[nodiscard]] HipForwardMergeStatistics hip_forward_merge_statistics() noexcept;
+
 // Optional extension implemented by hip weight storage: the O(#blocks) scale
 // validation that the dispatcher runs before every launch
 // (src/core/backend/nn/quantized_linear/dispatch.cpp:98-151) only has to run

@@ -526,6 +526,100 @@ void test_forward_group() {
     }
 }
 
+void test_merged_forwards() {
+    // The decoder's pattern, unchanged callers: three projections of one
+    // input and then one of another, each through the dispatcher.  Results are
+    // those of the CPU oracle in every mode; with
+    // RIFTCO_TRANSFORMER_HIP_MERGE=1 the four requests become two launches,
+    // and what is held back is launched before anything can observe it.
+    namespace detail = riftco_transformer::backend_detail;
+    const char* option = std::getenv("RIFTCO_TRANSFORMER_HIP_MERGE");
+    const bool merging = option != nullptr && std::string_view(option) == "1";
+    const std::size_t widths[] = {96, 64, 130};
+    for (const bool double_quantized : {false, true}) {
+        std::vector<HostWeight> weights;
+        std::vector<std::unique_ptr<backend::QuantizedWeightStorage>> storages;
+        for (std::size_t m = 0; m < 3; ++m) {
+            weights.push_back(quantize(
+                pseudo_normal(widths[m] * 256, 0.02F, 70 + m), widths[m], 256,
+                64, double_quantized, 256));
+            storages.push_back(to_hip(weights.back()));
+        }
+        for (const std::size_t rows : {std::size_t{1}, std::size_t{4}}) {
+            const auto input = pseudo_normal(rows * 256, 1.0F, 80 + rows);
+            const auto other_input = pseudo_normal(rows * 256, 1.0F, 90 + rows);
+            auto source = backend::make_tensor_storage(kHip, input);
+            auto other_source = backend::make_tensor_storage(kHip, other_input);
+            std::vector<std::unique_ptr<backend::TensorStorage>> targets;
+            for (std::size_t m = 0; m < 3; ++m) {
+                targets.push_back(backend::make_tensor_storage(
+                    kHip, rows * widths[m], 0.0F));
+            }
+            auto other_target =
+                backend::make_tensor_storage(kHip, rows * widths[0], 0.0F);
+            const auto before = detail::hip_forward_merge_statistics();
+            for (std::size_t m = 0; m < 3; ++m) {
+                backend::dispatch_quantized_linear_forward(
+                    kHip, {*source, *storages[m], *targets[m],
+                           {rows, 256, widths[m], 64}});
+            }
+            backend::dispatch_quantized_linear_forward(
+                kHip, {*other_source, *storages[0], *other_target,
+                       {rows, 256, widths[0], 64}});
+            // twice into the same output: the second call must find the
+            // first one launched, not share a launch with it
+            backend::dispatch_quantized_linear_forward(
+                kHip, {*other_source, *storages[0], *other_target,
+                       {rows, 256, widths[0], 64}});
+            for (std::size_t m = 0; m < 3; ++m) {
+                const auto data = std::as_const(*targets[m]).data();
+                require_close({data.begin(), data.end()},
+                              oracle_forward(input, weights[m]),
+                              "a forward that may have been merged must match "
+                              "the CPU oracle");
+            }
+            const auto data = std::as_const(*other_target).data();
+            require_close({data.begin(), data.end()},
+                          oracle_forward(other_input, weights[0]),
+                          "two forwards into one output, one after the other");
+            const auto after = detail::hip_forward_merge_statistics();
+            if (merging) {
+                require(after.requests - before.requests == 5 &&
+                            after.launches - before.launches == 3,
+                        "five forwards (three sharing an input, two into one "
+                        "output) must become three launches");
+            } else {
+                require(after.requests == 0 && after.launches == 0,
+                        "nothing is merged unless it was asked for");
+            }
+        }
+        // a tensor that is released while a launch that writes it is held
+        // back: the launch goes out first (no write into recycled memory)
+        const auto input = pseudo_normal(256, 1.0F, 99);
+        auto source = backend::make_tensor_storage(kHip, input);
+        auto kept = backend::make_tensor_storage(kHip, widths[1], 0.0F);
+        {
+            auto dropped = backend::make_tensor_storage(kHip, widths[0], 0.0F);
+            backend::dispatch_quantized_linear_forward(
+                kHip, {*source, *storages[0], *dropped,
+                       {1, 256, widths[0], 64}});
+        }
+        auto recycled = backend::make_tensor_storage(kHip, widths[0], 7.0F);
+        backend::dispatch_quantized_linear_forward(
+            kHip, {*source, *storages[1], *kept, {1, 256, widths[1], 64}});
+        const auto untouched = std::as_const(*recycled).data();
+        for (const float value : untouched) {
+            require(value == 7.0F,
+                    "a held-back launch must not write into a buffer that "
+                    "was released and handed out again");
+        }
+        const auto data = std::as_const(*kept).data();
+        require_close({data.begin(), data.end()},
+                      oracle_forward(input, weights[1]),
+                      "forward after a released output");
+    }
+}
+
 void test_tensor_storage() {
     auto filled = backend::make_tensor_storage(kHip, 5, 1.5F);
     require(filled->backend() == kHip && filled->size() == 5 &&
@@ -1005,6 +1099,7 @@ int main(int argc, char** argv) {
         test_accelerator_oracle();
         test_transformer_sized_layer();
         test_forward_group();
+        test_merged_forwards();
         test_tensor_storage();
         test_dispatch_validation();
         test_packed_model_state();

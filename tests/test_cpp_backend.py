@@ -47,9 +47,12 @@ def test_adapter_on_the_host_only_runtime():
     {"RIFTCO_TRANSFORMER_HIP_POOL": "0"},
     {"RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
     {"RIFTCO_TRANSFORMER_HIP_POOL": "0", "RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
+    {"RIFTCO_TRANSFORMER_HIP_MERGE": "1"},
+    {"RIFTCO_TRANSFORMER_HIP_POOL": "0", "RIFTCO_TRANSFORMER_HIP_MERGE": "1"},
 ])
 def test_adapter_options_on_the_host_only_runtime(options):
-    """Without the buffer pool, and without the per-operation synchronise."""
+    """Without the buffer pool, without the per-operation synchronise, and
+    with decode-sized forwards that share an input merged into one launch."""
     expect_pass(run(RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE,
                     RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1", **options))
 
@@ -165,6 +168,7 @@ def test_adapter_on_the_real_library():
 @pytest.mark.parametrize("options", [
     {"RIFTCO_TRANSFORMER_HIP_POOL": "0"},
     {"RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
+    {"RIFTCO_TRANSFORMER_HIP_MERGE": "1"},
 ])
 def test_adapter_options_on_the_real_library(options):
     """The pool switched off, and operations queued without a synchronise per
