@@ -66,6 +66,10 @@ namespace rthip {
 namespace {
 
 constexpr int kWorkgroupThreads = 512;
+// Four teams: a workgroup of sixteen wavefronts (teams stay 256 threads wide).
+constexpr int workgroup_threads(int teams) {
+    return teams == 4 ? 2 * kWorkgroupThreads : kWorkgroupThreads;
+}
 constexpr int kSegment = 16;       // weights per thread per row visit
 constexpr unsigned kComputeUnits = 256;
 // Row totals a team may park in LDS before the final barrier, per wavefront.
@@ -163,14 +167,14 @@ static_assert(RTHIP_GEMV_ROWS <= 4, "two scale loads cover four rows");
 // before: every member selection folds to member 0).
 template <int kX, int kSegments, int kRows, int kTeams, int kDepth,
           bool kDoubleQuantized, bool kGrouped>
-__global__ __launch_bounds__(kWorkgroupThreads) void gemv_forward_kernel(
+__global__ __launch_bounds__(workgroup_threads(kTeams)) void gemv_forward_kernel(
     const float* __restrict__ x, GemvGroup group, unsigned second_level_shift,
     unsigned x_rows, unsigned input_width, unsigned block_shift,
     unsigned batch_count, unsigned iterations, LoraEpilogue lora
 ) {
-    constexpr int kThreads = kWorkgroupThreads;
+    constexpr int kThreads = workgroup_threads(kTeams);
     // threads that share one weight row
-    constexpr int kTeamThreads = kWorkgroupThreads / kTeams;
+    constexpr int kTeamThreads = kThreads / kTeams;
     constexpr int kTeamWaves = kTeamThreads / kWave;
     constexpr int kValues = kRows * kX;
     constexpr unsigned kMaxIterations = kParkedValues / kValues;
@@ -595,14 +599,23 @@ struct Launch {
     std::size_t count;
 };
 
+// Launches that read this many bytes of codes or more run sixteen wavefronts
+// per workgroup instead of eight: a long run gains from the fuller issue
+// slots (32000 x 4096: 17.2 -> 16.8 us, nested scales 19.6 -> 17.9 us), a
+// short one loses more at its start (4096 x 4096: 4.7 -> 5.2 us; two
+// 11008 x 4096 in one launch: 12.9 -> 14.3 us).
+constexpr std::size_t kLargeLaunchBytes = std::size_t{60} << 20;
+
 template <int kX, int kSegments, bool kDoubleQuantized, bool kGrouped,
-          bool kWide = false>
+          bool kWide = false, bool kLarge = false>
 void launch_instance(const Launch& launch, hipStream_t stream) {
     // Two teams (eight wavefronts) per workgroup measured best on MI355X; a
     // thread that carries more x rows or segments takes fewer weight rows per
     // batch so that its registers fit.
     constexpr bool kLight = kX * kSegments == 1;
-    constexpr int kTeams = kWide ? 1 : (kLight ? RTHIP_GEMV_TEAMS : 2);
+    static_assert(!kLarge || (kX * kSegments == 1 && !kWide));
+    constexpr int kTeams =
+        kWide ? 1 : (kLarge ? 4 : (kLight ? RTHIP_GEMV_TEAMS : 2));
     // Rows of three and more segments per thread (wider than 8192 weights)
     // also take two: a 4096 x 11008 weight has only two four-row batches per
     // team, and the multiply of the last one is exposed (9.3 -> 8.6 us).
@@ -649,7 +662,7 @@ void launch_instance(const Launch& launch, hipStream_t stream) {
     }
     const unsigned iterations = (team_groups + blocks - 1) / blocks;
     gemv_forward_kernel<kX, kSegments, kRows, kTeams, kDepth, kDoubleQuantized,
-                        kGrouped><<<blocks, kWorkgroupThreads, 0, stream>>>(
+                        kGrouped><<<blocks, workgroup_threads(kTeams), 0, stream>>>(
         first.activations, group, first.weight.second_level_shift,
         static_cast<unsigned>(first.rows),
         static_cast<unsigned>(first.input_width), first.block_shift,
@@ -670,6 +683,18 @@ void launch_segments(const Launch& launch, hipStream_t stream) {
     }
     switch (segments_per_thread(p, 256)) {
     case 1:
+        if constexpr (kX == 1) {
+            std::size_t code_bytes = 0;
+            for (std::size_t m = 0; m < launch.count; ++m) {
+                code_bytes += launch.problems[m].output_width *
+                              launch.problems[m].input_width / 2;
+            }
+            if (code_bytes >= kLargeLaunchBytes) {
+                launch_instance<1, 1, kDoubleQuantized, kGrouped, false, true>(
+                    launch, stream);
+                break;
+            }
+        }
         launch_instance<kX, 1, kDoubleQuantized, kGrouped>(launch, stream);
         break;
     case 2:

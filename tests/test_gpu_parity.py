@@ -361,6 +361,37 @@ def test_group_of_weights_that_share_an_input(gpu, package, library, oracle,
                     f"member {m} at {rows} rows vs CPU oracle: {drift:.3g}"
 
 
+@pytest.mark.parametrize("double_quantized", [False, True])
+def test_launches_that_read_more_than_sixty_megabytes(gpu, package, library,
+                                                      oracle,
+                                                      double_quantized):
+    """From 60 MB of codes per launch on, the decode kernel runs sixteen
+    wavefronts per workgroup: the vocabulary projection (32000 x 4096) against
+    the CPU oracle, and four 11008 x 4096 weights in one launch against one
+    launch each (eight wavefronts per workgroup), bit for bit."""
+    in_w = 4096
+    x = helpers.normal(401, (1, in_w), 1.0)
+    x_device = to_device(x)
+    head = oracle.quantize(helpers.normal(400, (32000, in_w), 0.02), 64,
+                           double_quantized, 256)
+    y = host(gpu.linear_forward(x_device, upload(gpu, head)))
+    drift = helpers.normalized_error(
+        y, oracle.forward(x, head, None), in_w, helpers.rms(x),
+        helpers.rms(oracle.dequantize(head)))
+    # the largest deviation of 32000 outputs, not of 4096: twice the margin
+    assert drift <= 2 * TOLERANCE, f"32000 x 4096 vs CPU oracle: {drift:.3g}"
+    del head
+    weights = [upload(gpu, oracle.quantize(
+        helpers.normal(402 + m, (11008, in_w), 0.02), 64, double_quantized,
+        256)) for m in range(2)]
+    members = [weights[0], weights[1], weights[1], weights[0]]
+    together = gpu.linear_forward_group(x_device, members)
+    for m, weight in enumerate(members):
+        helpers.assert_bit_equal(host(together[m]),
+                                 host(gpu.linear_forward(x_device, weight)),
+                                 f"member {m} of a 90 MB launch")
+
+
 def test_group_arguments_are_checked(gpu, package, library, oracle):
     weight = upload(gpu, oracle.quantize(helpers.normal(1, (64, 64), 0.02),
                                          64, False, 256))
