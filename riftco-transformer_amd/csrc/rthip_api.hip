@@ -194,6 +194,19 @@ int32_t select_forward(const rthip::LinearProblem& problem) {
     return RTHIP_NF4_ALGORITHM_GENERIC;
 }
 
+// Row counts just above the small-batch kernels' limit run as two launches
+// of those kernels (AUTO only; see linear_forward_common).
+constexpr std::size_t kSplitHeadRows = 64;
+constexpr std::size_t kForwardSplitMaxRows = 112;
+constexpr std::size_t kBackwardSplitMaxRows = 96;
+bool split_rows(std::size_t rows, std::size_t limit) {
+    return rows > kSplitHeadRows && rows <= limit;
+}
+bool small_batch_family(int32_t algorithm) {
+    return algorithm == RTHIP_NF4_ALGORITHM_RESIDENT ||
+           algorithm == RTHIP_NF4_ALGORITHM_SKINNY;
+}
+
 int32_t select_input_backward(const rthip::LinearProblem& problem) {
     if (problem.rows <= rthip::kSmallBackwardMaxRows &&
         rthip::small_input_backward_supports(problem)) {
@@ -203,6 +216,59 @@ int32_t select_input_backward(const rthip::LinearProblem& problem) {
         return RTHIP_NF4_ALGORITHM_MFMA;
     }
     return RTHIP_NF4_ALGORITHM_GENERIC;
+}
+
+// Just past the small-batch kernels' 64 rows the tiled kernel would run a
+// 128-row tile that is mostly padding (65 rows of 11008 x 4096: 117 us against
+// 57 us at 64 rows).  AUTO then sends the first 64 rows and the rest through
+// the small-batch families, one launch after the other (74 us; equal from
+// about 112 rows on).  True if `problem` is such a case; head and tail are
+// then the two problems and their families.
+struct RowSplit {
+    rthip::LinearProblem head, tail;
+    int32_t head_family, tail_family;
+};
+bool forward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
+    if (!split_rows(problem.rows, kForwardSplitMaxRows)) {
+        return false;
+    }
+    split->head = problem;
+    split->head.rows = kSplitHeadRows;
+    split->tail = problem;
+    split->tail.rows = problem.rows - kSplitHeadRows;
+    if (problem.activations != nullptr) {  // null: a shape query
+        split->tail.activations += kSplitHeadRows * problem.input_width;
+        split->tail.result += kSplitHeadRows * problem.output_width;
+    }
+    if (split->tail.lora.reduced != nullptr) {
+        split->tail.lora.reduced += kSplitHeadRows * problem.lora.rank;
+    }
+    split->head_family = select_forward(split->head);
+    split->tail_family = select_forward(split->tail);
+    return small_batch_family(split->head_family) &&
+           (small_batch_family(split->tail_family) ||
+            split->tail_family == RTHIP_NF4_ALGORITHM_GEMV);
+}
+// The input backward likewise up to 96 rows (11008 x 4096: 117 -> 86...100
+// us), unless dx is much wider than dy, where the tiled kernel is as fast
+// (4096 x 11008: 117 against 113...132 us).
+bool backward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
+    if (!split_rows(problem.rows, kBackwardSplitMaxRows) ||
+        problem.input_width > 2 * problem.output_width) {
+        return false;
+    }
+    split->head = problem;
+    split->head.rows = kSplitHeadRows;
+    split->tail = problem;
+    split->tail.rows = problem.rows - kSplitHeadRows;
+    if (problem.activations != nullptr) {  // null: a shape query
+        split->tail.activations += kSplitHeadRows * problem.output_width;
+        split->tail.result += kSplitHeadRows * problem.input_width;
+    }
+    split->head_family = select_input_backward(split->head);
+    split->tail_family = select_input_backward(split->tail);
+    return split->head_family == RTHIP_NF4_ALGORITHM_SKINNY &&
+           split->tail_family == RTHIP_NF4_ALGORITHM_SKINNY;
 }
 
 }  // namespace
@@ -337,10 +403,15 @@ rthip_status rthip_nf4_select_algorithm(
     problem.input_width = input_width;
     problem.output_width = output_width;
     problem.block_shift = block_shift;
+    RowSplit split;
     if (direction == 0) {
-        *algorithm = select_forward(problem);
+        *algorithm = forward_row_split(problem, &split)
+                         ? split.head_family
+                         : select_forward(problem);
     } else if (direction == 1) {
-        *algorithm = select_input_backward(problem);
+        *algorithm = backward_row_split(problem, &split)
+                         ? split.head_family
+                         : select_input_backward(problem);
     } else {
         return fail(RTHIP_INVALID_ARGUMENT,
                     "direction must be 0 (forward) or 1 (input backward)");
@@ -411,9 +482,10 @@ rthip_status linear_forward_common(
         problem.lora.scale = lora.scale;
     }
 
-    if (algorithm == RTHIP_NF4_ALGORITHM_AUTO) {
-        algorithm = select_forward(problem);
-    }
+    // One family on one problem; RTHIP_OK means "launched".
+    const auto launch = [hip_stream](int32_t algorithm,
+                                     const rthip::LinearProblem& problem)
+        -> rthip_status {
     switch (algorithm) {
     case RTHIP_NF4_ALGORITHM_GENERIC:
         rthip::launch_generic_forward(problem, hip_stream);
@@ -469,6 +541,30 @@ rthip_status linear_forward_common(
     default:
         return fail(RTHIP_INVALID_ARGUMENT, "unknown algorithm %d",
                     static_cast<int>(algorithm));
+    }
+    return RTHIP_OK;
+    };
+
+    if (algorithm == RTHIP_NF4_ALGORITHM_AUTO) {
+        RowSplit split;
+        if (forward_row_split(problem, &split)) {
+            if (const rthip_status status =
+                    launch(split.head_family, split.head);
+                status != RTHIP_OK) {
+                return status;
+            }
+            if (const rthip_status status =
+                    launch(split.tail_family, split.tail);
+                status != RTHIP_OK) {
+                return status;
+            }
+            return finish_launch("NF4 linear forward launch");
+        }
+        algorithm = select_forward(problem);
+    }
+    if (const rthip_status status = launch(algorithm, problem);
+        status != RTHIP_OK) {
+        return status;
     }
     return finish_launch("NF4 linear forward launch");
 }
@@ -779,9 +875,9 @@ rthip_status rthip_nf4_linear_input_backward_with(
     problem.output_width = output_width;
     const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
 
-    if (algorithm == RTHIP_NF4_ALGORITHM_AUTO) {
-        algorithm = select_input_backward(problem);
-    }
+    const auto launch = [hip_stream](int32_t algorithm,
+                                     const rthip::LinearProblem& problem)
+        -> rthip_status {
     switch (algorithm) {
     case RTHIP_NF4_ALGORITHM_GENERIC:
         rthip::launch_generic_input_backward(problem, hip_stream);
@@ -820,6 +916,30 @@ rthip_status rthip_nf4_linear_input_backward_with(
     default:
         return fail(RTHIP_INVALID_ARGUMENT, "unknown algorithm %d",
                     static_cast<int>(algorithm));
+    }
+    return RTHIP_OK;
+    };
+
+    if (algorithm == RTHIP_NF4_ALGORITHM_AUTO) {
+        RowSplit split;
+        if (backward_row_split(problem, &split)) {
+            if (const rthip_status status =
+                    launch(split.head_family, split.head);
+                status != RTHIP_OK) {
+                return status;
+            }
+            if (const rthip_status status =
+                    launch(split.tail_family, split.tail);
+                status != RTHIP_OK) {
+                return status;
+            }
+            return finish_launch("NF4 linear input-backward launch");
+        }
+        algorithm = select_input_backward(problem);
+    }
+    if (const rthip_status status = launch(algorithm, problem);
+        status != RTHIP_OK) {
+        return status;
     }
     return finish_launch("NF4 linear input-backward launch");
 }

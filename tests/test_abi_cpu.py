@@ -49,7 +49,6 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     # small batches -> weights decoded straight into MFMA operands
     assert select(fwd, 16, 256, 768, 64) == package.ALGORITHM_SKINNY
     assert select(fwd, 64, 11008, 4096, 64) == package.ALGORITHM_SKINNY
-    assert select(fwd, 65, 4096, 11008, 64) == package.ALGORITHM_MFMA
     assert select(fwd, 16, 128, 768, 32) == package.ALGORITHM_SKINNY
     # up to 64 rows and a row width of 1024..4096 -> x resident in registers
     assert select(fwd, 16, 4096, 11008, 64) == package.ALGORITHM_RESIDENT
@@ -57,7 +56,11 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(fwd, 8, 3072, 1000, 32) == package.ALGORITHM_RESIDENT
     assert select(fwd, 17, 4096, 4096, 64) == package.ALGORITHM_RESIDENT
     assert select(fwd, 64, 4096, 11008, 64) == package.ALGORITHM_RESIDENT
-    assert select(fwd, 65, 4096, 11008, 64) == package.ALGORITHM_MFMA
+    # 65...112 rows: the first 64 and the rest as two small-batch launches
+    # (the family of the first 64 rows is reported), the tiled GEMM after that
+    assert select(fwd, 65, 4096, 11008, 64) == package.ALGORITHM_RESIDENT
+    assert select(fwd, 112, 11008, 4096, 64) == package.ALGORITHM_SKINNY
+    assert select(fwd, 113, 4096, 11008, 64) == package.ALGORITHM_MFMA
     assert select(fwd, 16, 11008, 4096, 64) == package.ALGORITHM_SKINNY
     assert select(fwd, 16, 5120, 4096, 64) == package.ALGORITHM_SKINNY
     # (row width a multiple of 32 but not of 64 -> tiled GEMM)
@@ -70,6 +73,10 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(bwd, 1, 4096, 11008, 64) == package.ALGORITHM_SKINNY
     assert select(bwd, 64, 11008, 4096, 64) == package.ALGORITHM_SKINNY
     assert select(bwd, 16, 40, 768, 32) == package.ALGORITHM_SKINNY
+    # 65...96 rows: two launches of it, unless dx is much wider than dy
+    assert select(bwd, 65, 4096, 11008, 64) == package.ALGORITHM_SKINNY
+    assert select(bwd, 96, 4096, 4096, 64) == package.ALGORITHM_SKINNY
+    assert select(bwd, 97, 4096, 11008, 64) == package.ALGORITHM_MFMA
     assert select(bwd, 65, 11008, 4096, 64) == package.ALGORITHM_MFMA
     assert select(bwd, 16, 36, 768, 32) == package.ALGORITHM_GENERIC
     # the reference's edge layout -> shape-agnostic kernels

@@ -216,7 +216,8 @@ def test_llama_rows_against_golden(gpu, package, library, oracle, name,
                                     weight_rms) <= TOLERANCE + own
 
 
-@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 16, 64, 130])
+@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 16, 64, 65, 67, 96, 97, 112,
+                                  113, 130])
 @pytest.mark.parametrize("double_quantized", [False, True])
 def test_row_counts_across_the_gemv_mfma_crossover(
         gpu, package, library, oracle, rows, double_quantized):
@@ -443,9 +444,15 @@ def test_small_batch_input_backward(gpu, package, library, oracle, out_w, in_w,
             helpers.assert_bit_equal(
                 host(gpu.linear_input_backward(dy_device, device_weight)),
                 first, f"{rows} rows, launch {launch}")
+    # 65...96 rows run as two launches of this kernel (unless dx is much
+    # wider than dy), more rows go to the tiled kernel
     assert library.select_algorithm(
-        package.INPUT_BACKWARD, 65, in_w, out_w,
+        package.INPUT_BACKWARD, 97, in_w, out_w,
         block) != package.ALGORITHM_SKINNY
+    rows = 80
+    x = helpers.normal(84 + rows, (rows, in_w), 1.0)
+    dy = helpers.normal(85 + rows, (rows, out_w), 1.0e-2)
+    check_layer(gpu, package, library, oracle, weight, x, dy, oracle_rows=2)
 
 
 def test_shared_output_tiles_are_added_in_a_fixed_order(gpu, package, library,
