@@ -616,7 +616,7 @@ def test_decode_shapes_small_batches(gpu, package, library, oracle):
     (768, 256, 64, 8, (1, 16)),         # the tiny parity layer
     (33, 33, 32, 1, (2,)),              # shape-agnostic kernels, rank one
     (1000, 1600, 64, 2, (1, 5, 70)),    # rank that is not a multiple of 4
-    (4096, 4096, 64, 16, (1, 4, 64, 300)),
+    (4096, 4096, 64, 16, (1, 4, 64, 100, 300)),  # 100: two launches
     (512, 2048, 128, 100, (3, 40)),     # more than one 64-row adapter chunk
 ])
 @pytest.mark.parametrize("double_quantized", [False, True])
