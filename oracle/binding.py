@@ -342,6 +342,9 @@ class Reference:
         lib.nf4ref_memory_usage.argtypes = [sz, sz, sz] + payload + [vp]
         lib.nf4ref_matmul.restype = i32
         lib.nf4ref_matmul.argtypes = [vp, vp, vp, sz, sz, sz]
+        lib.nf4ref_validate_scale_storage.restype = i32
+        lib.nf4ref_validate_scale_storage.argtypes = [
+            i32, vp, sz, vp, sz, vp, sz, sz, f32, sz]
         lib.nf4ref_lora_linear_forward.restype = i32
         lib.nf4ref_lora_linear_forward.argtypes = [
             vp, vp, vp, vp, sz, f32, vp, sz, sz, sz, sz] + payload
@@ -409,6 +412,13 @@ class Reference:
         # call that reaches it.
         self._run(0, None, weight, 0,
                   (weight.output_width, weight.input_width))
+
+    def validate_scale_storage(self, weight: Nf4Weight,
+                               expected_scale_count: int) -> None:
+        # require_scale_storage as the dispatcher applies it to a stored
+        # weight (dispatch.cpp:108-154, reached through :203-230)
+        self._check(self._lib.nf4ref_validate_scale_storage(
+            *self._payload_args(weight)[2:], expected_scale_count))
 
     def dequantize(self, weight: Nf4Weight) -> np.ndarray:
         return self._run(0, None, weight, 0,

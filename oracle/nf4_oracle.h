@@ -18,6 +18,14 @@
  *       tests/core/backend/test_quantized_linear_backend.cpp:89-169, an fp64
  *       brute force, and bit-for-bit agreement with the compiled reference
  *       (committed golden hashes/slices)
+ *   validate_payload                                - the payload rules the
+ *       reference's own tests exercise (tests/core/test_quantization.cpp:207-376)
+ *       and outcome + message of the compiled reference on damaged payloads
+ *   validate_scale_storage                          - outcome, exception type
+ *       and message of the compiled reference's dispatcher on forty sound and
+ *       damaged scale storages (committed as golden verdicts)
+ *   matmul, matmul_nt, add_bias, lora_linear_forward - bit-for-bit agreement
+ *       with the compiled reference's tensor operations
  * No function here is "parity unpinned".
  */
 #ifndef NF4_ORACLE_H

@@ -14,7 +14,10 @@
 //       src/core/backend/nn/quantized_linear/dispatch.hpp:19-27
 //   tensor_ops::matmul / transpose_2d / scale / add / broadcast_to
 //       include/riftco_transformer/core/tensor_ops.hpp:12-36
+//   require_scale_storage, reached through dispatch_quantized_linear_forward
+//       src/core/backend/nn/quantized_linear/dispatch.cpp:98-154,203-242
 
+#include "core/backend/adapter.hpp"
 #include "core/backend/nn/quantized_linear/dispatch.hpp"
 #include "riftco_transformer/core/backend.hpp"
 #include "riftco_transformer/core/quantized_weight.hpp"
@@ -298,6 +301,54 @@ int nf4ref_lora_linear_forward(
             ops::add(base, ops::scale(expanded, lora_scale));
         const auto data = result.data();
         std::copy(data.begin(), data.end(), y);
+    });
+}
+
+// The dispatcher's verdict on a scale storage held against an expected scale
+// count (require_scale_storage, dispatch.cpp:108-154).  The storage is built
+// by the CPU adapter itself, which checks nothing, with any combination of
+// arrays the caller asks for; the dispatcher then sees it through a forward
+// request whose dimensions (one row of 32 x expected_scale_count weights,
+// block size 32) make `expected_scale_count` the count it demands.  Packed
+// codes and tensors are sized to pass every check that runs before the scale
+// check (dispatch.cpp:317-333,203-230), so the first verdict that can differ
+// from "ok" is the scale storage's.
+int nf4ref_validate_scale_storage(
+    int encoding, const float* fp32_scales, std::size_t fp32_count,
+    const std::uint8_t* scale_codes, std::size_t scale_code_count,
+    const float* second_level, std::size_t second_level_count,
+    std::size_t second_level_block, float offset,
+    std::size_t expected_scale_count
+) {
+    return guarded([&] {
+        backend::Nf4ScaleStorageData data;
+        data.encoding = static_cast<backend::Nf4ScaleEncoding>(encoding);
+        if (fp32_count != 0) {
+            data.fp32_scales.assign(fp32_scales, fp32_scales + fp32_count);
+        }
+        if (scale_code_count != 0) {
+            data.quantized_scales.assign(scale_codes,
+                                         scale_codes + scale_code_count);
+        }
+        if (second_level_count != 0) {
+            data.second_level_scales.assign(
+                second_level, second_level + second_level_count);
+        }
+        data.second_level_block_size = second_level_block;
+        data.offset = offset;
+        const std::size_t input_width = 32 * expected_scale_count;
+        const auto* adapter =
+            backend::find_backend_adapter(ExecutionBackend::Cpu);
+        const auto weight = adapter->make_nf4_weight_storage(
+            std::vector<std::uint8_t>(input_width / 2, 0x77),
+            std::move(data));
+        const Tensor source({1, input_width}, ExecutionBackend::Cpu);
+        Tensor target({1, 1}, ExecutionBackend::Cpu);
+        backend::dispatch_quantized_linear_forward(
+            ExecutionBackend::Cpu,
+            {backend::tensor_storage(source), *weight,
+             backend::tensor_storage(target),
+             backend::QuantizedLinearDimensions{1, input_width, 1, 32}});
     });
 }
 

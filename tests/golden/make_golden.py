@@ -173,6 +173,18 @@ def packed_state(reference):
         json.dump(outcomes, handle, indent=1, sort_keys=True)
 
 
+def scale_storage_verdicts(reference):
+    """What the reference's dispatcher says about each scale storage of
+    helpers.scale_storage_cases() (its require_scale_storage, reached through
+    a forward request on the CPU backend)."""
+    verdicts = {
+        name: helpers.verdict(reference.validate_scale_storage, weight,
+                              expected)
+        for name, weight, expected in helpers.scale_storage_cases()}
+    with open(os.path.join(HERE, "scale_storage_verdicts.json"), "w") as out:
+        json.dump(verdicts, out, indent=1, sort_keys=True)
+
+
 def bits_of(array):
     return np.ascontiguousarray(array, dtype=np.float32).view(np.uint32)
 
@@ -180,6 +192,7 @@ def bits_of(array):
 def main():
     reference = Reference()
     packed_state(reference)
+    scale_storage_verdicts(reference)
     np.savez_compressed(os.path.join(HERE, "closed_form.npz"),
                         **closed_form(reference))
     arrays, meta1 = config1(reference)

@@ -187,3 +187,88 @@ def packed_state_mutations(blob: bytes):
         ("block_size_unchecked", patched(first + 8, "<Q", 7)),
     ]
     return cases
+
+
+def scale_storage_cases():
+    """(name, scale storage, expected scale count) triples for the
+    dispatcher's scale-storage check
+    (src/core/backend/nn/quantized_linear/dispatch.cpp:108-154): sound
+    storages of both encodings and, for every condition the check names, a
+    storage that breaks it alone -- and a few that break two, which pins the
+    order of the checks."""
+    from oracle.binding import (SCALE_DOUBLE_QUANTIZED_UINT8, SCALE_FLOAT32,
+                                Nf4Weight)
+    f32 = np.float32
+    big = float(np.finfo(np.float32).max)
+
+    def storage(encoding, fp32=None, codes=None, second=None, block=0,
+                offset=0.0):
+        return Nf4Weight(
+            1, 1, 32, np.array([0x07], np.uint8), encoding,
+            fp32_scales=None if fp32 is None else np.array(fp32, f32),
+            scale_codes=None if codes is None else np.array(codes, np.uint8),
+            second_level=None if second is None else np.array(second, f32),
+            second_level_block=block, offset=offset)
+
+    def legacy(scales, **more):
+        return storage(SCALE_FLOAT32, fp32=scales, **more)
+
+    def nested(codes, second, block=32, offset=0.5, **more):
+        return storage(SCALE_DOUBLE_QUANTIZED_UINT8, codes=codes,
+                       second=second, block=block, offset=offset, **more)
+
+    many = list(range(70))
+    return [
+        ("legacy ok", legacy([0.0, 1.5, big]), 3),
+        ("legacy one", legacy([2.0]), 1),
+        ("legacy too few", legacy([1.0, 2.0]), 3),
+        ("legacy too many", legacy([1.0, 2.0, 3.0]), 2),
+        ("legacy with scale codes", legacy([1.0], codes=[128]), 1),
+        ("legacy with second level", legacy([1.0], second=[1.0]), 1),
+        ("legacy with block size", legacy([1.0], block=32), 1),
+        ("legacy with offset", legacy([1.0], offset=0.25), 1),
+        ("legacy negative zero offset", legacy([1.0], offset=-0.0), 1),
+        ("legacy negative", legacy([1.0, -1.0e-30]), 2),
+        ("legacy negative zero", legacy([1.0, -0.0]), 2),
+        ("legacy infinite", legacy([np.inf, 1.0]), 2),
+        ("legacy nan", legacy([1.0, np.nan]), 2),
+        ("legacy too few and negative", legacy([-1.0]), 2),
+        ("nested ok", nested([0, 128, 255], [1.0]), 3),
+        ("nested two groups", nested(many, [1.0, 2.0, 0.0]), 70),
+        ("nested block 64", nested(many, [1.0, 0.5], block=64), 70),
+        ("nested with fp32", nested([128], [1.0], fp32=[1.0]), 1),
+        ("nested too few codes", nested([128, 128], [1.0]), 3),
+        ("nested too many codes", nested([128, 128, 128], [1.0]), 2),
+        ("nested zero block", nested([128], [1.0], block=0), 1),
+        ("nested block 16", nested([128], [1.0], block=16), 1),
+        ("nested block 48", nested([128], [1.0], block=48), 1),
+        ("nested block 8192", nested([128], [1.0], block=8192), 1),
+        ("nested infinite offset", nested([128], [1.0], offset=np.inf), 1),
+        ("nested nan offset", nested([128], [1.0], offset=np.nan), 1),
+        ("nested negative offset", nested([128], [1.0], offset=-0.5), 1),
+        ("nested negative zero offset", nested([128], [1.0], offset=-0.0), 1),
+        ("nested too few groups", nested(many, [1.0, 2.0]), 70),
+        ("nested too many groups", nested(many, [1.0, 2.0, 3.0, 4.0]), 70),
+        ("nested no groups", nested([128], []), 1),
+        ("nested negative second level", nested([128], [-1.0]), 1),
+        ("nested infinite second level", nested([128], [np.inf]), 1),
+        ("nested nan second level", nested(many, [1.0, np.nan, 1.0]), 70),
+        ("nested saturating sum", nested([255], [big], offset=big), 1),
+        ("nested clamped below", nested([1], [big], offset=1.0), 1),
+        ("nested overflowing product",
+         nested([255, 1], [big], offset=0.0), 2),
+        ("nested bad block and bad count",
+         nested(many, [1.0], block=16), 70),
+        ("nested bad count and negative second level",
+         nested(many, [-1.0], block=32), 70),
+        ("unknown encoding", storage(2, fp32=[1.0]), 1),
+    ]
+
+
+def verdict(function, *arguments):
+    """("ok", "") or (exception type name, message) of one call."""
+    try:
+        function(*arguments)
+    except (ValueError, OverflowError, RuntimeError, TypeError) as error:
+        return [type(error).__name__, str(error)]
+    return ["ok", ""]

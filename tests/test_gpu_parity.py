@@ -542,8 +542,8 @@ def test_zero_scale_blocks_and_saturated_scales(gpu, package, library,
 # ---- full-size properties -----------------------------------------------
 
 @pytest.mark.parametrize("out_w,in_w,double_quantized", [
-    (11008, 4096, False), (11008, 4096, True), (4096, 4096, True),
-    (4096, 11008, True)])
+    (11008, 4096, False), (11008, 4096, True), (4096, 4096, False),
+    (4096, 4096, True), (4096, 11008, True)])
 def test_prefill_shapes_at_full_size(gpu, package, library, oracle, out_w,
                                      in_w, double_quantized):
     """M = 2048 at the Llama-7B layer shapes.  Size-independent checks: every output

@@ -136,3 +136,22 @@ def test_payload_bytes_match_the_published_figures(oracle, digests):
     assert llama["down_proj"]["fp32"]["payload_bytes"] == 25362432
     assert llama["q_proj"]["dq"]["payload_bytes"] == 8654852
     assert llama["gate_proj"]["dq"]["payload_bytes"] == 23259908
+
+
+def test_scale_storage_verdicts(oracle):
+    """The restated scale-storage check gives the verdicts the compiled
+    reference's dispatcher gave (tests/golden/scale_storage_verdicts.json,
+    written by make_golden.py)."""
+    with open(os.path.join(GOLDEN, "scale_storage_verdicts.json")) as handle:
+        expected = json.load(handle)
+    cases = helpers.scale_storage_cases()
+    assert sorted(expected) == sorted(name for name, _, _ in cases)
+    outcomes = set()
+    for name, weight, count in cases:
+        got = helpers.verdict(oracle.validate_scale_storage, weight, count)
+        assert got == expected[name], name
+        outcomes.add(got[1])
+    # "ok" and every message the check can give for finite arithmetic (a
+    # non-finite reconstruction needs a non-finite second-level scale or
+    # offset, and those are rejected first)
+    assert len(outcomes) == 6

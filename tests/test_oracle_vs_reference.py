@@ -92,6 +92,17 @@ def test_validation_agrees(oracle, reference):
         assert str(mine.value) == str(theirs.value)
 
 
+def test_scale_storage_verdicts_agree(oracle, reference):
+    """nf4o_validate_scale_storage against the reference dispatcher's own
+    check (dispatch.cpp:108-154), outcome, exception type and message."""
+    for name, weight, expected in helpers.scale_storage_cases():
+        mine = helpers.verdict(oracle.validate_scale_storage, weight,
+                               expected)
+        theirs = helpers.verdict(reference.validate_scale_storage, weight,
+                                 expected)
+        assert mine == theirs, name
+
+
 def test_memory_usage_known_answers(oracle, reference):
     # tests/core/test_quantization.cpp:188-198 and :368-376
     values = np.repeat(np.arange(33, dtype=np.float32), 32)
