@@ -41,7 +41,7 @@ extern "C" {
 #endif
 
 #define RTHIP_ABI_VERSION_MAJOR 1u
-#define RTHIP_ABI_VERSION_MINOR 3u
+#define RTHIP_ABI_VERSION_MINOR 4u
 
 typedef int32_t rthip_status;
 
@@ -345,6 +345,16 @@ rthip_status rthip_nf4_check_payload(
     const float* secondary_scales, int32_t encoding,
     uint64_t second_level_block, float offset, uint64_t element_count,
     uint64_t block_size, void* stream);
+
+/*
+ * Frees the scratch buffers the library keeps per (device, stream) for
+ * kernels that pass partial results between workgroups (64 MiB each,
+ * allocated by the first call on a stream that needs one): the buffer of
+ * `stream` on the current device, or of every stream when every_stream != 0.
+ * Waits for the device to finish with them; a later call allocates afresh.
+ * No counterpart in the reference (its backends allocate per call).
+ */
+rthip_status rthip_release_workspaces(void* stream, int32_t every_stream);
 
 #ifdef __cplusplus
 }

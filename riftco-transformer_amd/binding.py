@@ -108,6 +108,7 @@ _PROTOTYPES = {
         _i32, [_ptr] + _WEIGHT + [_ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
     "rthip_nf4_linear_input_backward": (
         _i32, [_ptr] + _WEIGHT + [_ptr, _u64, _u64, _u64, _u64, _ptr]),
+    "rthip_release_workspaces": (_i32, [_ptr, _i32]),
     "rthip_nf4_linear_forward_with": (
         _i32,
         [_i32, _ptr] + _WEIGHT + [_ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
@@ -355,6 +356,11 @@ class Library:
             status = self._lib.rthip_nf4_linear_input_backward_with(
                 algorithm, dy_ptr, *weight.abi_arguments(), *tail)
         self._check(status)
+
+    def release_workspaces(self, stream: int = 0,
+                           every_stream: bool = True) -> None:
+        self._check(self._lib.rthip_release_workspaces(
+            stream, 1 if every_stream else 0))
 
     def check_payload(self, weight: DeviceWeight,
                       element_count: Optional[int] = None,

@@ -426,11 +426,13 @@ hipError_t launch_dense_matmul(const float* left, const float* right,
             const std::size_t steps_per_slice = (steps + slices - 1) / slices;
             shape.slice = static_cast<unsigned>(steps_per_slice * kTileK);
             slices = (shared + shape.slice - 1) / shape.slice;
-            float* workspace = nullptr;
-            if (const hipError_t status = stream_workspace(stream, &workspace);
+            WorkspaceLease lease;  // held until both launches are enqueued
+            if (const hipError_t status =
+                    lease_stream_workspace(stream, &lease);
                 status != hipSuccess) {
                 return status;
             }
+            float* const workspace = lease.data();
             const dim3 grid(static_cast<unsigned>(tiles_n),
                             static_cast<unsigned>(tiles_m),
                             static_cast<unsigned>(slices));
@@ -449,12 +451,13 @@ hipError_t launch_dense_matmul(const float* left, const float* right,
                 plan, static_cast<unsigned>(tiles),
                 kTileM * kTileN * sizeof(float), kStreamWorkspaceBytes);
             if (groups != 0) {
-                float* workspace = nullptr;
+                WorkspaceLease lease;
                 if (const hipError_t status =
-                        stream_workspace(stream, &workspace);
+                        lease_stream_workspace(stream, &lease);
                     status != hipSuccess) {
                     return status;
                 }
+                float* const workspace = lease.data();
                 dense_matmul_planned_kernel<<<plan.whole_tiles + groups,
                                               kThreads, 0, stream>>>(
                     left, right, out, workspace, shape, plan);

@@ -10,6 +10,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <mutex>
 
 namespace rthip {
 
@@ -53,9 +54,31 @@ void launch_gemv_group(const LinearProblem* problems, std::size_t count,
                        hipStream_t stream);
 
 // workspace.hip -- scratch memory shared by the kernels that pass partial
-// results between workgroups; one fixed-size buffer per (device, stream).
+// results between workgroups; one fixed-size buffer per (device, stream),
+// followed by kStatusWords 64-bit words for verdicts that go back to the host.
 constexpr std::size_t kStreamWorkspaceBytes = std::size_t{64} << 20;
-hipError_t stream_workspace(hipStream_t stream, float** out);
+constexpr std::size_t kStatusWords = 8;
+// The buffer, and the exclusive right to enqueue launches that use it: hold
+// the lease until the call's last launch is enqueued (two threads that launch
+// on one stream must not interleave their partial-result and sum kernels).
+class WorkspaceLease {
+public:
+    float* data() const { return data_; }
+    // the status words behind the float area (reset them with a kernel)
+    std::uint64_t* status_words() const {
+        return reinterpret_cast<std::uint64_t*>(
+            reinterpret_cast<char*>(data_) + kStreamWorkspaceBytes);
+    }
+
+private:
+    friend hipError_t lease_stream_workspace(hipStream_t, WorkspaceLease*);
+    float* data_ = nullptr;
+    std::unique_lock<std::mutex> lock_;
+};
+hipError_t lease_stream_workspace(hipStream_t stream, WorkspaceLease* lease);
+// Frees the buffer of `stream` (or of every stream) on the current device,
+// after the device has finished with it.
+hipError_t release_stream_workspaces(hipStream_t stream, bool every_stream);
 
 // nf4_skinny.hip -- forward only, up to 64 rows, decode straight into MFMA
 // operands.  Shapes whose output tiles are shared between workgroups use a

@@ -517,13 +517,14 @@ hipError_t launch_encoding(const LinearProblem& p, const GemmShape& shape,
     const unsigned groups =
         plan_tiles(plan, tiles, kTileM * kTileN * sizeof(float),
                    kStreamWorkspaceBytes);
-    float* workspace = nullptr;
+    WorkspaceLease lease;  // held until both launches are enqueued
     if (groups != 0) {
-        if (const hipError_t status = stream_workspace(stream, &workspace);
+        if (const hipError_t status = lease_stream_workspace(stream, &lease);
             status != hipSuccess) {
             return status;
         }
     }
+    float* const workspace = lease.data();
     static const hipError_t configured = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kernel),
         hipFuncAttributeMaxDynamicSharedMemorySize,

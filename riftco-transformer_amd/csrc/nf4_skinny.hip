@@ -511,13 +511,14 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     split.quotient = units / groups;
     split.remainder = units % groups;
     const bool partial_tiles = groups != tiles;
-    float* workspace = nullptr;
+    WorkspaceLease lease;  // held until both launches are enqueued
     if (partial_tiles) {
-        const hipError_t status = stream_workspace(stream, &workspace);
+        const hipError_t status = lease_stream_workspace(stream, &lease);
         if (status != hipSuccess) {
             return status;
         }
     }
+    float* const workspace = lease.data();
     kernel<<<groups, kThreads, kSharedBytes, stream>>>(
         p.activations, p.weight, p.bias, p.result, workspace,
         static_cast<unsigned>(p.rows), static_cast<unsigned>(p.input_width),

@@ -362,11 +362,13 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     const BackwardSplit split = split_weight_rows(
         p.rows, p.input_width, p.output_width, kStreamWorkspaceBytes);
     float* target = p.result;
+    WorkspaceLease lease;  // held until both launches are enqueued
     if (split.chunks > 1) {
-        if (const hipError_t status = stream_workspace(stream, &target);
+        if (const hipError_t status = lease_stream_workspace(stream, &lease);
             status != hipSuccess) {
             return status;
         }
+        target = lease.data();
     }
     const auto kernel = small_backward_kernel<kBlocks, kDoubleQuantized>;
     // More than the default 64 KB of LDS (table + parking space).

@@ -275,6 +275,7 @@ bool backward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
 
 extern "C" {
 
+
 uint32_t rthip_abi_version(void) {
     return (RTHIP_ABI_VERSION_MAJOR << 16) | RTHIP_ABI_VERSION_MINOR;
 }
@@ -957,6 +958,16 @@ rthip_status rthip_nf4_linear_input_backward(
         output_width, block_size, stream);
 }
 
+rthip_status rthip_release_workspaces(void* stream, int32_t every_stream) {
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    return from_hip(
+        rthip::release_stream_workspaces(static_cast<hipStream_t>(stream),
+                                         every_stream != 0),
+        "workspace release");
+}
+
 rthip_status rthip_nf4_dequantize(
     const uint8_t* codes, const void* primary_scales,
     const float* secondary_scales, int32_t encoding,
@@ -1041,22 +1052,22 @@ rthip_status rthip_nf4_quantize(
         return status;
     }
     const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
-    // [0]: status bits, [1]: the offset (a float)
-    unsigned* words = nullptr;
+    // [0]: status bits, [1]: the offset (a float): the first status word of
+    // the stream workspace, cleared by a kernel (no allocation per call, and
+    // no memset node if the stream is being captured).
+    rthip::WorkspaceLease lease;
     if (const hipError_t error =
-            hipMalloc(reinterpret_cast<void**>(&words), 2 * sizeof(unsigned));
+            rthip::lease_stream_workspace(hip_stream, &lease);
         error != hipSuccess) {
-        return from_hip(error, "quantizer status allocation");
+        return from_hip(error, "quantizer workspace allocation");
     }
-    hipError_t error = hipMemsetAsync(words, 0, 2 * sizeof(unsigned),
-                                      hip_stream);
+    unsigned* const words = reinterpret_cast<unsigned*>(lease.status_words());
     unsigned host_words[2] = {0U, 0U};
-    if (error == hipSuccess) {
-        problem.status = words;
-        problem.offset = reinterpret_cast<float*>(words + 1);
-        rthip::launch_quantize(problem, hip_stream);
-        error = hipGetLastError();
-    }
+    rthip::launch_fill(reinterpret_cast<float*>(words), 0.0F, 2, hip_stream);
+    problem.status = words;
+    problem.offset = reinterpret_cast<float*>(words + 1);
+    rthip::launch_quantize(problem, hip_stream);
+    hipError_t error = hipGetLastError();
     if (error == hipSuccess) {
         error = hipMemcpyAsync(host_words, words, sizeof(host_words),
                                hipMemcpyDeviceToHost, hip_stream);
@@ -1064,12 +1075,8 @@ rthip_status rthip_nf4_quantize(
     if (error == hipSuccess) {
         error = hipStreamSynchronize(hip_stream);
     }
-    const hipError_t released = hipFree(words);
     if (error != hipSuccess) {
         return from_hip(error, "NF4 quantize");
-    }
-    if (released != hipSuccess) {
-        return from_hip(released, "quantizer status release");
     }
     if ((host_words[0] & 1U) != 0U) {
         return fail(RTHIP_INVALID_ARGUMENT,
@@ -1120,12 +1127,16 @@ rthip_status rthip_nf4_check_payload(
                              weight.second_level_shift;
     }
     const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
-    unsigned long long* words = nullptr;
-    if (const hipError_t error = hipMalloc(reinterpret_cast<void**>(&words),
-                                           3 * sizeof(unsigned long long));
+    // three status words of the stream workspace (initialised by the launch)
+    rthip::WorkspaceLease lease;
+    if (const hipError_t error =
+            rthip::lease_stream_workspace(hip_stream, &lease);
         error != hipSuccess) {
-        return from_hip(error, "payload check allocation");
+        return from_hip(error, "payload check workspace allocation");
     }
+    static_assert(sizeof(unsigned long long) == sizeof(std::uint64_t));
+    unsigned long long* const words =
+        reinterpret_cast<unsigned long long*>(lease.status_words());
     unsigned long long host_words[3] = {0, 0, 0};
     rthip::launch_check_payload(weight, element_count, block_shift,
                                 second_level_count, words, hip_stream);
@@ -1137,12 +1148,8 @@ rthip_status rthip_nf4_check_payload(
     if (error == hipSuccess) {
         error = hipStreamSynchronize(hip_stream);
     }
-    const hipError_t released = hipFree(words);
     if (error != hipSuccess) {
         return from_hip(error, "NF4 payload check");
-    }
-    if (released != hipSuccess) {
-        return from_hip(released, "payload check release");
     }
     // The reference's order: unused nibble, offset, second-level scales,
     // then the blocks.

@@ -242,6 +242,8 @@ rthip_status rthip_nf4_linear_input_backward(
     return RTHIP_OK;
 }
 
+rthip_status rthip_release_workspaces(void*, int32_t) { return RTHIP_OK; }
+
 rthip_status rthip_nf4_linear_forward_with(
     int32_t, const float* x, const uint8_t* codes, const void* primary_scales,
     const float* secondary_scales, int32_t encoding,
