@@ -41,7 +41,7 @@ extern "C" {
 #endif
 
 #define RTHIP_ABI_VERSION_MAJOR 1u
-#define RTHIP_ABI_VERSION_MINOR 4u
+#define RTHIP_ABI_VERSION_MINOR 5u
 
 typedef int32_t rthip_status;
 
@@ -355,6 +355,31 @@ rthip_status rthip_nf4_check_payload(
  * No counterpart in the reference (its backends allocate per call).
  */
 rthip_status rthip_release_workspaces(void* stream, int32_t every_stream);
+
+/*
+ * rthip_nf4_linear_input_backward for callers that cannot allocate: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  Same arguments and
+ * the same result, bit for bit, but it covers the small-batch family only
+ * (rows <= 64, input_width % 8 == 0, output_width % 4 == 0, aligned
+ * pointers; RTHIP_UNSUPPORTED otherwise) and keeps the partial sums of the
+ * weight-row chunks in a device array that is part of the library image
+ * (RTHIP_NO_ALLOC_SCRATCH_BYTES on every GPU the library runs on, held until
+ * the process ends) instead of the per-stream workspace.  A problem whose
+ * partial sums -- chunks x rows x input_width x 4 bytes, chunks <= 16 --
+ * exceed that size is refused with RTHIP_UNSUPPORTED and a message that
+ * names both sizes.  It calls no hipMalloc, hipFree or allocating library
+ * routine.  Every call on a GPU shares that GPU's array: calls that overlap
+ * on one GPU (two streams, or two graphs replayed at once) race; calls on
+ * one stream are ordered and safe.
+ */
+#define RTHIP_NO_ALLOC_SCRATCH_BYTES (24u << 20)
+rthip_status rthip_nf4_linear_input_backward_no_alloc(
+    const float* dy, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, float* dx, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream);
 
 #ifdef __cplusplus
 }

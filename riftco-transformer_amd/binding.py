@@ -108,6 +108,8 @@ _PROTOTYPES = {
         _i32, [_ptr] + _WEIGHT + [_ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
     "rthip_nf4_linear_input_backward": (
         _i32, [_ptr] + _WEIGHT + [_ptr, _u64, _u64, _u64, _u64, _ptr]),
+    "rthip_nf4_linear_input_backward_no_alloc": (
+        _i32, [_ptr] + _WEIGHT + [_ptr, _u64, _u64, _u64, _u64, _ptr]),
     "rthip_release_workspaces": (_i32, [_ptr, _i32]),
     "rthip_nf4_linear_forward_with": (
         _i32,
@@ -356,6 +358,16 @@ class Library:
             status = self._lib.rthip_nf4_linear_input_backward_with(
                 algorithm, dy_ptr, *weight.abi_arguments(), *tail)
         self._check(status)
+
+    def linear_input_backward_no_alloc(self, dy_ptr: int,
+                                       weight: DeviceWeight, dx_ptr: int,
+                                       rows: int, stream: int = 0) -> None:
+        """The small-batch input backward with its partial sums in the
+        library's own device array: nothing is allocated."""
+        self._check(self._lib.rthip_nf4_linear_input_backward_no_alloc(
+            dy_ptr, *weight.abi_arguments(), dx_ptr, rows,
+            weight.input_width, weight.output_width, weight.block_size,
+            stream))
 
     def release_workspaces(self, stream: int = 0,
                            every_stream: bool = True) -> None:

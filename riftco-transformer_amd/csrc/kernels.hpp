@@ -29,6 +29,11 @@ struct LinearProblem {
     // forward only: low-rank adapter term added in the epilogue
     // (lora.reduced == nullptr: none)
     LoraEpilogue lora{nullptr, nullptr, 0U, 0.0F};
+    // Memory for partial results that the caller brings (a launcher that
+    // needs more than scratch_bytes fails with hipErrorOutOfMemory); null:
+    // the launcher leases the stream workspace.
+    float* scratch = nullptr;
+    std::size_t scratch_bytes = 0;
 };
 
 // nf4_generic.hip
@@ -102,6 +107,8 @@ constexpr std::size_t kSmallBackwardMaxRows = 64;
 bool small_input_backward_supports(const LinearProblem& problem);
 hipError_t launch_small_input_backward(const LinearProblem& problem,
                                        hipStream_t stream);
+// Bytes of partial sums the launch above writes outside dx (0: none).
+std::size_t small_input_backward_scratch_bytes(const LinearProblem& problem);
 
 // lora.hip -- reduced[rows, rank] = x A^T, the input of the adapter epilogue.
 void launch_lora_reduce(const float* x, const float* a, float* reduced,

@@ -364,11 +364,23 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     float* target = p.result;
     WorkspaceLease lease;  // held until both launches are enqueued
     if (split.chunks > 1) {
-        if (const hipError_t status = lease_stream_workspace(stream, &lease);
-            status != hipSuccess) {
-            return status;
+        if (p.scratch != nullptr) {
+            // the caller's memory; the split is the one the stream
+            // workspace would get, so the sums are the same bit for bit
+            if (static_cast<std::size_t>(split.chunks) * p.rows *
+                    p.input_width * sizeof(float) >
+                p.scratch_bytes) {
+                return hipErrorOutOfMemory;
+            }
+            target = p.scratch;
+        } else {
+            if (const hipError_t status =
+                    lease_stream_workspace(stream, &lease);
+                status != hipSuccess) {
+                return status;
+            }
+            target = lease.data();
         }
-        target = lease.data();
     }
     const auto kernel = small_backward_kernel<kBlocks, kDoubleQuantized>;
     // More than the default 64 KB of LDS (table + parking space).
@@ -417,6 +429,15 @@ bool small_input_backward_supports(const LinearProblem& p) {
            reinterpret_cast<std::uintptr_t>(p.weight.codes) % 4 == 0 &&
            reinterpret_cast<std::uintptr_t>(p.activations) % 16 == 0 &&
            reinterpret_cast<std::uintptr_t>(p.result) % 4 == 0;
+}
+
+std::size_t small_input_backward_scratch_bytes(const LinearProblem& p) {
+    // the split never depends on who brings the memory
+    const BackwardSplit split = split_weight_rows(
+        p.rows, p.input_width, p.output_width, kStreamWorkspaceBytes);
+    return split.chunks > 1 ? static_cast<std::size_t>(split.chunks) *
+                                  p.rows * p.input_width * sizeof(float)
+                            : 0;
 }
 
 hipError_t launch_small_input_backward(const LinearProblem& p,

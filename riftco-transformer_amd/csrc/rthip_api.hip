@@ -271,9 +271,61 @@ bool backward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
            split->tail_family == RTHIP_NF4_ALGORITHM_SKINNY;
 }
 
+// ---- the entry point that allocates nothing ------------------------------
+//
+// Partial sums of the small-batch input backward, for callers that cannot
+// call hipMalloc.  Every GPU holds its own copy of this array at its own
+// address; host code never passes the array's name to a kernel or a copy
+// (that name is a host-side stand-in), only the address that
+// hipGetSymbolAddress gave for the current device.
+constexpr std::size_t kStaticScratchBytes = RTHIP_NO_ALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) float
+    scratch[kStaticScratchBytes / sizeof(float)];
+
+constexpr int kMaxScratchDevices = 64;
+
+// The device address of `scratch` on the current device (looked up once per
+// device, with that device current).
+rthip_status static_scratch(float** out) {
+    static std::mutex guard;
+    static float* address[kMaxScratchDevices] = {};
+    int device = 0;
+    if (const hipError_t error = hipGetDevice(&device); error != hipSuccess) {
+        return from_hip(error, "current device query");
+    }
+    if (device < 0 || device >= kMaxScratchDevices) {
+        return fail(RTHIP_UNSUPPORTED, "device ordinal %d is out of range",
+                    device);
+    }
+    const std::lock_guard<std::mutex> lock(guard);
+    if (address[device] == nullptr) {
+        float* found = nullptr;
+        if (const hipError_t error = hipGetSymbolAddress(
+                reinterpret_cast<void**>(&found), HIP_SYMBOL(scratch));
+            error != hipSuccess) {
+            return from_hip(error, "static scratch address lookup");
+        }
+        if (found == nullptr) {
+            return fail(RTHIP_RUNTIME_ERROR,
+                        "static scratch address lookup returned null");
+        }
+        address[device] = found;
+    }
+    *out = address[device];
+    return RTHIP_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+static rthip_status input_backward_common(
+    int32_t algorithm, const float* dy, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset, float* dx,
+    uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream, float* partial_sums,
+    std::size_t partial_sum_bytes);
 
 
 uint32_t rthip_abi_version(void) {
@@ -843,6 +895,23 @@ rthip_status rthip_nf4_linear_input_backward_with(
     uint64_t rows, uint64_t input_width, uint64_t output_width,
     uint64_t block_size, void* stream
 ) {
+    return input_backward_common(
+        algorithm, dy, codes, primary_scales, secondary_scales, encoding,
+        second_level_block, offset, dx, rows, input_width, output_width,
+        block_size, stream, nullptr, 0);
+}
+
+// One input backward.  partial_sums == nullptr: any family, partial results
+// in the stream workspace.  Otherwise: the small-batch family only, partial
+// results in that memory, nothing allocated.
+static rthip_status input_backward_common(
+    int32_t algorithm, const float* dy, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset, float* dx,
+    uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream, float* partial_sums,
+    std::size_t partial_sum_bytes
+) {
     if (dy == nullptr || dx == nullptr) {
         return fail(RTHIP_INVALID_ARGUMENT,
                     "upstream and input gradient must not be null");
@@ -874,7 +943,30 @@ rthip_status rthip_nf4_linear_input_backward_with(
     problem.rows = rows;
     problem.input_width = input_width;
     problem.output_width = output_width;
+    problem.scratch = partial_sums;
+    problem.scratch_bytes = partial_sum_bytes;
     const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+    if (partial_sums != nullptr) {
+        if (rows > rthip::kSmallBackwardMaxRows ||
+            !rthip::small_input_backward_supports(problem)) {
+            return fail(RTHIP_UNSUPPORTED,
+                        "the entry point that allocates nothing covers the "
+                        "small-batch input backward only: rows <= %zu, a row "
+                        "width that is a multiple of 8, an output width that "
+                        "is a multiple of 4 and aligned pointers",
+                        rthip::kSmallBackwardMaxRows);
+        }
+        const std::size_t needed =
+            rthip::small_input_backward_scratch_bytes(problem);
+        if (needed > partial_sum_bytes) {
+            return fail(RTHIP_UNSUPPORTED,
+                        "this input backward needs %zu bytes for partial "
+                        "sums; the entry point that allocates nothing has "
+                        "%zu",
+                        needed, partial_sum_bytes);
+        }
+        algorithm = RTHIP_NF4_ALGORITHM_SKINNY;
+    }
 
     const auto launch = [hip_stream](int32_t algorithm,
                                      const rthip::LinearProblem& problem)
@@ -956,6 +1048,28 @@ rthip_status rthip_nf4_linear_input_backward(
         RTHIP_NF4_ALGORITHM_AUTO, dy, codes, primary_scales, secondary_scales,
         encoding, second_level_block, offset, dx, rows, input_width,
         output_width, block_size, stream);
+}
+
+rthip_status rthip_nf4_linear_input_backward_no_alloc(
+    const float* dy, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, float* dx, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream
+) {
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    float* partial_sums = nullptr;
+    if (const rthip_status status = static_scratch(&partial_sums);
+        status != RTHIP_OK) {
+        return status;
+    }
+    return input_backward_common(
+        RTHIP_NF4_ALGORITHM_SKINNY, dy, codes, primary_scales,
+        secondary_scales, encoding, second_level_block, offset, dx, rows,
+        input_width, output_width, block_size, stream, partial_sums,
+        kStaticScratchBytes);
 }
 
 rthip_status rthip_release_workspaces(void* stream, int32_t every_stream) {

@@ -242,6 +242,21 @@ rthip_status rthip_nf4_linear_input_backward(
     return RTHIP_OK;
 }
 
+rthip_status rthip_nf4_linear_input_backward_no_alloc(
+    const float* dy, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, float* dx, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream) {
+    if (rows > 64) {
+        return fail(RTHIP_UNSUPPORTED, "more than 64 rows");
+    }
+    return rthip_nf4_linear_input_backward(
+        dy, codes, primary_scales, secondary_scales, encoding,
+        second_level_block, offset, dx, rows, input_width, output_width,
+        block_size, stream);
+}
+
 rthip_status rthip_release_workspaces(void*, int32_t) { return RTHIP_OK; }
 
 rthip_status rthip_nf4_linear_forward_with(
