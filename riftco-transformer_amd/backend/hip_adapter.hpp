@@ -87,11 +87,15 @@ struct HipForwardMergeStatistics {
 // validation that the dispatcher runs before every launch
 // (src/core/backend/nn/quantized_linear/dispatch.cpp:98-151) only has to run
 // once for storage that can never change.
+// (A reference tree whose dispatcher has been taught to consult it declares
+// the interface itself, beside QuantizedWeightStorage, and says so.)
+#ifndef RIFTCO_TRANSFORMER_HAS_SCALE_VALIDATION_MEMO
 class ScaleValidationMemo {
 public:
     virtual ~ScaleValidationMemo() = default;
     [[nodiscard]] virtual bool scales_validated() const noexcept = 0;
     virtual void mark_scales_validated() const noexcept = 0;
 };
+#endif
 
 }  // namespace riftco_transformer::backend_detail
