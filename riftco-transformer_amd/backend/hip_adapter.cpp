@@ -35,6 +35,7 @@
 #endif
 
 #include <array>
+#include <atomic>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
@@ -423,12 +424,19 @@ public:
 
     // A writable span: from here on the host copy may be newer than HBM.
     [[nodiscard]] std::span<float> data() noexcept override {
-        refresh_host();
+        launch_pending_forwards_or_abort();
+        const std::lock_guard<std::mutex> lock(sync_);
+        refresh_host_locked();
         freshest_ = Freshest::Host;
         return host_;
     }
+    // Readers may come from several threads at once (two forwards that share
+    // an input, a forward and a host read): the lazily synchronised state is
+    // guarded, and the span stays valid because the host copy is sized once.
     [[nodiscard]] std::span<const float> data() const noexcept override {
-        refresh_host();
+        launch_pending_forwards_or_abort();
+        const std::lock_guard<std::mutex> lock(sync_);
+        refresh_host_locked();
         return host_;
     }
 
@@ -449,6 +457,7 @@ public:
 
     // HBM pointer with the tensor's current contents.
     [[nodiscard]] const float* device_for_read() const {
+        const std::lock_guard<std::mutex> lock(sync_);
         if (freshest_ == Freshest::Host) {
             const HipRuntime& runtime = require_runtime();
             check(runtime,
@@ -462,6 +471,7 @@ public:
 
     // HBM pointer that a kernel is about to overwrite completely.
     [[nodiscard]] float* device_for_overwrite() noexcept {
+        const std::lock_guard<std::mutex> lock(sync_);
         freshest_ = Freshest::Device;
         return static_cast<float*>(device_.get());
     }
@@ -480,8 +490,9 @@ private:
 
     // noexcept by contract: a failing device read-back ends the process, as a
     // failing access to a managed CUDA allocation would.
-    void refresh_host() const noexcept {
-        launch_pending_forwards_or_abort();
+    // (sync_ held; queued forwards have been launched by the caller, outside
+    // the lock: launching them reads and writes other tensors' state)
+    void refresh_host_locked() const noexcept {
         if (freshest_ != Freshest::Device) {
             return;
         }
@@ -497,6 +508,7 @@ private:
 
     std::size_t count_;
     DeviceBuffer device_;
+    mutable std::mutex sync_;  // guards host_ and freshest_
     mutable std::vector<float> host_;
     mutable Freshest freshest_;
 };
@@ -627,10 +639,10 @@ public:
     }
 
     [[nodiscard]] bool scales_validated() const noexcept override {
-        return scales_validated_;
+        return scales_validated_.load(std::memory_order_acquire);
     }
     void mark_scales_validated() const noexcept override {
-        scales_validated_ = true;
+        scales_validated_.store(true, std::memory_order_release);
     }
 
     [[nodiscard]] Nf4ScaleEncoding encoding() const noexcept {
@@ -671,7 +683,7 @@ private:
     WeightArray<float> second_level_scales_;
     std::size_t second_level_block_size_;
     float offset_;
-    mutable bool scales_validated_ = false;
+    mutable std::atomic<bool> scales_validated_{false};
 };
 
 const HipTensorStorage& require_hip_tensor(const TensorStorage& storage,

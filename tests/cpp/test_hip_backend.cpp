@@ -379,8 +379,11 @@ void require_byte_preserving(const backend::QuantizedWeightStorage& storage,
     const auto scales = storage.scale_storage();
     const auto same_floats = [](std::span<const float> a,
                                 const std::vector<float>& b) {
+        // (memcmp must not see the null pointers of two empty arrays)
         return a.size() == b.size() &&
-               std::memcmp(a.data(), b.data(), b.size() * sizeof(float)) == 0;
+               (b.empty() ||
+                std::memcmp(a.data(), b.data(), b.size() * sizeof(float)) ==
+                    0);
     };
     require(same_floats(scales.fp32_scales, weight.scales.fp32_scales) &&
                 same_floats(scales.second_level_scales,

@@ -57,6 +57,75 @@ def test_adapter_options_on_the_host_only_runtime(options):
                     RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1", **options))
 
 
+SANITIZER_ENVIRONMENT = {
+    # the harness preloads a library of its own; ASan only insists on being
+    # first in the list, which has no bearing on what is checked here
+    "ASAN_OPTIONS": "verify_asan_link_order=0:detect_leaks=1:"
+                    "abort_on_error=0:exitcode=23",
+    "UBSAN_OPTIONS": "halt_on_error=1:print_stacktrace=1:exitcode=23",
+    "TSAN_OPTIONS": "halt_on_error=1:exitcode=23",
+}
+
+
+def run_sanitized(program, runtime, **environment):
+    binary = os.path.join(BUILD, program)
+    library = os.path.join(BUILD, runtime)
+    assert os.path.exists(binary) and os.path.exists(library), \
+        f"{program} is not built (make -C tests/cpp sanitize)"
+    env = {k: v for k, v in os.environ.items()
+           if not k.startswith(("RIFTCO_TRANSFORMER_", "FAKE_RTHIP_"))}
+    env.update(SANITIZER_ENVIRONMENT)
+    env["RIFTCO_TRANSFORMER_TEST_GOLDEN"] = os.path.join(HERE, "golden")
+    env["RIFTCO_TRANSFORMER_HIP_LIBRARY"] = library
+    env["RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP"] = "1"
+    env.update(environment)
+    return subprocess.run([binary], env=env, capture_output=True, text=True,
+                          timeout=600)
+
+
+@pytest.mark.parametrize("options", [
+    {"FAKE_RTHIP_CAN_FAIL": "1"},
+    {"RIFTCO_TRANSFORMER_HIP_POOL": "0"},
+    {"RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
+    {"RIFTCO_TRANSFORMER_HIP_MERGE": "1"},
+    {"FAKE_RTHIP_NO_BAR": "1"},
+])
+def test_adapter_under_address_and_undefined_behaviour_sanitizers(options):
+    """The whole host side -- adapter (buffer pool, held-back launches, the
+    lazily synchronised host copies, spans into device memory), run-time
+    binding, dispatcher, packed-state reader, and the test runtime -- built
+    with -fsanitize=address,undefined, as the reference's `sanitize` preset
+    builds its host code (cmake/RiftcoTransformerSanitizers.cmake)."""
+    result = run_sanitized(os.path.join("asan", "test_hip_backend"),
+                           os.path.join("asan", "librthip_fake.so"),
+                           **options)
+    assert result.returncode == 0, result.stdout + result.stderr[-4000:]
+    assert "hip backend tests passed" in result.stdout
+    assert "runtime error" not in result.stderr
+    assert "AddressSanitizer" not in result.stderr
+
+
+@pytest.mark.parametrize("options", [
+    {},
+    {"RIFTCO_TRANSFORMER_HIP_POOL": "0"},
+    {"RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
+    {"RIFTCO_TRANSFORMER_HIP_MERGE": "1"},
+])
+def test_adapter_from_four_threads_under_thread_sanitizer(options):
+    """tests/cpp/test_threads.cpp: four threads share a weight, an input and
+    the buffer pool; forward, input backward, host reads, storage release,
+    and tensors whose first download or upload happens under contention.
+    Every result equals the single-threaded one and ThreadSanitizer reports
+    nothing (the counterpart of the reference's thread test of backend
+    selection, tests/core/backend/test_backend.cpp:355-395)."""
+    result = run_sanitized(os.path.join("tsan", "test_threads"),
+                           os.path.join("tsan", "librthip_fake.so"),
+                           **options)
+    assert result.returncode == 0, result.stdout + result.stderr[-4000:]
+    assert "hip backend thread tests passed" in result.stdout
+    assert "ThreadSanitizer" not in result.stderr
+
+
 def test_adapter_keeps_a_counted_mirror_without_host_visible_memory():
     expect_pass(run(RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE,
                     RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1",

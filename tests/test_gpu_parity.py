@@ -479,6 +479,74 @@ def test_shared_output_tiles_are_added_in_a_fixed_order(gpu, package, library,
                 f"launch {launch}")
 
 
+def test_two_host_threads_launch_on_one_stream(gpu, package, library, oracle):
+    """Kernels that hand partial results to a second kernel through the
+    stream's scratch buffer (the small-batch forward and input backward, the
+    tiled kernel's leftover tiles) are launched from two host threads at once
+    on the same stream, each thread with its own input: a thread's sum kernel
+    must never read the other thread's partial results.  Every output equals,
+    bit for bit, the one the same call gives alone."""
+    import threading
+    import torch
+    stream = torch.cuda.current_stream().cuda_stream
+    cases = [  # (out_w, in_w, rows, direction)
+        (4096, 11008, 16, "forward"),     # small batch, partial tiles
+        (11008, 4096, 16, "backward"),    # row chunks
+        (1000, 4096 + 256, 40, "forward"),
+        (11008, 4096, 300, "forward"),    # tiled kernel, leftover tiles
+    ]
+    for out_w, in_w, rows, direction in cases:
+        weight = oracle.quantize(helpers.normal(95, (out_w, in_w), 0.02), 64,
+                                 False, 256)
+        device_weight = upload(gpu, weight)
+        width = in_w if direction == "forward" else out_w
+        other = out_w if direction == "forward" else in_w
+        inputs = [to_device(helpers.normal(96 + t, (rows, width), 1.0))
+                  for t in range(2)]
+
+        def call(source, target):
+            if direction == "forward":
+                library.linear_forward(source.data_ptr(), device_weight, None,
+                                       target.data_ptr(), rows, stream)
+            else:
+                library.linear_input_backward(source.data_ptr(),
+                                              device_weight,
+                                              target.data_ptr(), rows, stream)
+
+        expected = []
+        for source in inputs:
+            target = torch.empty(rows, other, device="cuda")
+            call(source, target)
+            expected.append(host(target))
+        outputs = [[torch.empty(rows, other, device="cuda")
+                    for _ in range(40)] for _ in range(2)]
+        start = threading.Barrier(2)
+        failures = []
+
+        def worker(index):
+            try:
+                start.wait()
+                for target in outputs[index]:
+                    call(inputs[index], target)
+            except Exception as error:  # noqa: BLE001
+                failures.append(error)
+
+        threads = [threading.Thread(target=worker, args=(t,))
+                   for t in range(2)]
+        for thread in threads:
+            thread.start()
+        for thread in threads:
+            thread.join()
+        assert not failures, failures
+        torch.cuda.synchronize()
+        for index in range(2):
+            for launch, target in enumerate(outputs[index]):
+                helpers.assert_bit_equal(
+                    host(target), expected[index],
+                    f"{direction} {out_w}x{in_w}, thread {index}, "
+                    f"launch {launch}")
+
+
 @pytest.mark.parametrize("rows,out_w,in_w,double_quantized", [
     (300, 1000, 1024, False),   # 24 tiles, each cut into four runs
     (130, 260, 1056, True),     # 6 tiles, runs of 8 and 9 steps
