@@ -25,14 +25,21 @@ The same JSON line carries
   large_launches
                 M = 1 launches of 74 and 101 MB (lm_head; four gate/up weights
                 in one grouped launch)
+  practical_roof
+                a plain streaming read of the same sizes, one launch per
+                buffer, and an empty launch: what the device gives a kernel
+                that only reads, beside the 8 TB/s of the data sheet
   small_batch_input_backward
                 the input backward at M in {1, 16, 64}, nested scales
   lora          the fused bias + rank-16 adapter forward beside the plain one
   matmul        dense fp32 matmul at layer and adapter shapes
   quantizer     the device quantizer on one 11008 x 4096 weight (wall clock,
                 the call returns after the work is done)
-  cpu_baseline  the reference CPU backend (oracle/_ref, else the C
-                restatement) timed on this host, single thread, on one layer
+  cpu_baseline  the reference CPU backend (kind "reference": oracle/_ref, built
+                in the build container from the reference's own sources and
+                shipped prebuilt; kind "port": the C restatement, where that
+                library is absent) timed on this host, single thread, on one
+                layer; host_cpu names the processor
 
 Packed payloads are synthetic: uniformly random nibbles (NF4 codes of normal
 weights are close to uniform by construction) and block scales drawn around
@@ -195,11 +202,8 @@ def bench_decode(package, device, torch, layers, steps, warmup, use_graph,
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": (GROUPED_KERNEL_HBM_BYTES if grouped
-                        else DOMINANT_KERNEL_HBM_BYTES),
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
-                              "scaled by a copy of known size "
-                              "(profiles/decode_gemv_hbm_traffic_pmc.txt)",
+            "traffic": profiled_traffic(grouped)[0],
+            "traffic_source": profiled_traffic(grouped)[1],
             "kernel": "gemv_forward_kernel<rows=1, K=4096%s>" % (
                 ", grouped" if grouped else ""),
             "bytes_per_launch": dominant_bytes / len(dominant),
@@ -208,15 +212,54 @@ def bench_decode(package, device, torch, layers, steps, warmup, use_graph,
     }
 
 
-# HBM bytes per launch of the dominant kernel (average over its 4:2 mix of
-# 4096x4096 and 11008x4096 weights), measured with rocprofv3 counters in runs
-# of their own -- a counter run cannot be nested inside this timing run:
-# FETCH_SIZE 7329.2 x 2.00 KiB (the factor a copy kernel of known size gives)
-# plus WRITE_SIZE 25.0 x 1.00 KiB.  Algorithmic bytes: 14 745 600.
-DOMINANT_KERNEL_HBM_BYTES = int((7329.2 * 2.00 + 25.0) * 1024)
-# The same for the grouped launches (q/k/v and gate/up, 1:1): FETCH_SIZE
-# 19424.1 x 2.00 KiB plus WRITE_SIZE 67.0 KiB.  Algorithmic: 39 518 208.
-GROUPED_KERNEL_HBM_BYTES = int((19424.1 * 2.00 + 67.0) * 1024)
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles",
+                               "decode_gemv_hbm_traffic_pmc.txt")
+
+
+def profiled_traffic(grouped):
+    """HBM bytes per launch of the dominant kernel as the tracked rocprofv3
+    counter summary has them (a counter run cannot be nested inside this
+    timing run): FETCH_SIZE and WRITE_SIZE averages of the K = 4096 GEMV
+    instantiation, each scaled by what the same counter read for torch's
+    2^28-element copy (2^20 KiB read, 2^20 KiB written).  Returns (bytes,
+    where it came from), or (None, why not) when the summary cannot be read
+    -- a kernel whose template arguments changed since it was profiled shows
+    up here as "no row", not as a stale figure."""
+    section = ("projections that share x in one launch" if grouped
+               else "one launch per projection")
+    grouped_flag = "true>" if grouped else "false>"
+    try:
+        with open(TRAFFIC_PROFILE) as handle:
+            text = handle.read()
+    except OSError as error:
+        return None, "no profile: %s" % error
+    if section not in text:
+        return None, "the profile has no section '%s'" % section
+    body = text[text.index(section):]
+    if not grouped and "projections that share x" in body:
+        body = body[:body.index("projections that share x")]
+    readings = {}
+    for line in body.splitlines():
+        fields = line.split()
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            if counter not in fields:
+                continue
+            average = float(fields[fields.index(counter) + 2])
+            if line.startswith("at::native::vectorized_elementwise_kernel"):
+                readings[counter, "copy"] = average
+            elif (line.startswith("rthip::gemv_forward_kernel<1, 1,") and
+                  line.split(">")[0].endswith(grouped_flag[:-1])):
+                readings[counter, "kernel"] = average
+    try:
+        kib = sum(readings[counter, "kernel"] * 2.0 ** 20 /
+                  readings[counter, "copy"]
+                  for counter in ("FETCH_SIZE", "WRITE_SIZE"))
+    except KeyError as missing:
+        return None, "the profile has no row for %s" % (missing.args[0],)
+    return int(kib * 1024), (
+        "profiles/decode_gemv_hbm_traffic_pmc.txt: rocprofv3 --pmc "
+        "FETCH_SIZE / WRITE_SIZE per dispatch, each scaled by its reading "
+        "for a copy of 2^30 B")
 
 
 def bench_gemm(package, device, torch, steps):
@@ -332,6 +375,48 @@ def bench_large_launches(package, device, torch, steps):
                          "frac": gbs / HBM_PEAK_GBS, "traffic": None},
         })
         del groups
+    return results
+
+
+def bench_practical_roof(package, torch, steps):
+    """What the device gives a kernel that only reads: one launch of a plain
+    streaming read (rthip_probe_streaming_read) per buffer, buffers rotating
+    through more than the last-level cache, replayed as a graph exactly like
+    the decode step; and an empty launch of the same grid.  The sizes are the
+    packed payloads of the decode shapes and of the large launches."""
+    library = package.load_library()
+    stream = lambda: torch.cuda.current_stream().cuda_stream
+    results = {"streaming_read": []}
+
+    def timed(body, launches):
+        body()
+        torch.cuda.synchronize()
+        replay = capture(torch, body)
+        replay()
+        return time_region(torch, replay, steps) / (steps * launches) * 1e3
+
+    copies = 24
+    results["empty_launch_us"] = timed(
+        lambda: [library.probe_empty_launch(stream()) for _ in range(copies)],
+        copies)
+    for label, size in (("4096x4096 payload", 9437184),
+                        ("11008x4096 payload", 25362432),
+                        ("32000x4096 payload", 73728000),
+                        ("256 MiB", 256 << 20)):
+        count = max(3, -(-(640 << 20) // size))  # >= 640 MB in rotation
+        buffers = [torch.empty(size, dtype=torch.uint8, device="cuda")
+                   for _ in range(count)]
+        for buffer in buffers:
+            buffer.random_(0, 256)
+        microseconds = timed(
+            lambda: [library.probe_streaming_read(b.data_ptr(), size,
+                                                  stream())
+                     for b in buffers], count)
+        results["streaming_read"].append({
+            "what": label, "bytes": size, "us": microseconds,
+            "gb_per_s": size / microseconds / 1e3,
+            "frac_of_peak": size / microseconds / 1e3 / HBM_PEAK_GBS})
+        del buffers
     return results
 
 
@@ -455,6 +540,17 @@ def bench_quantizer(package, device, torch):
     return results
 
 
+def host_cpu_model():
+    try:
+        with open("/proc/cpuinfo") as handle:
+            for line in handle:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(budget_seconds=12.0):
     """The reference CPU backend (oracle/_ref when built, else the C
     restatement) on this host, single thread: whole Llama-7B layers (7
@@ -505,7 +601,8 @@ def cpu_baseline(budget_seconds=12.0):
         }
     return {
         "value": total_bytes / seconds / 1e9, "unit": "GB/s", "cores": 1,
-        "kind": backend.kind, "seconds": seconds,
+        "kind": backend.kind, "host_cpu": host_cpu_model(),
+        "seconds": seconds,
         "sample": "%d passes over one Llama-7B layer (7 projections at M=1, "
                   "fp32 scales, %.1f MB packed per pass)"
                   % (passes, total_bytes / passes / 1e6),
@@ -641,6 +738,8 @@ def main():
                                                 max(3, arguments.steps // 4))
         line["large_launches"] = bench_large_launches(
             package, device, torch, max(3, arguments.steps // 2))
+        line["practical_roof"] = bench_practical_roof(
+            package, torch, max(3, arguments.steps // 2))
         line["small_batch_input_backward"] = bench_small_batch_backward(
             package, device, torch, max(3, arguments.steps // 4))
         line["lora"] = bench_lora(package, device, torch,
