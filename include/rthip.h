@@ -74,7 +74,10 @@ enum {
     RTHIP_NF4_ALGORITHM_AUTO = 0,
     /* one thread per output, per-element decode, any shape or block size */
     RTHIP_NF4_ALGORITHM_GENERIC = 1,
-    /* wavefront-reduced streaming GEMV for small row counts (HBM-bound) */
+    /* streaming kernels for decode-sized row counts (up to 4; HBM-bound):
+     * forward, a wavefront-reduced GEMV; input backward, the packed weight
+     * walked row by row as it lies in memory, a lane owning sixteen of its
+     * columns, products on the 4x4x1 matrix instruction */
     RTHIP_NF4_ALGORITHM_GEMV = 2,
     /* LDS-tiled fp32 MFMA GEMM with dequantisation fused into the tile load */
     RTHIP_NF4_ALGORITHM_MFMA = 3,

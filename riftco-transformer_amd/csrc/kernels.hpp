@@ -110,6 +110,15 @@ hipError_t launch_small_input_backward(const LinearProblem& problem,
 // Bytes of partial sums the launch above writes outside dx (0: none).
 std::size_t small_input_backward_scratch_bytes(const LinearProblem& problem);
 
+// nf4_stream_backward.hip -- input backward for up to four rows: the weight
+// is streamed as it lies in memory, a lane owning sixteen columns, the
+// products on the 4 x 4 x 1 matrix instruction.  Uses the stream workspace
+// when the weight rows are cut into ranges.
+constexpr std::size_t kStreamBackwardMaxRows = 4;
+bool stream_input_backward_supports(const LinearProblem& problem);
+hipError_t launch_stream_input_backward(const LinearProblem& problem,
+                                        hipStream_t stream);
+
 // lora.hip -- reduced[rows, rank] = x A^T, the input of the adapter epilogue.
 void launch_lora_reduce(const float* x, const float* a, float* reduced,
                         std::size_t rows, std::size_t input_width,

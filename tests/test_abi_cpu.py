@@ -70,7 +70,14 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(bwd, 2048, 11008, 4096, 64) == package.ALGORITHM_MFMA
     # up to 64 rows and a row width that is a multiple of 8 -> the backward
     # kernel that walks the weight as it lies in memory
-    assert select(bwd, 1, 4096, 11008, 64) == package.ALGORITHM_SKINNY
+    # decode-sized input backward: the weight streamed as it lies in memory
+    assert select(bwd, 1, 4096, 11008, 64) == package.ALGORITHM_GEMV
+    assert select(bwd, 4, 11008, 4096, 64) == package.ALGORITHM_GEMV
+    assert select(bwd, 2, 4096, 4096, 64) == package.ALGORITHM_GEMV
+    # (three and four rows of a small weight: the small-batch kernel)
+    assert select(bwd, 4, 4096, 4096, 64) == package.ALGORITHM_SKINNY
+    assert select(bwd, 4, 4096, 4096, 32) == package.ALGORITHM_SKINNY
+    assert select(bwd, 5, 4096, 11008, 64) == package.ALGORITHM_SKINNY
     assert select(bwd, 64, 11008, 4096, 64) == package.ALGORITHM_SKINNY
     assert select(bwd, 16, 40, 768, 32) == package.ALGORITHM_SKINNY
     # 65...96 rows: two launches of it, unless dx is much wider than dy

@@ -431,9 +431,12 @@ def test_small_batch_input_backward(gpu, package, library, oracle, out_w, in_w,
     weight = oracle.quantize(dense, block, double_quantized, second)
     device_weight = upload(gpu, weight)
     for rows in (1, 7, 16, 17, 40, 64):
+        # (up to four rows may belong to the streaming family instead; the
+        # small-batch kernel still runs them, pinned, in check_layer)
         assert library.select_algorithm(
-            package.INPUT_BACKWARD, rows, in_w, out_w,
-            block) == package.ALGORITHM_SKINNY
+            package.INPUT_BACKWARD, rows, in_w, out_w, block) in (
+                (package.ALGORITHM_SKINNY, package.ALGORITHM_GEMV)
+                if rows <= 4 else (package.ALGORITHM_SKINNY,))
         x = helpers.normal(84 + rows, (rows, in_w), 1.0)
         dy = helpers.normal(85 + rows, (rows, out_w), 1.0e-2)
         check_layer(gpu, package, library, oracle, weight, x, dy,
@@ -453,6 +456,56 @@ def test_small_batch_input_backward(gpu, package, library, oracle, out_w, in_w,
     x = helpers.normal(84 + rows, (rows, in_w), 1.0)
     dy = helpers.normal(85 + rows, (rows, out_w), 1.0e-2)
     check_layer(gpu, package, library, oracle, weight, x, dy, oracle_rows=2)
+
+
+@pytest.mark.parametrize("out_w,in_w,block,second,double_quantized", [
+    (4096, 4096, 64, 256, False),    # 4 column groups x 64 ranges of rows
+    (4096, 4096, 64, 256, True),
+    (4096, 11008, 64, 256, True),    # 11 column groups, the last one part empty
+    (11008, 4096, 64, 256, True),    # ranges that end inside a wavefront's turn
+    (11008, 4096, 64, 256, False),
+    (132, 1280, 128, 32, True),      # two groups, three ranges, 33 chunks
+    (1028, 8192, 4096, 32, False),   # blocks of 4096: 64 lanes share a scale
+    (8, 64, 64, 32, False),          # four lanes, two chunks
+    (4, 2048, 2048, 32, True),       # a single chunk
+])
+def test_streaming_input_backward(gpu, package, library, oracle, out_w, in_w,
+                                  block, second, double_quantized):
+    """One to four rows of dy against the packed weight streamed row by row,
+    products on the 4x4x1 matrix instruction: against the oracle, fp64 and the
+    other families, and repeated launches bit for bit (the ranges of weight
+    rows are added in ascending order)."""
+    dense = helpers.normal(183, (out_w, in_w), 0.02)
+    dense[out_w // 2] = 0.0
+    weight = oracle.quantize(dense, block, double_quantized, second)
+    device_weight = upload(gpu, weight)
+    for rows in (1, 2, 3, 4):
+        # (three and four rows of a small weight go to the small-batch kernel;
+        # check_layer still runs this family on them, pinned)
+        if rows <= 2 or out_w * in_w >= 1 << 25:
+            assert library.select_algorithm(
+                package.INPUT_BACKWARD, rows, in_w, out_w,
+                block) == package.ALGORITHM_GEMV
+        x = helpers.normal(184 + rows, (rows, in_w), 1.0)
+        dy = helpers.normal(185 + rows, (rows, out_w), 1.0e-2)
+        check_layer(gpu, package, library, oracle, weight, x, dy)
+        dy_device = to_device(dy)
+        first = host(gpu.linear_input_backward(
+            dy_device, device_weight, algorithm=package.ALGORITHM_GEMV))
+        for launch in range(3):
+            helpers.assert_bit_equal(
+                host(gpu.linear_input_backward(
+                    dy_device, device_weight,
+                    algorithm=package.ALGORITHM_GEMV)),
+                first, f"{rows} rows, launch {launch}")
+    # five rows, a block size of 32, a width that is no multiple of 16: not
+    # this family's
+    assert library.select_algorithm(
+        package.INPUT_BACKWARD, 5, in_w, out_w, block) != package.ALGORITHM_GEMV
+    assert library.select_algorithm(
+        package.INPUT_BACKWARD, 1, 4096, 4096, 32) != package.ALGORITHM_GEMV
+    assert library.select_algorithm(
+        package.INPUT_BACKWARD, 1, 4104, 4096, 64) != package.ALGORITHM_GEMV
 
 
 def test_shared_output_tiles_are_added_in_a_fixed_order(gpu, package, library,
@@ -1141,6 +1194,14 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
         # with its row chunks summed through the workspace
         outputs["small backward"] = gpu.linear_input_backward(
             upstream[:40].contiguous(), device_weight)
+        # up to four rows: the weight streamed row by row, the row ranges
+        # summed through the workspace, on the vector ALU (one row) and on the
+        # 4x4x1 matrix instruction (three)
+        for rows in (1, 3):
+            outputs[f"streaming backward, {rows}"] = \
+                gpu.linear_input_backward(
+                    upstream[:rows].contiguous(), device_weight,
+                    algorithm=package.ALGORITHM_GEMV)
         return outputs
 
     def refill(seed):
