@@ -625,6 +625,9 @@ def main():
     parser.add_argument("--small-batch-only", action="store_true",
                         help="run only the launches of up to 64 rows, "
                              "forward and input backward (for counter runs)")
+    parser.add_argument("--practical-roof-only", action="store_true",
+                        help="run only the streaming-read and empty-launch "
+                             "probes (for rocprofv3 kernel traces)")
     parser.add_argument("--traffic-calibration", action="store_true",
                         help="for rocprofv3 --pmc runs: a 1 GiB elementwise "
                              "copy of known traffic, then one decode step "
@@ -647,6 +650,11 @@ def main():
     library = package.load_library()
     if not torch.cuda.is_available() or not library.is_available():
         sys.exit("bench.py: no usable MI355X: " + library.last_error())
+
+    if arguments.practical_roof_only:
+        print(json.dumps({"practical_roof": bench_practical_roof(
+            package, torch, arguments.steps)}))
+        return
 
     if arguments.traffic_calibration:
         # torch's elementwise kernel reads 2^30 B and writes 2^30 B per call:

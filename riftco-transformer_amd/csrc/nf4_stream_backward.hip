@@ -383,7 +383,6 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
                        static_cast<unsigned>(p.input_width),
                        static_cast<unsigned>(p.output_width), p.block_shift,
                        plan);
-#ifndef LAB_NO_SUM
     if (plan.row_ranges > 1) {
         const unsigned elements =
             static_cast<unsigned>(p.rows * p.input_width);
@@ -392,18 +391,13 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
                                      kSumElements * kSumSlices, 0, stream>>>(
             target, p.result, elements, plan.row_ranges);
     }
-#endif
     return hipSuccess;
 }
 
 template <bool kDoubleQuantized>
 hipError_t launch_encoding(const LinearProblem& p, hipStream_t stream) {
-#ifdef LAB_ALWAYS_MATRIX
-    return launch_instance<kDoubleQuantized, true>(p, stream);
-#else
     return p.rows == 1 ? launch_instance<kDoubleQuantized, false>(p, stream)
                        : launch_instance<kDoubleQuantized, true>(p, stream);
-#endif
 }
 
 }  // namespace

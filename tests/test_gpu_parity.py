@@ -1012,11 +1012,15 @@ def test_abi_rejects_bad_arguments(gpu, package, library, oracle):
                                device_weight.primary_scales, None)
     with pytest.raises(package.InvalidArgument):
         library.linear_forward(x.data_ptr(), bad, None, y.data_ptr(), 1)
-    with pytest.raises(package.Unsupported):
-        library.linear_input_backward(x.data_ptr(), device_weight,
+    odd = oracle.quantize(helpers.normal(96, (3, 33), 0.02), 32)
+    with pytest.raises(package.Unsupported):       # blocks of 32, 33 columns
+        library.linear_input_backward(x.data_ptr(), upload(gpu, odd),
                                       y.data_ptr(), 1,
                                       algorithm=package.ALGORITHM_GEMV)
-    odd = oracle.quantize(helpers.normal(96, (3, 33), 0.02), 32)
+    with pytest.raises(package.Unsupported):       # five rows of dy
+        library.linear_input_backward(x.data_ptr(), device_weight,
+                                      y.data_ptr(), 5,
+                                      algorithm=package.ALGORITHM_GEMV)
     with pytest.raises(package.Unsupported):
         library.linear_forward(x.data_ptr(), upload(gpu, odd), None,
                                y.data_ptr(), 1,
