@@ -154,6 +154,10 @@ class Oracle:
         lib.nf4o_lora_linear_forward.restype = None
         lib.nf4o_lora_linear_forward.argtypes = [
             vp, vp, sp, vp, vp, vp, sz, ctypes.c_float, vp, sz, sz, sz, sz]
+        lib.nf4o_lora_linear_backward.restype = None
+        lib.nf4o_lora_linear_backward.argtypes = [
+            vp, vp, vp, sp, vp, vp, sz, ctypes.c_float, vp, vp, vp, sz, sz,
+            sz, sz]
         lib.nf4o_validate_payload.restype = i32
         lib.nf4o_validate_payload.argtypes = [
             sz, sz, vp, sz, sp, ctypes.POINTER(ctypes.c_char_p)]
@@ -284,6 +288,24 @@ class Oracle:
             weight.input_width, weight.output_width, weight.block_size)
         return out
 
+    def lora_backward(self, dy, x, weight: Nf4Weight, lora_a, lora_b,
+                      lora_scale: float):
+        """(dx, dA, dB) of a Linear with a packed weight and an adapter."""
+        x = _f32(x).reshape(-1, weight.input_width)
+        dy = _f32(dy).reshape(-1, weight.output_width)
+        lora_a, lora_b = _f32(lora_a), _f32(lora_b)
+        dx = np.empty_like(x)
+        d_a = np.empty_like(lora_a)
+        d_b = np.empty_like(lora_b)
+        view = _scales_struct(weight)
+        self._lib.nf4o_lora_linear_backward(
+            dy.ctypes.data, x.ctypes.data, weight.codes.ctypes.data,
+            ctypes.byref(view), lora_a.ctypes.data, lora_b.ctypes.data,
+            lora_a.shape[0], lora_scale, dx.ctypes.data, d_a.ctypes.data,
+            d_b.ctypes.data, x.shape[0], weight.input_width,
+            weight.output_width, weight.block_size)
+        return dx, d_a, d_b
+
     # -- validation ------------------------------------------------------
     def validate_payload(self, weight: Nf4Weight) -> None:
         view = _scales_struct(weight)
@@ -345,6 +367,10 @@ class Reference:
         lib.nf4ref_validate_scale_storage.restype = i32
         lib.nf4ref_validate_scale_storage.argtypes = [
             i32, vp, sz, vp, sz, vp, sz, sz, f32, sz]
+        lib.nf4ref_lora_linear_backward.restype = i32
+        lib.nf4ref_lora_linear_backward.argtypes = [
+            vp, sz, sz, vp, vp, vp, vp, vp, sz, f32, sz, sz, sz, vp, vp, vp,
+            vp]
         lib.nf4ref_lora_linear_forward.restype = i32
         lib.nf4ref_lora_linear_forward.argtypes = [
             vp, vp, vp, vp, sz, f32, vp, sz, sz, sz, sz] + payload
@@ -459,6 +485,30 @@ class Reference:
             weight.output_width, weight.block_size,
             *self._payload_args(weight)))
         return out
+
+    def lora_linear_step(self, dense_weight, block_size: int,
+                         scale_block_size: int, x, dy, lora_a, lora_b,
+                         alpha: float, bias=None):
+        """Forward and backward through a real Linear of the reference that
+        packs `dense_weight` itself and carries an adapter with the given A
+        and B: returns (y, dx, dA, dB).  scale_block_size 0: fp32 scales."""
+        dense_weight = _f32(dense_weight)
+        output_width, input_width = dense_weight.shape
+        x = _f32(x).reshape(-1, input_width)
+        dy = _f32(dy).reshape(-1, output_width)
+        lora_a, lora_b = _f32(lora_a), _f32(lora_b)
+        bias = None if bias is None else _f32(bias)
+        y = np.empty((x.shape[0], output_width), dtype=np.float32)
+        dx = np.empty_like(x)
+        d_a = np.empty_like(lora_a)
+        d_b = np.empty_like(lora_b)
+        self._check(self._lib.nf4ref_lora_linear_backward(
+            dense_weight.ctypes.data, block_size, scale_block_size,
+            _ptr(bias), x.ctypes.data, dy.ctypes.data, lora_a.ctypes.data,
+            lora_b.ctypes.data, lora_a.shape[0], alpha, x.shape[0],
+            input_width, output_width, y.ctypes.data, dx.ctypes.data,
+            d_a.ctypes.data, d_b.ctypes.data))
+        return y, dx, d_a, d_b
 
     def memory_usage(self, weight: Nf4Weight) -> dict:
         out = np.zeros(9, dtype=np.uintp)

@@ -389,6 +389,67 @@ void nf4o_lora_linear_forward(const float* x, const uint8_t* codes,
     free(expanded);
 }
 
+void nf4o_lora_linear_backward(const float* dy, const float* x,
+                               const uint8_t* codes, const nf4o_scales* scales,
+                               const float* lora_a, const float* lora_b,
+                               size_t rank, float lora_scale, float* dx,
+                               float* d_lora_a, float* d_lora_b, size_t rows,
+                               size_t input_width, size_t output_width,
+                               size_t block_size) {
+    float* reduced = (float*)malloc(sizeof(float) * rows * rank);
+    float* scaled = (float*)malloc(sizeof(float) * rows * output_width);
+    float* d_reduced = (float*)malloc(sizeof(float) * rows * rank);
+    float* adapter_dx = (float*)malloc(sizeof(float) * rows * input_width);
+    size_t index;
+    size_t row;
+    size_t column;
+    size_t slot;
+    /* forward value the second matmul's closure keeps: x . A^T */
+    nf4o_matmul_nt(x, lora_a, reduced, rows, input_width, rank);
+    /* operator*(value, scalar): upstream times the constant, elementwise */
+    for (index = 0; index < rows * output_width; ++index) {
+        scaled[index] = dy[index] * lora_scale;
+    }
+    /* matmul(reduced, B^T): left gets upstream . (B^T)^T = scaled . B */
+    nf4o_matmul(scaled, lora_b, d_reduced, rows, output_width, rank);
+    /* ... right gets reduced^T . upstream, [rank, output]; transpose_2d
+     * hands its transpose to B */
+    for (column = 0; column < output_width; ++column) {
+        for (slot = 0; slot < rank; ++slot) {
+            float total = 0.0F;
+            for (row = 0; row < rows; ++row) {
+                total += reduced[row * rank + slot] *
+                         scaled[row * output_width + column];
+            }
+            d_lora_b[column * rank + slot] = 0.0F + total;
+        }
+    }
+    /* matmul(x, A^T): left gets d_reduced . A, right x^T . d_reduced,
+     * [input, rank], whose transpose goes to A */
+    nf4o_matmul(d_reduced, lora_a, adapter_dx, rows, rank, input_width);
+    for (slot = 0; slot < rank; ++slot) {
+        for (column = 0; column < input_width; ++column) {
+            float total = 0.0F;
+            for (row = 0; row < rows; ++row) {
+                total += x[row * input_width + column] *
+                         d_reduced[row * rank + slot];
+            }
+            d_lora_a[slot * input_width + column] = 0.0F + total;
+        }
+    }
+    /* quantized_linear's closure, then one rounded addition per element as
+     * the two contributions meet at x */
+    nf4o_linear_input_backward(dy, codes, scales, dx, rows, input_width,
+                               output_width, block_size);
+    for (index = 0; index < rows * input_width; ++index) {
+        dx[index] = (0.0F + dx[index]) + adapter_dx[index];
+    }
+    free(reduced);
+    free(scaled);
+    free(d_reduced);
+    free(adapter_dx);
+}
+
 size_t nf4o_scale_payload_bytes(const nf4o_scales* scales) {
     if (scales->encoding == NF4O_SCALE_FLOAT32) {
         return scales->fp32_count * sizeof(float);

@@ -26,6 +26,10 @@
  *       damaged scale storages (committed as golden verdicts)
  *   matmul, matmul_nt, add_bias, lora_linear_forward - bit-for-bit agreement
  *       with the compiled reference's tensor operations
+ *   lora_linear_backward                            - bit-for-bit agreement
+ *       with the gradients the compiled reference's autograd leaves on x and
+ *       on the adapter's parameters of a real Linear (packed weight, adapter
+ *       attached), committed as golden vectors
  * No function here is "parity unpinned".
  */
 #ifndef NF4_ORACLE_H
@@ -170,6 +174,28 @@ void nf4o_lora_linear_forward(const float* x, const uint8_t* codes,
                               size_t rank, float lora_scale, float* y,
                               size_t rows, size_t input_width,
                               size_t output_width, size_t block_size);
+
+/* The backward pass the reference's autograd runs through that Linear when
+ * the base weight is packed (frozen) and the adapter trains: the closures of
+ * src/core/autograd/operations.cpp recorded by LowRankAdapter::forward
+ * (src/nn/low_rank_adapter.cpp:126-151) and quantized_linear
+ * (src/nn/quantized_linear.cpp:60-80), met by Variable::accumulate_gradient
+ * (src/core/autograd/graph.cpp:218-242):
+ *   scaled    = dy * lora_scale                     operator* (:176-194)
+ *   d_reduced = matmul(scaled, B)                   matmul    (:252-277)
+ *   dB        = transpose(matmul(reduced^T, scaled))  with reduced = x.A^T
+ *   dA        = transpose(matmul(x^T, d_reduced))   transpose_2d (:480-492)
+ *   dx        = dy.deq(W) + matmul(d_reduced, A)
+ * every product summed in ascending order of the contracted index in fp32,
+ * every step rounded on its own.  x and dy are the values of one call
+ * (gradients start from zero, as after zero_gradient). */
+void nf4o_lora_linear_backward(const float* dy, const float* x,
+                               const uint8_t* codes, const nf4o_scales* scales,
+                               const float* lora_a, const float* lora_b,
+                               size_t rank, float lora_scale, float* dx,
+                               float* d_lora_a, float* d_lora_b, size_t rows,
+                               size_t input_width, size_t output_width,
+                               size_t block_size);
 
 /* require_canonical_payload, src/core/quantization/quantized_weight.cpp:102-174.
  * Returns NF4O_OK or the status of the exception the reference throws;

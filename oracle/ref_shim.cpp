@@ -16,6 +16,9 @@
 //       include/riftco_transformer/core/tensor_ops.hpp:12-36
 //   require_scale_storage, reached through dispatch_quantized_linear_forward
 //       src/core/backend/nn/quantized_linear/dispatch.cpp:98-154,203-242
+//   Linear (packed weight, attach_lora, forward) and Variable::backward
+//       include/riftco_transformer/nn/linear.hpp:16-60,
+//       include/riftco_transformer/core/autograd.hpp:31-50
 
 #include "core/backend/adapter.hpp"
 #include "core/backend/nn/quantized_linear/dispatch.hpp"
@@ -23,6 +26,7 @@
 #include "riftco_transformer/core/quantized_weight.hpp"
 #include "riftco_transformer/core/tensor.hpp"
 #include "riftco_transformer/core/tensor_ops.hpp"
+#include "riftco_transformer/nn/linear.hpp"
 
 #include <algorithm>
 #include <cstddef>
@@ -30,6 +34,7 @@
 #include <cstring>
 #include <exception>
 #include <optional>
+#include <random>
 #include <stdexcept>
 #include <string>
 #include <utility>
@@ -349,6 +354,89 @@ int nf4ref_validate_scale_storage(
             {backend::tensor_storage(source), *weight,
              backend::tensor_storage(target),
              backend::QuantizedLinearDimensions{1, input_width, 1, 32}});
+    });
+}
+
+// One training step's gradients through a real Linear of the reference: the
+// dense weight is packed by the Linear itself (quantize_weight_nf4 or its
+// double-quantised form), an adapter is attached and given the caller's A and
+// B, forward(x) builds the autograd graph and backward(dy) runs it.  What
+// comes back is what the reference leaves on x and on the adapter's two
+// parameters, plus the forward value.  scale_block_size == 0: fp32 scales.
+int nf4ref_lora_linear_backward(
+    const float* dense_weight, std::size_t block_size,
+    std::size_t scale_block_size, const float* bias_or_null, const float* x,
+    const float* dy, const float* lora_a, const float* lora_b,
+    std::size_t rank, float alpha, std::size_t rows, std::size_t input_width,
+    std::size_t output_width, float* y, float* dx, float* d_lora_a,
+    float* d_lora_b
+) {
+    using riftco_transformer::Linear;
+    using riftco_transformer::Variable;
+    return guarded([&] {
+        Tensor weight({output_width, input_width},
+                      std::vector<float>(
+                          dense_weight,
+                          dense_weight + output_width * input_width),
+                      ExecutionBackend::Cpu);
+        std::optional<Linear> linear;
+        if (bias_or_null != nullptr) {
+            linear.emplace(std::move(weight),
+                           Tensor({output_width},
+                                  std::vector<float>(
+                                      bias_or_null,
+                                      bias_or_null + output_width),
+                                  ExecutionBackend::Cpu));
+        } else {
+            linear.emplace(std::move(weight));
+        }
+        if (scale_block_size == 0) {
+            linear->quantize_weight_nf4(block_size);
+        } else {
+            linear->quantize_weight_nf4_double_quantized(block_size,
+                                                         scale_block_size);
+        }
+        std::mt19937 random(0);
+        linear->attach_lora(rank, alpha, random);
+        riftco_transformer::Parameter* a = nullptr;
+        riftco_transformer::Parameter* b = nullptr;
+        const auto adapter_parameters = linear->lora_parameters();
+        for (const auto& named : adapter_parameters) {
+            if (named.name == "lora_a.weight") {
+                a = named.parameter;
+            } else if (named.name == "lora_b.weight") {
+                b = named.parameter;
+            }
+        }
+        if (a == nullptr || b == nullptr) {
+            throw std::runtime_error("adapter parameters not found");
+        }
+        a->set_value(Tensor({rank, input_width},
+                            std::vector<float>(lora_a,
+                                               lora_a + rank * input_width),
+                            ExecutionBackend::Cpu));
+        b->set_value(Tensor({output_width, rank},
+                            std::vector<float>(lora_b,
+                                               lora_b + output_width * rank),
+                            ExecutionBackend::Cpu));
+        const Variable input(
+            Tensor({rows, input_width},
+                   std::vector<float>(x, x + rows * input_width),
+                   ExecutionBackend::Cpu),
+            true);
+        const Variable output = linear->forward(input);
+        output.backward(
+            Tensor({rows, output_width},
+                   std::vector<float>(dy, dy + rows * output_width),
+                   ExecutionBackend::Cpu));
+        const auto copy = [](const Tensor& tensor, float* target) {
+            const auto data = tensor.data();
+            std::copy(data.begin(), data.end(), target);
+        };
+        copy(output.value(), y);
+        copy(input.gradient(), dx);
+        copy(a->gradient(), d_lora_a);
+        copy(b->gradient(), d_lora_b);
     });
 }
 

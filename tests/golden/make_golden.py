@@ -185,6 +185,29 @@ def scale_storage_verdicts(reference):
         json.dump(verdicts, out, indent=1, sort_keys=True)
 
 
+def lora_steps(reference) -> dict:
+    """Forward value and the gradients on x, A and B that the reference's
+    autograd leaves after one backward pass through a real Linear (packed
+    weight, adapter attached) for each of helpers.LORA_STEP_CASES."""
+    arrays = {}
+    for name in helpers.LORA_STEP_CASES:
+        case = helpers.lora_step_inputs(name)
+        y, dx, d_a, d_b = reference.lora_linear_step(
+            case["dense"], case["block"], case["second"], case["x"],
+            case["dy"], case["lora_a"], case["lora_b"], case["alpha"],
+            bias=case["bias"])
+        arrays[f"{name}_y"] = y
+        arrays[f"{name}_dx"] = dx
+        arrays[f"{name}_d_lora_a"] = d_a
+        arrays[f"{name}_d_lora_b"] = d_b
+        arrays[f"{name}_inputs_sha256"] = np.frombuffer(
+            helpers.sha256(np.concatenate(
+                [case[key].ravel() for key in
+                 ("dense", "x", "dy", "lora_a", "lora_b")])).encode(),
+            dtype=np.uint8)
+    return arrays
+
+
 def bits_of(array):
     return np.ascontiguousarray(array, dtype=np.float32).view(np.uint32)
 
@@ -193,6 +216,8 @@ def main():
     reference = Reference()
     packed_state(reference)
     scale_storage_verdicts(reference)
+    np.savez_compressed(os.path.join(HERE, "lora_steps.npz"),
+                        **lora_steps(reference))
     np.savez_compressed(os.path.join(HERE, "closed_form.npz"),
                         **closed_form(reference))
     arrays, meta1 = config1(reference)

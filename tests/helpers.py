@@ -272,3 +272,34 @@ def verdict(function, *arguments):
     except (ValueError, OverflowError, RuntimeError, TypeError) as error:
         return [type(error).__name__, str(error)]
     return ["ok", ""]
+
+
+# ---- one training step through a Linear with a packed weight and an adapter --
+
+# name: (rows, input_width, output_width, rank, alpha, block size, second-level
+#        block size or 0 for fp32 scales, with bias)
+LORA_STEP_CASES = {
+    "rank3_fp32": (5, 128, 24, 3, 8.0, 64, 0, False),
+    "rank4_nested_bias": (3, 256, 40, 4, 16.0, 32, 32, True),
+    "one_row_rank1": (1, 64, 8, 1, 2.0, 64, 0, True),
+    "odd_widths_nested": (7, 192, 33, 5, 8.0, 64, 256, False),
+    "rank16": (9, 512, 48, 16, 32.0, 64, 0, False),
+}
+
+
+def lora_step_inputs(name: str) -> dict:
+    """Seeded inputs of LORA_STEP_CASES[name]."""
+    rows, in_w, out_w, rank, alpha, block, second, with_bias = \
+        LORA_STEP_CASES[name]
+    seed = 500 + 10 * sorted(LORA_STEP_CASES).index(name)
+    return {
+        "dense": normal(seed, (out_w, in_w), 0.02),
+        "x": normal(seed + 1, (rows, in_w), 1.0),
+        "dy": normal(seed + 2, (rows, out_w), 1.0e-2),
+        "lora_a": normal(seed + 3, (rank, in_w), 0.05),
+        "lora_b": normal(seed + 4, (out_w, rank), 0.05),
+        "bias": normal(seed + 5, (out_w,), 0.01) if with_bias else None,
+        "alpha": alpha, "rank": rank, "block": block, "second": second,
+        # LowRankAdapter's scale: alpha / float(rank), one rounded division
+        "scale": float(np.float32(alpha) / np.float32(rank)),
+    }

@@ -31,8 +31,8 @@ What it does, in a scratch directory outside this repository:
    (hip_adapter.cpp with -DRIFTCO_TRANSFORMER_IN_TREE, hip_runtime.cpp,
    packed_state.cpp) with g++ and links them with the objects of the
    unedited reference sources that oracle/Makefile already built
-   (oracle/_ref/obj) plus the reference's autograd sources, which
-   test_backend.cpp needs;
+   (oracle/_ref/obj: tensor, quantization, backend, autograd and the few
+   nn/ files of a Linear);
 4. leaves the test programs (the accelerator test twice: as it is, and with
    the RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP gate on) in tests/in_tree/build/ (git-ignored; they
    travel to the GPU box, where tests/test_in_tree.py runs them against the
@@ -61,13 +61,6 @@ BUILD = os.path.join(HERE, "build")
 EDITED_SOURCES = [
     "src/core/backend/registry.cpp",
     "src/core/backend/nn/quantized_linear/dispatch.cpp",
-]
-# ... and those test_backend.cpp needs beyond what oracle/Makefile builds.
-EXTRA_SOURCES = [
-    "src/core/autograd/checkpoint.cpp",
-    "src/core/autograd/custom_gradient.cpp",
-    "src/core/autograd/graph.cpp",
-    "src/core/autograd/operations.cpp",
 ]
 # program -> (source, extra compiler flags)
 TESTS = {
@@ -234,7 +227,7 @@ def build(tree):
                 "-I" + os.path.join(tree, "src")]
     objects = os.path.join(tree, "obj")
     jobs = []
-    for source in EDITED_SOURCES + EXTRA_SOURCES:
+    for source in EDITED_SOURCES:
         jobs.append((os.path.join(tree, source),
                      os.path.join(objects, source + ".o"), includes))
     for name in ("hip_adapter.cpp", "hip_runtime.cpp", "packed_state.cpp"):

@@ -155,3 +155,27 @@ def test_scale_storage_verdicts(oracle):
     # non-finite reconstruction needs a non-finite second-level scale or
     # offset, and those are rejected first)
     assert len(outcomes) == 6
+
+
+@pytest.mark.parametrize("name", sorted(helpers.LORA_STEP_CASES))
+def test_lora_steps(oracle, name):
+    """Forward value and gradients of a Linear with a packed weight and an
+    adapter, as the compiled reference's autograd produced them."""
+    golden = np.load(os.path.join(GOLDEN, "lora_steps.npz"))
+    case = helpers.lora_step_inputs(name)
+    digest = helpers.sha256(np.concatenate(
+        [case[key].ravel() for key in
+         ("dense", "x", "dy", "lora_a", "lora_b")]))
+    assert digest == bytes(golden[f"{name}_inputs_sha256"]).decode()
+    weight = oracle.quantize(case["dense"], case["block"],
+                             case["second"] != 0, case["second"] or 256)
+    helpers.assert_bit_equal(
+        oracle.lora_forward(case["x"], weight, case["lora_a"],
+                            case["lora_b"], case["scale"], case["bias"]),
+        golden[f"{name}_y"])
+    dx, d_a, d_b = oracle.lora_backward(
+        case["dy"], case["x"], weight, case["lora_a"], case["lora_b"],
+        case["scale"])
+    helpers.assert_bit_equal(dx, golden[f"{name}_dx"], "dx")
+    helpers.assert_bit_equal(d_a, golden[f"{name}_d_lora_a"], "dA")
+    helpers.assert_bit_equal(d_b, golden[f"{name}_d_lora_b"], "dB")

@@ -4,6 +4,7 @@ restates (paths under /root/reference)."""
 import numpy as np
 import pytest
 
+import helpers
 from oracle.binding import (SCALE_DOUBLE_QUANTIZED_UINT8, SCALE_FLOAT32,
                             Nf4Weight)
 
@@ -173,6 +174,59 @@ def test_lora_composes_its_scaled_low_rank_delta(oracle):
     bias = np.array([14.5, 4.5], dtype=np.float32)
     y = oracle.lora_forward(x, weight, lora_a, lora_b, 4.0 / 2.0, bias)
     assert y.tolist() == [[24.5, 14.5]]
+
+
+def test_lora_backward_of_that_fixture_by_hand(oracle):
+    """The same adapter (tests/nn/test_lora.cpp:208-244) with the upstream
+    gradient of that test, [1, -0.5]: scaled upstream [2, -1]; through B,
+    d(reduced) = [2*1 + (-1)(-1), 2*2 + (-1)*3] = [3, 1]; reduced = x A^T =
+    [1, 2]; so dB = outer([2, -1], [1, 2]), dA = outer([3, 1], x), and with an
+    all-zero base weight dx = [3, 1] A = [3, 1, 0, ...]."""
+    weight = oracle.quantize(np.zeros((2, 32), dtype=np.float32), 32)
+    x = np.zeros((1, 32), dtype=np.float32)
+    x[0, :3] = [1.0, 2.0, 3.0]
+    lora_a = np.zeros((2, 32), dtype=np.float32)
+    lora_a[0, 0] = 1.0
+    lora_a[1, 1] = 1.0
+    lora_b = np.array([[1.0, 2.0], [-1.0, 3.0]], dtype=np.float32)
+    dy = np.array([[1.0, -0.5]], dtype=np.float32)
+    dx, d_a, d_b = oracle.lora_backward(dy, x, weight, lora_a, lora_b, 2.0)
+    assert d_b.tolist() == [[2.0, 4.0], [-1.0, -2.0]]
+    want_a = np.zeros((2, 32), dtype=np.float32)
+    want_a[0, :3] = [3.0, 6.0, 9.0]
+    want_a[1, :3] = [1.0, 2.0, 3.0]
+    assert np.array_equal(d_a, want_a)
+    want_x = np.zeros((1, 32), dtype=np.float32)
+    want_x[0, :2] = [3.0, 1.0]
+    assert np.array_equal(dx, want_x)
+
+
+@pytest.mark.parametrize("double_quantized", [False, True])
+def test_lora_backward_against_float64(oracle, double_quantized):
+    """dx, dA, dB as fp64 matrix products of the loss's differential:
+    y = x deq(W)^T + s (x A^T) B^T, so dx = dy deq(W) + s (dy B) A,
+    dA = s (dy B)^T x, dB = s dy^T (x A^T).  A swapped operand, a dropped
+    scale or a missing base term moves the result by its full size."""
+    rows, in_w, out_w, rank, scale = 6, 256, 40, 4, 2.5
+    weight = oracle.quantize(helpers.normal(71, (out_w, in_w), 0.02), 64,
+                             double_quantized, 32)
+    x = helpers.normal(72, (rows, in_w), 1.0)
+    dy = helpers.normal(73, (rows, out_w), 1.0)
+    lora_a = helpers.normal(74, (rank, in_w), 0.05)
+    lora_b = helpers.normal(75, (out_w, rank), 0.05)
+    dx, d_a, d_b = oracle.lora_backward(dy, x, weight, lora_a, lora_b, scale)
+    dense = oracle.dequantize(weight).astype(np.float64)
+    x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+    a64, b64 = lora_a.astype(np.float64), lora_b.astype(np.float64)
+    through_b = scale * (dy64 @ b64)
+    assert np.allclose(dx, dy64 @ dense + through_b @ a64,
+                       rtol=1e-4, atol=1e-5)
+    assert np.allclose(d_a, through_b.T @ x64, rtol=1e-4, atol=1e-5)
+    assert np.allclose(d_b, scale * dy64.T @ (x64 @ a64.T),
+                       rtol=1e-4, atol=1e-5)
+    # and each term is there at its full size
+    assert np.abs(through_b @ a64).max() > 1e-2
+    assert np.abs(dy64 @ dense).max() > 1e-2
 
 
 def test_matmul_small_integer_case(oracle):

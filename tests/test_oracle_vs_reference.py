@@ -147,3 +147,25 @@ def test_lora_linear_forward_bitwise(oracle, reference, shape, block, rank,
     helpers.assert_bit_equal(
         oracle.lora_forward(x, weight, lora_a, lora_b, 16.0 / rank, bias),
         reference.lora_forward(x, weight, lora_a, lora_b, 16.0 / rank, bias))
+
+
+@pytest.mark.parametrize("name", sorted(helpers.LORA_STEP_CASES))
+def test_lora_linear_step_bitwise(oracle, reference, name):
+    """The restated adapter backward against the gradients the reference's
+    autograd leaves on x, A and B of a real Linear that packed the weight
+    itself (quantize_weight_nf4[_double_quantized], attach_lora, forward,
+    backward)."""
+    case = helpers.lora_step_inputs(name)
+    y, dx, d_a, d_b = reference.lora_linear_step(
+        case["dense"], case["block"], case["second"], case["x"], case["dy"],
+        case["lora_a"], case["lora_b"], case["alpha"], bias=case["bias"])
+    weight = oracle.quantize(case["dense"], case["block"],
+                             case["second"] != 0, case["second"] or 256)
+    helpers.assert_bit_equal(
+        oracle.lora_forward(case["x"], weight, case["lora_a"],
+                            case["lora_b"], case["scale"], case["bias"]), y)
+    ours = oracle.lora_backward(case["dy"], case["x"], weight, case["lora_a"],
+                                case["lora_b"], case["scale"])
+    helpers.assert_bit_equal(ours[0], dx, "dx")
+    helpers.assert_bit_equal(ours[1], d_a, "dA")
+    helpers.assert_bit_equal(ours[2], d_b, "dB")
