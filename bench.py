@@ -31,7 +31,9 @@ The same JSON line carries
                 that only reads, beside the 8 TB/s of the data sheet
   small_batch_input_backward
                 the input backward at M in {1, 16, 64}, nested scales
-  lora          the fused bias + rank-16 adapter forward beside the plain one
+  lora          the fused bias + rank-16 adapter forward beside the plain one,
+                and the backward pass with the adapter (d_reduced, dA, dB and
+                the adapter's share of dx) beside the plain input backward
   matmul        dense fp32 matmul at layer and adapter shapes
   quantizer     the device quantizer on one 11008 x 4096 weight (wall clock,
                 the call returns after the work is done)
@@ -451,7 +453,9 @@ def bench_small_batch_backward(package, device, torch, steps):
 
 def bench_lora(package, device, torch, steps):
     """The fused bias + low-rank adapter forward (rank 16) beside the plain
-    forward on the same weights: what the adapter costs per call."""
+    forward on the same weights, and the same for the backward pass (dx with
+    the adapter's share in its epilogue, plus d_reduced, dA and dB): what the
+    adapter costs per call."""
     results = []
     rank = 16
     for name, out_w, in_w in (LAYER_SHAPES[0], LAYER_SHAPES[4]):
@@ -477,8 +481,46 @@ def bench_lora(package, device, torch, steps):
                         source, weight, lora_a, lora_b, 1.0, bias=bias,
                         out=target, reduced=reduced)
 
+            # the backward pass of the same layer: the packed product alone,
+            # the adapter's own gradients (d_reduced, dA, dB), and both with
+            # the adapter's share of dx in the epilogue
+            upstream = torch.randn(rows, out_w, device="cuda") * 1.0e-2
+            gradient = torch.empty(rows, in_w, device="cuda")
+            d_reduced = torch.empty(rows, rank, device="cuda")
+            d_a = torch.empty_like(lora_a)
+            d_b = torch.empty_like(lora_b)
+            library = package.load_library()
+            stream = lambda: torch.cuda.current_stream().cuda_stream
+
+            def adapter_gradients():
+                library.lora_backward(
+                    upstream.data_ptr(), source.data_ptr(),
+                    reduced.data_ptr(), lora_b.data_ptr(), rank, 1.0,
+                    d_reduced.data_ptr(), d_a.data_ptr(), d_b.data_ptr(),
+                    rows, in_w, out_w, stream())
+
+            def plain_backward():
+                for weight in used:
+                    device.linear_input_backward(upstream, weight,
+                                                 out=gradient)
+
+            def gradients_only():
+                for weight in used:
+                    adapter_gradients()
+
+            def fused_backward():
+                for weight in used:
+                    adapter_gradients()
+                    library.lora_linear_input_backward(
+                        upstream.data_ptr(), weight, lora_a.data_ptr(),
+                        d_reduced.data_ptr(), rank, gradient.data_ptr(), rows,
+                        stream())
+
             timings = {}
-            for label, body in (("plain", plain), ("fused", fused)):
+            for label, body in (("plain", plain), ("fused", fused),
+                                ("plain_backward", plain_backward),
+                                ("gradients_only", gradients_only),
+                                ("fused_backward", fused_backward)):
                 body()
                 torch.cuda.synchronize()
                 body = capture(torch, body)
@@ -488,6 +530,9 @@ def bench_lora(package, device, torch, steps):
             results.append({
                 "shape": name, "rows": rows, "rank": rank,
                 "plain_us": timings["plain"], "with_adapter_us": timings["fused"],
+                "input_backward_us": timings["plain_backward"],
+                "adapter_gradients_us": timings["gradients_only"],
+                "backward_with_adapter_us": timings["fused_backward"],
             })
         del weights
     return results
@@ -625,6 +670,9 @@ def main():
     parser.add_argument("--small-batch-only", action="store_true",
                         help="run only the launches of up to 64 rows, "
                              "forward and input backward (for counter runs)")
+    parser.add_argument("--adapter-only", action="store_true",
+                        help="run only the low-rank adapter section, forward "
+                             "and backward (for rocprofv3 kernel traces)")
     parser.add_argument("--practical-roof-only", action="store_true",
                         help="run only the streaming-read and empty-launch "
                              "probes (for rocprofv3 kernel traces)")
@@ -669,6 +717,11 @@ def main():
         print(json.dumps({"traffic_calibration": "done",
                           "copy_bytes_read": 2 ** 30,
                           "copy_bytes_written": 2 ** 30}))
+        return
+
+    if arguments.adapter_only:
+        print(json.dumps({"lora": bench_lora(package, device, torch,
+                                             arguments.steps)}))
         return
 
     if arguments.gemm_only:

@@ -41,7 +41,7 @@ extern "C" {
 #endif
 
 #define RTHIP_ABI_VERSION_MAJOR 1u
-#define RTHIP_ABI_VERSION_MINOR 6u
+#define RTHIP_ABI_VERSION_MINOR 7u
 
 typedef int32_t rthip_status;
 
@@ -255,6 +255,55 @@ rthip_status rthip_lora_reduce(const float* x, const float* lora_a,
                                uint64_t input_width, uint64_t lora_rank,
                                void* stream);
 
+/*
+ * The adapter's gradients for one upstream gradient dy [rows, output_width]:
+ *
+ *   d_reduced = (dy * lora_scale) . B                 [rows, lora_rank]
+ *   d_lora_b  = (dy * lora_scale)^T . reduced         [output_width, lora_rank]
+ *   d_lora_a  = d_reduced^T . x                       [lora_rank, input_width]
+ *
+ * What the reference's autograd computes for LowRankAdapter::forward
+ * (src/nn/low_rank_adapter.cpp:126-151) through the closures of operator*,
+ * matmul and transpose_2d (src/core/autograd/operations.cpp:176-194,252-277,
+ * 480-492): five dense matmuls over materialised transposes plus an
+ * elementwise multiply there, three launches here (d_reduced, then the two
+ * outer products; dy and x are each read once per product, dy * lora_scale is
+ * rounded per element and never stored).  `reduced` is x.A^T as the forward
+ * left it in its caller-provided buffer.  The gradients are written, not
+ * added to what the buffers hold (the reference starts every backward pass
+ * from zeroed gradients, src/core/autograd/graph.cpp:218-242).  d_lora_a
+ * and/or d_lora_b may be NULL: that product is skipped (x and reduced may
+ * then be NULL as well).  d_reduced is always written; the fused input
+ * backward below consumes it.
+ */
+rthip_status rthip_lora_backward(
+    const float* dy, const float* x, const float* reduced,
+    const float* lora_b, uint64_t lora_rank, float lora_scale,
+    float* d_reduced, float* d_lora_a, float* d_lora_b, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, void* stream);
+
+/*
+ * dx = dy.deq(W) + d_reduced.A
+ *
+ * The gradient that reaches the input of a Linear with a packed weight and an
+ * adapter: quantized_linear's closure (src/nn/quantized_linear.cpp:60-80)
+ * and the left-operand closure of the adapter's first matmul
+ * (src/core/autograd/operations.cpp:252-277), which the reference adds with
+ * one rounded addition per element where both arrive at x
+ * (Variable::accumulate_gradient, src/core/autograd/graph.cpp:218-242).
+ * Here the rank-sized sum is the epilogue of the packed-weight input
+ * backward: one pass over dx instead of a dense matmul, a temporary and an
+ * add.  lora_a is [lora_rank, input_width], d_reduced [rows, lora_rank] from
+ * rthip_lora_backward on the same stream.
+ */
+rthip_status rthip_nf4_lora_linear_input_backward(
+    const float* dy, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, const float* lora_a,
+    const float* d_reduced, uint64_t lora_rank, float* dx, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream);
+
 /* The same two operations with the kernel family pinned (tests, measurement).
  * RTHIP_UNSUPPORTED when `algorithm` cannot handle the shape. */
 rthip_status rthip_nf4_linear_forward_with(
@@ -277,6 +326,14 @@ rthip_status rthip_nf4_linear_input_backward_with(
     const void* primary_scales, const float* secondary_scales,
     int32_t encoding, uint64_t second_level_block, float offset, float* dx,
     uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream);
+
+rthip_status rthip_nf4_lora_linear_input_backward_with(
+    int32_t algorithm, const float* dy, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset,
+    const float* lora_a, const float* d_reduced, uint64_t lora_rank,
+    float* dx, uint64_t rows, uint64_t input_width, uint64_t output_width,
     uint64_t block_size, void* stream);
 
 /* Which family AUTO selects for a shape: direction 0 = forward, 1 = input

@@ -132,6 +132,15 @@ _PROTOTYPES = {
         _i32,
         [_i32, _ptr] + _WEIGHT + [_ptr, _ptr, _ptr, _u64, _f32, _ptr, _ptr,
                                   _u64, _u64, _u64, _u64, _ptr]),
+    "rthip_lora_backward": (
+        _i32, [_ptr, _ptr, _ptr, _ptr, _u64, _f32, _ptr, _ptr, _ptr, _u64,
+               _u64, _u64, _ptr]),
+    "rthip_nf4_lora_linear_input_backward": (
+        _i32, [_ptr] + _WEIGHT + [_ptr, _ptr, _u64, _ptr, _u64, _u64, _u64,
+                                  _u64, _ptr]),
+    "rthip_nf4_lora_linear_input_backward_with": (
+        _i32, [_i32, _ptr] + _WEIGHT + [_ptr, _ptr, _u64, _ptr, _u64, _u64,
+                                        _u64, _u64, _ptr]),
     "rthip_nf4_select_algorithm": (
         _i32, [_i32, _u64, _u64, _u64, _u64, ctypes.POINTER(_i32)]),
     "rthip_nf4_dequantize": (_i32, _WEIGHT + [_ptr, _u64, _u64, _ptr]),
@@ -346,6 +355,37 @@ class Library:
         else:
             status = self._lib.rthip_nf4_lora_linear_forward_with(
                 algorithm, x_ptr, *weight.abi_arguments(), *tail)
+        self._check(status)
+
+    def lora_backward(self, dy_ptr: int, x_ptr: Optional[int],
+                      reduced_ptr: Optional[int], lora_b_ptr: int, rank: int,
+                      lora_scale: float, d_reduced_ptr: int,
+                      d_lora_a_ptr: Optional[int],
+                      d_lora_b_ptr: Optional[int], rows: int,
+                      input_width: int, output_width: int,
+                      stream: int = 0) -> None:
+        """rthip_lora_backward: d_reduced, and dA / dB where a buffer is
+        given."""
+        self._check(self._lib.rthip_lora_backward(
+            dy_ptr, x_ptr, reduced_ptr, lora_b_ptr, rank, lora_scale,
+            d_reduced_ptr, d_lora_a_ptr, d_lora_b_ptr, rows, input_width,
+            output_width, stream))
+
+    def lora_linear_input_backward(self, dy_ptr: int, weight: DeviceWeight,
+                                   lora_a_ptr: int, d_reduced_ptr: int,
+                                   rank: int, dx_ptr: int, rows: int,
+                                   stream: int = 0,
+                                   algorithm: Optional[int] = None) -> None:
+        """dx = dy . deq(W) + d_reduced . A."""
+        tail = [lora_a_ptr, d_reduced_ptr, rank, dx_ptr, rows,
+                weight.input_width, weight.output_width, weight.block_size,
+                stream]
+        if algorithm is None:
+            status = self._lib.rthip_nf4_lora_linear_input_backward(
+                dy_ptr, *weight.abi_arguments(), *tail)
+        else:
+            status = self._lib.rthip_nf4_lora_linear_input_backward_with(
+                algorithm, dy_ptr, *weight.abi_arguments(), *tail)
         self._check(status)
 
     def linear_input_backward(self, dy_ptr: int, weight: DeviceWeight,

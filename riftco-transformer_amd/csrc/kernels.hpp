@@ -26,8 +26,8 @@ struct LinearProblem {
     std::size_t input_width;
     std::size_t output_width;
     unsigned block_shift;  // log2(block_size)
-    // forward only: low-rank adapter term added in the epilogue
-    // (lora.reduced == nullptr: none)
+    // low-rank adapter term added in the epilogue (lora.reduced == nullptr:
+    // none); forward: reduced . B^T, input backward: d_reduced . A
     LoraEpilogue lora{nullptr, nullptr, 0U, 0.0F};
     // Memory for partial results that the caller brings (a launcher that
     // needs more than scratch_bytes fails with hipErrorOutOfMemory); null:
@@ -118,6 +118,26 @@ constexpr std::size_t kStreamBackwardMaxRows = 4;
 bool stream_input_backward_supports(const LinearProblem& problem);
 hipError_t launch_stream_input_backward(const LinearProblem& problem,
                                         hipStream_t stream);
+
+// lora_backward.hip -- the adapter's gradients: d_reduced = (dy * scale) . B
+// (always), dB = ((dy * scale)^T . reduced) when d_b is not null and
+// dA = (d_reduced^T . x) when d_a is not null.
+struct LoraBackwardProblem {
+    const float* upstream;     // dy [rows, output_width]
+    const float* activations;  // x [rows, input_width] (dA only)
+    const float* reduced;      // x . A^T [rows, rank] (dB only)
+    const float* b;            // [output_width, rank]
+    float* d_reduced;          // [rows, rank]
+    float* d_a;                // [rank, input_width] or null
+    float* d_b;                // [output_width, rank] or null
+    std::size_t rows;
+    std::size_t input_width;
+    std::size_t output_width;
+    std::size_t rank;
+    float scale;
+};
+hipError_t launch_lora_backward(const LoraBackwardProblem& problem,
+                                hipStream_t stream);
 
 // lora.hip -- reduced[rows, rank] = x A^T, the input of the adapter epilogue.
 void launch_lora_reduce(const float* x, const float* a, float* reduced,

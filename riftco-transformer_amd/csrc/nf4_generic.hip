@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void generic_forward_kernel(
 __global__ __launch_bounds__(256) void generic_input_backward_kernel(
     const float* __restrict__ dy, Nf4WeightView weight,
     float* __restrict__ dx, std::size_t rows, std::size_t input_width,
-    std::size_t output_width, unsigned block_shift
+    std::size_t output_width, unsigned block_shift, LoraEpilogue lora
 ) {
     const std::size_t stride =
         static_cast<std::size_t>(gridDim.x) * blockDim.x;
@@ -107,7 +107,10 @@ __global__ __launch_bounds__(256) void generic_input_backward_kernel(
         const float total =
             ((partial[0] + partial[1]) + (partial[2] + partial[3])) +
             ((partial[4] + partial[5]) + (partial[6] + partial[7]));
-        dx[index] = total;
+        dx[index] = lora.reduced == nullptr
+                        ? total
+                        : total + lora_term(lora, static_cast<unsigned>(row),
+                                            static_cast<unsigned>(column));
     }
 }
 
@@ -167,7 +170,7 @@ void launch_generic_input_backward(const LinearProblem& p,
     generic_input_backward_kernel<<<grid_for(gradients, 256), 256, 0,
                                     stream>>>(
         p.activations, p.weight, p.result, p.rows, p.input_width,
-        p.output_width, p.block_shift);
+        p.output_width, p.block_shift, p.lora);
 }
 
 void launch_dequantize(const Nf4WeightView& weight, float* out,

@@ -391,7 +391,7 @@ __device__ __forceinline__ void gemm_segment(
             for (int e = 0; e < 16; ++e) {
                 term[e] = 0.0F;
             }
-            if constexpr (!kBackward) {
+            {
                 if (lora.reduced != nullptr) {  // uniform
                     const float* reduced_rows[16];
 #pragma unroll
@@ -406,8 +406,10 @@ __device__ __forceinline__ void gemm_segment(
                     }
                     lora_terms<16>(
                         term,
-                        lora.b + static_cast<std::size_t>(column) * lora.rank,
-                        reduced_rows, lora.rank, lora.scale);
+                        lora.b + static_cast<std::size_t>(column) *
+                                     lora.row_stride,
+                        reduced_rows, lora.rank, lora.scale,
+                        lora.rank_stride);
                 }
             }
 #pragma unroll

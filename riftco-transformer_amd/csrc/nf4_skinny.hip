@@ -270,8 +270,10 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
                         }
                         lora_terms<4>(
                             term,
-                            lora.b + static_cast<std::size_t>(n) * lora.rank,
-                            reduced_rows, lora.rank, lora.scale);
+                            lora.b + static_cast<std::size_t>(n) *
+                                         lora.row_stride,
+                            reduced_rows, lora.rank, lora.scale,
+                            lora.rank_stride);
                     }
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {

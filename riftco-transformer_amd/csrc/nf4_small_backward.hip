@@ -333,7 +333,8 @@ __global__ __launch_bounds__(kThreads) void small_backward_kernel(
 // count would wait for them one after the other).
 __global__ __launch_bounds__(256) void small_backward_sum_kernel(
     const float* __restrict__ partial, float* __restrict__ dx,
-    unsigned elements, unsigned chunks
+    unsigned elements, unsigned chunks, unsigned input_width,
+    LoraEpilogue lora
 ) {
     const unsigned element = blockIdx.x * blockDim.x + threadIdx.x;
     if (element >= elements) {
@@ -354,6 +355,9 @@ __global__ __launch_bounds__(256) void small_backward_sum_kernel(
             sum += parts[chunk];
         }
     }
+    if (lora.reduced != nullptr) {  // uniform
+        sum += lora_term(lora, element / input_width, element % input_width);
+    }
     dx[element] = sum;
 }
 
@@ -363,7 +367,10 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
         p.rows, p.input_width, p.output_width, kStreamWorkspaceBytes);
     float* target = p.result;
     WorkspaceLease lease;  // held until both launches are enqueued
-    if (split.chunks > 1) {
+    // (an adapter term is added by the second kernel, which then runs for
+    // a single chunk too)
+    const bool two_kernels = split.chunks > 1 || p.lora.reduced != nullptr;
+    if (two_kernels) {
         if (p.scratch != nullptr) {
             // the caller's memory; the split is the one the stream
             // workspace would get, so the sums are the same bit for bit
@@ -395,11 +402,12 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
         p.activations, p.weight, target, static_cast<unsigned>(p.rows),
         static_cast<unsigned>(p.input_width),
         static_cast<unsigned>(p.output_width), p.block_shift, split);
-    if (split.chunks > 1) {
+    if (two_kernels) {
         const unsigned elements =
             static_cast<unsigned>(p.rows * p.input_width);
         small_backward_sum_kernel<<<(elements + 255) / 256, 256, 0, stream>>>(
-            target, p.result, elements, split.chunks);
+            target, p.result, elements, split.chunks,
+            static_cast<unsigned>(p.input_width), p.lora);
     }
     return hipSuccess;
 }

@@ -293,7 +293,8 @@ constexpr unsigned kMaxRanges = 256;
 __global__ __launch_bounds__(kSumElements * kSumSlices)
 void stream_backward_sum_kernel(
     const float* __restrict__ partial, float* __restrict__ dx,
-    unsigned elements, unsigned ranges
+    unsigned elements, unsigned ranges, unsigned input_width,
+    LoraEpilogue lora
 ) {
     __shared__ float slices[kSumSlices][kSumElements];
     const unsigned in_block = threadIdx.x % kSumElements;
@@ -328,6 +329,10 @@ void stream_backward_sum_kernel(
         for (int other = 1; other < kSumSlices; ++other) {
             total += slices[other][in_block];
         }
+        if (lora.reduced != nullptr) {  // uniform
+            total += lora_term(lora, element / input_width,
+                               element % input_width);
+        }
         dx[element] = total;
     }
 }
@@ -359,7 +364,10 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     const StreamBackwardPlan plan = plan_for(p);
     float* target = p.result;
     WorkspaceLease lease;  // held until both launches are enqueued
-    if (plan.row_ranges > 1) {
+    // (an adapter term is added by the second kernel, which then runs for
+    // a single range too)
+    const bool two_kernels = plan.row_ranges > 1 || p.lora.reduced != nullptr;
+    if (two_kernels) {
         if (const hipError_t status = lease_stream_workspace(stream, &lease);
             status != hipSuccess) {
             return status;
@@ -383,13 +391,14 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
                        static_cast<unsigned>(p.input_width),
                        static_cast<unsigned>(p.output_width), p.block_shift,
                        plan);
-    if (plan.row_ranges > 1) {
+    if (two_kernels) {
         const unsigned elements =
             static_cast<unsigned>(p.rows * p.input_width);
         stream_backward_sum_kernel<<<(elements + kSumElements - 1) /
                                          kSumElements,
                                      kSumElements * kSumSlices, 0, stream>>>(
-            target, p.result, elements, plan.row_ranges);
+            target, p.result, elements, plan.row_ranges,
+            static_cast<unsigned>(p.input_width), p.lora);
     }
     return hipSuccess;
 }

@@ -276,6 +276,9 @@ bool backward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
         split->tail.activations += kSplitHeadRows * problem.output_width;
         split->tail.result += kSplitHeadRows * problem.input_width;
     }
+    if (split->tail.lora.reduced != nullptr) {
+        split->tail.lora.reduced += kSplitHeadRows * problem.lora.rank;
+    }
     split->head_family = select_input_backward(split->head);
     split->tail_family = select_input_backward(split->tail);
     // (a tail of up to four rows goes to the streaming family)
@@ -338,7 +341,7 @@ static rthip_status input_backward_common(
     int32_t encoding, uint64_t second_level_block, float offset, float* dx,
     uint64_t rows, uint64_t input_width, uint64_t output_width,
     uint64_t block_size, void* stream, float* partial_sums,
-    std::size_t partial_sum_bytes);
+    std::size_t partial_sum_bytes, const rthip::LoraEpilogue& adapter);
 
 
 uint32_t rthip_abi_version(void) {
@@ -546,6 +549,8 @@ rthip_status linear_forward_common(
         problem.lora.b = lora.b;
         problem.lora.rank = static_cast<unsigned>(lora.rank);
         problem.lora.scale = lora.scale;
+        problem.lora.row_stride = static_cast<unsigned>(lora.rank);
+        problem.lora.rank_stride = 1;
     }
 
     // One family on one problem; RTHIP_OK means "launched".
@@ -911,7 +916,146 @@ rthip_status rthip_nf4_linear_input_backward_with(
     return input_backward_common(
         algorithm, dy, codes, primary_scales, secondary_scales, encoding,
         second_level_block, offset, dx, rows, input_width, output_width,
-        block_size, stream, nullptr, 0);
+        block_size, stream, nullptr, 0, rthip::LoraEpilogue{});
+}
+
+rthip_status rthip_nf4_lora_linear_input_backward_with(
+    int32_t algorithm, const float* dy, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset,
+    const float* lora_a, const float* d_reduced, uint64_t lora_rank,
+    float* dx, uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream
+) {
+    if (lora_a == nullptr || d_reduced == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "the adapter's A matrix and the reduced gradient must "
+                    "not be null");
+    }
+    if (lora_rank == 0 || lora_rank > (1ULL << 20)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "LoRA rank must be greater than zero (and at most 2^20)");
+    }
+    if (rows == 0 || input_width == 0 || output_width == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "quantized linear dimensions must be greater than zero");
+    }
+    if (input_width > UINT32_MAX || rows > UINT32_MAX ||
+        lora_rank > UINT64_MAX / sizeof(float) / rows ||
+        lora_rank > UINT64_MAX / sizeof(float) / input_width) {
+        return fail(RTHIP_INVALID_ARGUMENT, "LoRA dimensions overflow");
+    }
+    if (static_cast<const void*>(dx) == static_cast<const void*>(lora_a) ||
+        static_cast<const void*>(dx) == static_cast<const void*>(d_reduced)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "the input gradient must not alias an adapter operand");
+    }
+    rthip::LoraEpilogue adapter{};
+    adapter.reduced = d_reduced;
+    adapter.b = lora_a;
+    adapter.rank = static_cast<unsigned>(lora_rank);
+    adapter.scale = 1.0F;
+    adapter.row_stride = 1;
+    adapter.rank_stride = static_cast<unsigned>(input_width);
+    return input_backward_common(
+        algorithm, dy, codes, primary_scales, secondary_scales, encoding,
+        second_level_block, offset, dx, rows, input_width, output_width,
+        block_size, stream, nullptr, 0, adapter);
+}
+
+rthip_status rthip_nf4_lora_linear_input_backward(
+    const float* dy, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, const float* lora_a,
+    const float* d_reduced, uint64_t lora_rank, float* dx, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream
+) {
+    return rthip_nf4_lora_linear_input_backward_with(
+        RTHIP_NF4_ALGORITHM_AUTO, dy, codes, primary_scales, secondary_scales,
+        encoding, second_level_block, offset, lora_a, d_reduced, lora_rank,
+        dx, rows, input_width, output_width, block_size, stream);
+}
+
+rthip_status rthip_lora_backward(
+    const float* dy, const float* x, const float* reduced,
+    const float* lora_b, uint64_t lora_rank, float lora_scale,
+    float* d_reduced, float* d_lora_a, float* d_lora_b, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, void* stream
+) {
+    if (dy == nullptr || lora_b == nullptr || d_reduced == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "upstream, the adapter's B matrix and the reduced "
+                    "gradient must not be null");
+    }
+    if (d_lora_a != nullptr && x == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "the gradient of A needs the layer's input");
+    }
+    if (d_lora_b != nullptr && reduced == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "the gradient of B needs the reduced activations");
+    }
+    if (rows == 0 || input_width == 0 || output_width == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "quantized linear dimensions must be greater than zero");
+    }
+    if (lora_rank == 0 || lora_rank > (1ULL << 20)) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "LoRA rank must be greater than zero (and at most 2^20)");
+    }
+    if (!std::isfinite(lora_scale)) {
+        return fail(RTHIP_INVALID_ARGUMENT, "LoRA scale must be finite");
+    }
+    constexpr uint64_t kMaxElements = UINT64_MAX / sizeof(float);
+    if (rows > kMaxElements / output_width ||
+        rows > kMaxElements / input_width ||
+        lora_rank > kMaxElements / rows ||
+        lora_rank > kMaxElements / input_width ||
+        lora_rank > kMaxElements / output_width) {
+        return fail(RTHIP_INVALID_ARGUMENT, "LoRA dimensions overflow");
+    }
+    const void* const outputs[3] = {d_reduced, d_lora_a, d_lora_b};
+    const void* const inputs[4] = {dy, x, reduced, lora_b};
+    for (int out = 0; out < 3; ++out) {
+        if (outputs[out] == nullptr) {
+            continue;
+        }
+        for (const void* input : inputs) {
+            if (outputs[out] == input) {
+                return fail(RTHIP_INVALID_ARGUMENT,
+                            "an adapter gradient must not alias an input");
+            }
+        }
+        for (int other = 0; other < out; ++other) {
+            if (outputs[out] == outputs[other]) {
+                return fail(RTHIP_INVALID_ARGUMENT,
+                            "two adapter gradients share one buffer");
+            }
+        }
+    }
+    if (const rthip_status status = require_device(); status != RTHIP_OK) {
+        return status;
+    }
+    rthip::LoraBackwardProblem problem{};
+    problem.upstream = dy;
+    problem.activations = x;
+    problem.reduced = reduced;
+    problem.b = lora_b;
+    problem.d_reduced = d_reduced;
+    problem.d_a = d_lora_a;
+    problem.d_b = d_lora_b;
+    problem.rows = rows;
+    problem.input_width = input_width;
+    problem.output_width = output_width;
+    problem.rank = lora_rank;
+    problem.scale = lora_scale;
+    if (const hipError_t status = rthip::launch_lora_backward(
+            problem, static_cast<hipStream_t>(stream));
+        status != hipSuccess) {
+        return from_hip(status, "adapter-backward workspace allocation");
+    }
+    return finish_launch("adapter backward launch");
 }
 
 // One input backward.  partial_sums == nullptr: any family, partial results
@@ -923,7 +1067,7 @@ static rthip_status input_backward_common(
     int32_t encoding, uint64_t second_level_block, float offset, float* dx,
     uint64_t rows, uint64_t input_width, uint64_t output_width,
     uint64_t block_size, void* stream, float* partial_sums,
-    std::size_t partial_sum_bytes
+    std::size_t partial_sum_bytes, const rthip::LoraEpilogue& adapter
 ) {
     if (dy == nullptr || dx == nullptr) {
         return fail(RTHIP_INVALID_ARGUMENT,
@@ -958,6 +1102,7 @@ static rthip_status input_backward_common(
     problem.output_width = output_width;
     problem.scratch = partial_sums;
     problem.scratch_bytes = partial_sum_bytes;
+    problem.lora = adapter;
     const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
     if (partial_sums != nullptr) {
         if (rows > rthip::kSmallBackwardMaxRows ||
@@ -1096,7 +1241,7 @@ rthip_status rthip_nf4_linear_input_backward_no_alloc(
         RTHIP_NF4_ALGORITHM_SKINNY, dy, codes, primary_scales,
         secondary_scales, encoding, second_level_block, offset, dx, rows,
         input_width, output_width, block_size, stream, partial_sums,
-        kStaticScratchBytes);
+        kStaticScratchBytes, rthip::LoraEpilogue{});
 }
 
 rthip_status rthip_probe_streaming_read(const void* data, uint64_t bytes,

@@ -137,6 +137,42 @@ def lora_linear_forward(x: torch.Tensor, weight: DeviceWeight,
     return out, reduced
 
 
+def lora_linear_backward(dy: torch.Tensor, x: torch.Tensor,
+                         weight: DeviceWeight, lora_a: torch.Tensor,
+                         lora_b: torch.Tensor, lora_scale: float,
+                         reduced: torch.Tensor,
+                         algorithm: Optional[int] = None):
+    """The backward pass of a Linear with a packed (frozen) weight and a
+    trainable adapter, through rthip_lora_backward and
+    rthip_nf4_lora_linear_input_backward: returns (dx, dA, dB).  `reduced` is
+    x . A^T as lora_linear_forward returned it."""
+    for tensor in (dy, x, lora_a, lora_b, reduced):
+        assert tensor.is_cuda and tensor.dtype == torch.float32 and \
+            tensor.is_contiguous()
+    rows = x.numel() // weight.input_width
+    rank = lora_a.shape[0]
+    assert dy.numel() == rows * weight.output_width
+    assert tuple(lora_a.shape) == (rank, weight.input_width)
+    assert tuple(lora_b.shape) == (weight.output_width, rank)
+    assert reduced.numel() == rows * rank
+    d_reduced = torch.empty((rows, rank), dtype=torch.float32,
+                            device=x.device)
+    d_a = torch.empty_like(lora_a)
+    d_b = torch.empty_like(lora_b)
+    dx = torch.empty((rows, weight.input_width), dtype=torch.float32,
+                     device=x.device)
+    library = load_library()
+    library.lora_backward(
+        dy.data_ptr(), x.data_ptr(), reduced.data_ptr(), lora_b.data_ptr(),
+        rank, float(lora_scale), d_reduced.data_ptr(), d_a.data_ptr(),
+        d_b.data_ptr(), rows, weight.input_width, weight.output_width,
+        _stream())
+    library.lora_linear_input_backward(
+        dy.data_ptr(), weight, lora_a.data_ptr(), d_reduced.data_ptr(), rank,
+        dx.data_ptr(), rows, _stream(), algorithm)
+    return dx, d_a, d_b
+
+
 def matmul(left: torch.Tensor, right: torch.Tensor,
            out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """left [..., rows, shared] x right [..., shared, columns] through

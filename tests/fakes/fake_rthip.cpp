@@ -386,6 +386,86 @@ rthip_status rthip_nf4_lora_linear_forward_with(
         stream);
 }
 
+rthip_status rthip_lora_backward(
+    const float* dy, const float* x, const float* reduced,
+    const float* lora_b, uint64_t lora_rank, float lora_scale,
+    float* d_reduced, float* d_lora_a, float* d_lora_b, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, void*) {
+    if (dy == nullptr || lora_b == nullptr || d_reduced == nullptr ||
+        (d_lora_a != nullptr && x == nullptr) ||
+        (d_lora_b != nullptr && reduced == nullptr) || rows == 0 ||
+        input_width == 0 || output_width == 0 || lora_rank == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "invalid adapter backward arguments");
+    }
+    std::vector<float> scaled(rows * output_width);
+    for (size_t index = 0; index < scaled.size(); ++index) {
+        scaled[index] = dy[index] * lora_scale;
+    }
+    nf4o_matmul(scaled.data(), lora_b, d_reduced, rows, output_width,
+                lora_rank);
+    for (uint64_t o = 0; d_lora_b != nullptr && o < output_width; ++o) {
+        for (uint64_t j = 0; j < lora_rank; ++j) {
+            float total = 0.0F;
+            for (uint64_t m = 0; m < rows; ++m) {
+                total += reduced[m * lora_rank + j] *
+                         scaled[m * output_width + o];
+            }
+            d_lora_b[o * lora_rank + j] = total;
+        }
+    }
+    for (uint64_t j = 0; d_lora_a != nullptr && j < lora_rank; ++j) {
+        for (uint64_t i = 0; i < input_width; ++i) {
+            float total = 0.0F;
+            for (uint64_t m = 0; m < rows; ++m) {
+                total += x[m * input_width + i] * d_reduced[m * lora_rank + j];
+            }
+            d_lora_a[j * input_width + i] = total;
+        }
+    }
+    return RTHIP_OK;
+}
+
+rthip_status rthip_nf4_lora_linear_input_backward(
+    const float* dy, const uint8_t* codes, const void* primary_scales,
+    const float* secondary_scales, int32_t encoding,
+    uint64_t second_level_block, float offset, const float* lora_a,
+    const float* d_reduced, uint64_t lora_rank, float* dx, uint64_t rows,
+    uint64_t input_width, uint64_t output_width, uint64_t block_size,
+    void* stream) {
+    if (lora_a == nullptr || d_reduced == nullptr || lora_rank == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "invalid adapter input backward arguments");
+    }
+    if (const rthip_status status = rthip_nf4_linear_input_backward(
+            dy, codes, primary_scales, secondary_scales, encoding,
+            second_level_block, offset, dx, rows, input_width, output_width,
+            block_size, stream);
+        status != RTHIP_OK) {
+        return status;
+    }
+    std::vector<float> through_a(rows * input_width);
+    nf4o_matmul(d_reduced, lora_a, through_a.data(), rows, lora_rank,
+                input_width);
+    for (size_t index = 0; index < through_a.size(); ++index) {
+        dx[index] = dx[index] + through_a[index];
+    }
+    return RTHIP_OK;
+}
+
+rthip_status rthip_nf4_lora_linear_input_backward_with(
+    int32_t, const float* dy, const uint8_t* codes,
+    const void* primary_scales, const float* secondary_scales,
+    int32_t encoding, uint64_t second_level_block, float offset,
+    const float* lora_a, const float* d_reduced, uint64_t lora_rank,
+    float* dx, uint64_t rows, uint64_t input_width, uint64_t output_width,
+    uint64_t block_size, void* stream) {
+    return rthip_nf4_lora_linear_input_backward(
+        dy, codes, primary_scales, secondary_scales, encoding,
+        second_level_block, offset, lora_a, d_reduced, lora_rank, dx, rows,
+        input_width, output_width, block_size, stream);
+}
+
 rthip_status rthip_nf4_quantize(
     const float* values, uint64_t element_count, uint64_t block_size,
     int32_t encoding, uint64_t second_level_block, uint8_t* codes,

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol(package, library):
 
 
 def test_abi_version(package, library):
-    assert library.abi_version() == (1, 6)
+    assert library.abi_version() == (1, 7)
 
 
 def test_select_algorithm_is_pure_host_logic(package, library):
@@ -137,6 +137,46 @@ def test_lora_arguments_are_checked_before_any_device_work(package, library):
         library.lora_reduce(0x3000, 0, 0x7000, 1, 64, 8)
     with pytest.raises(package.InvalidArgument):
         library.lora_reduce(0x3000, 0x5000, 0x7000, 1, 64, 0)
+
+
+def test_adapter_backward_arguments_are_checked_first(package, library):
+    weight = package.DeviceWeight(
+        64, 64, 64, package.SCALE_FLOAT32, _Fake(0x1000), _Fake(0x2000), None)
+    call = library.lora_backward
+    # (dy, x, reduced, B, rank, scale, d_reduced, dA, dB, rows, I, O)
+    with pytest.raises(package.InvalidArgument):  # no B
+        call(0x3000, 0x4000, 0x5000, 0, 8, 1.0, 0x7000, 0x8000, 0x9000, 1,
+             64, 64)
+    with pytest.raises(package.InvalidArgument):  # dA wanted, no x
+        call(0x3000, None, 0x5000, 0x6000, 8, 1.0, 0x7000, 0x8000, 0x9000,
+             1, 64, 64)
+    assert "input" in library.last_error()
+    with pytest.raises(package.InvalidArgument):  # dB wanted, no reduced
+        call(0x3000, 0x4000, None, 0x6000, 8, 1.0, 0x7000, 0x8000, 0x9000,
+             1, 64, 64)
+    with pytest.raises(package.InvalidArgument):  # rank zero
+        call(0x3000, 0x4000, 0x5000, 0x6000, 0, 1.0, 0x7000, 0x8000, 0x9000,
+             1, 64, 64)
+    with pytest.raises(package.InvalidArgument):  # scale not finite
+        call(0x3000, 0x4000, 0x5000, 0x6000, 8, float("nan"), 0x7000, 0x8000,
+             0x9000, 1, 64, 64)
+    with pytest.raises(package.InvalidArgument):  # dA written over x
+        call(0x3000, 0x4000, 0x5000, 0x6000, 8, 1.0, 0x7000, 0x4000, 0x9000,
+             1, 64, 64)
+    assert "alias" in library.last_error()
+    with pytest.raises(package.InvalidArgument):  # dA and dB in one buffer
+        call(0x3000, 0x4000, 0x5000, 0x6000, 8, 1.0, 0x7000, 0x8000, 0x8000,
+             1, 64, 64)
+    fused = library.lora_linear_input_backward
+    # (dy, weight, A, d_reduced, rank, dx, rows)
+    with pytest.raises(package.InvalidArgument):  # no A
+        fused(0x3000, weight, 0, 0x7000, 8, 0x4000, 1)
+    with pytest.raises(package.InvalidArgument):  # rank zero
+        fused(0x3000, weight, 0x5000, 0x7000, 0, 0x4000, 1)
+    with pytest.raises(package.InvalidArgument):  # dx over d_reduced
+        fused(0x3000, weight, 0x5000, 0x7000, 8, 0x7000, 1)
+    with pytest.raises(package.InvalidArgument):  # dx over dy
+        fused(0x3000, weight, 0x5000, 0x7000, 8, 0x3000, 1)
 
 
 def test_group_arguments_are_checked_before_any_device_work(package, library):

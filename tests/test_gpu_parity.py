@@ -801,6 +801,122 @@ def test_lora_linear_forward(gpu, package, library, oracle, out_w, in_w,
                 f"lora forward/{name} rows={rows} vs oracle: {drift:.3g}"
 
 
+def adapter_backward_exact(dy, x, deq, lora_a, lora_b, lora_scale):
+    """fp64: (dx, dA, dB, d_reduced) of y = x deq^T + s (x A^T) B^T."""
+    dy64, x64 = dy.astype(np.float64), x.astype(np.float64)
+    a64, b64 = lora_a.astype(np.float64), lora_b.astype(np.float64)
+    through_b = lora_scale * (dy64 @ b64)
+    return (dy64 @ deq + through_b @ a64, through_b.T @ x64,
+            lora_scale * dy64.T @ (x64 @ a64.T), through_b)
+
+
+@pytest.mark.parametrize("out_w,in_w,block,rank,row_counts", [
+    (768, 256, 64, 8, (1, 16)),         # the tiny parity layer
+    (33, 33, 32, 1, (2,)),              # shape-agnostic kernels, rank one
+    (1000, 1600, 64, 2, (1, 5, 70)),    # rank that is not a multiple of 4
+    (4096, 4096, 64, 16, (1, 3, 64, 80, 300)),  # 80: two launches
+    (512, 2048, 128, 100, (3, 40)),     # more than one chunk of the rank
+    (4096, 11008, 64, 24, (2, 17)),     # dx wider than dy, rank 24
+])
+@pytest.mark.parametrize("double_quantized", [False, True])
+def test_lora_linear_backward(gpu, package, library, oracle, out_w, in_w,
+                              block, rank, row_counts, double_quantized):
+    """dx = dy.deq(W) + ((dy s).B).A, dA and dB through rthip_lora_backward
+    and rthip_nf4_lora_linear_input_backward, every input-backward family,
+    against fp64 and (where the CPU finishes in seconds) against the oracle's
+    restatement of the reference's autograd.  Tolerance: 1e-5 of the standard
+    deviation of each gradient (plus the oracle's own distance from fp64 for
+    the comparison with the oracle)."""
+    import torch
+    dense = helpers.normal(170, (out_w, in_w), 0.02)
+    weight = oracle.quantize(dense, block, double_quantized, 64)
+    device_weight = upload(gpu, weight)
+    deq = oracle.dequantize(weight).astype(np.float64)
+    lora_a = helpers.normal(171, (rank, in_w), 0.05)
+    lora_b = helpers.normal(172, (out_w, rank), 0.05)
+    lora_scale = 16.0 / rank
+    a_device, b_device = to_device(lora_a), to_device(lora_b)
+    for rows in row_counts:
+        x = helpers.normal(173 + rows, (rows, in_w), 1.0)
+        dy = helpers.normal(174 + rows, (rows, out_w), 1.0e-2)
+        exact = adapter_backward_exact(dy, x, deq, lora_a, lora_b, lora_scale)
+        units = [helpers.rms(value) for value in exact]
+        cpu = None
+        if rows * out_w * in_w <= 3.0e8:
+            cpu = oracle.lora_backward(dy, x, weight, lora_a, lora_b,
+                                       lora_scale)
+        x_device, dy_device = to_device(x), to_device(dy)
+        reduced = torch.empty((rows, rank), device="cuda")
+        library.lora_reduce(x_device.data_ptr(), a_device.data_ptr(),
+                            reduced.data_ptr(), rows, in_w, rank)
+        ran = 0
+        for family in families(package):
+            try:
+                got = gpu.lora_linear_backward(
+                    dy_device, x_device, device_weight, a_device, b_device,
+                    lora_scale, reduced, algorithm=family)
+            except package.Unsupported:
+                assert family is not None
+                continue
+            ran += 1
+            got = [host(value) for value in got]
+            name = package.ALGORITHM_NAMES[family or 0]
+            for index, what in enumerate(("dx", "dA", "dB")):
+                error = np.abs(got[index] - exact[index]).max() / units[index]
+                assert error <= TOLERANCE, \
+                    f"{what}/{name} rows={rows} vs fp64: {error:.3g}"
+                if cpu is not None:
+                    cpu_error = np.abs(cpu[index] - exact[index]).max() / \
+                        units[index]
+                    drift = np.abs(got[index] - cpu[index]).max() / \
+                        units[index]
+                    assert drift <= TOLERANCE + cpu_error, \
+                        f"{what}/{name} rows={rows} vs oracle: {drift:.3g}"
+        assert ran >= 2   # AUTO and at least the shape-agnostic family
+
+
+def test_lora_backward_pieces_and_repeat_launches(gpu, package, library,
+                                                  oracle):
+    """d_reduced alone (no buffers for dA and dB), the gradients of a second
+    call bit-equal to the first, and an adapter with B = 0 (a fresh adapter):
+    dA and the adapter's share of dx vanish, dx equals the plain backward."""
+    import torch
+    rows, out_w, in_w, rank, scale = 12, 1536, 1024, 16, 2.0
+    weight = oracle.quantize(helpers.normal(180, (out_w, in_w), 0.02), 64)
+    device_weight = upload(gpu, weight)
+    x = to_device(helpers.normal(181, (rows, in_w), 1.0))
+    dy_host = helpers.normal(182, (rows, out_w), 1.0e-2)
+    dy = to_device(dy_host)
+    lora_a = to_device(helpers.normal(183, (rank, in_w), 0.05))
+    lora_b_host = helpers.normal(184, (out_w, rank), 0.05)
+    lora_b = to_device(lora_b_host)
+    reduced = torch.empty((rows, rank), device="cuda")
+    library.lora_reduce(x.data_ptr(), lora_a.data_ptr(), reduced.data_ptr(),
+                        rows, in_w, rank)
+    d_reduced = torch.full((rows, rank), 7.0, device="cuda")
+    library.lora_backward(dy.data_ptr(), None, None, lora_b.data_ptr(), rank,
+                          scale, d_reduced.data_ptr(), None, None, rows,
+                          in_w, out_w)
+    exact = scale * (dy_host.astype(np.float64) @
+                     lora_b_host.astype(np.float64))
+    assert np.abs(host(d_reduced) - exact).max() / helpers.rms(exact) \
+        <= TOLERANCE
+    first = [host(value) for value in gpu.lora_linear_backward(
+        dy, x, device_weight, lora_a, lora_b, scale, reduced)]
+    second = [host(value) for value in gpu.lora_linear_backward(
+        dy, x, device_weight, lora_a, lora_b, scale, reduced)]
+    for one, two in zip(first, second):
+        helpers.assert_bit_equal(one, two)
+    zero_b = torch.zeros_like(lora_b)
+    dx, d_a, d_b = gpu.lora_linear_backward(dy, x, device_weight, lora_a,
+                                            zero_b, scale, reduced)
+    assert not host(d_a).any()
+    assert host(d_b).any()
+    helpers.assert_bit_equal(host(dx),
+                             host(gpu.linear_input_backward(dy,
+                                                            device_weight)))
+
+
 def test_lora_forward_with_a_precomputed_first_product(gpu, package, library,
                                                        oracle):
     """One rthip_lora_reduce over the stacked A matrices of two projections
