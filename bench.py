@@ -22,6 +22,9 @@ The same JSON line carries
   gemm          M = 2048 forward and input-backward GEMMs (prefill / training
                 shapes) with their fp32-MFMA rooflines
   small_batch   M in {1, 4, 16, 64} on the three distinct shapes
+  small_batch_groups
+                q/k/v and gate/up at M in {4, 16, 64}: one launch per
+                projection against one launch per group
   large_launches
                 M = 1 launches of 74 and 101 MB (lm_head; four gate/up weights
                 in one grouped launch)
@@ -333,6 +336,59 @@ def bench_small_batch(package, device, torch, steps):
                 "tflop_per_s": 2.0 * rows * out_w * in_w / milliseconds / 1e9,
             })
         del weights
+    return results
+
+
+def bench_small_batch_groups(package, device, torch, steps):
+    """Projections that read the same x (q/k/v; gate/up) at M in {4, 16, 64}:
+    one launch per projection against one launch per group
+    (rthip_nf4_linear_forward_group).  us and rates are per GROUP."""
+    library = package.load_library()
+    results = []
+    for name, shapes in (("q/k/v", [(4096, 4096)] * 3),
+                         ("gate/up", [(11008, 4096)] * 2)):
+        copies = 12 if name == "q/k/v" else 6
+        groups = [[synthetic_weight(package, torch, out_w, in_w, False,
+                                    1200 + 10 * copy + index)
+                   for index, (out_w, in_w) in enumerate(shapes)]
+                  for copy in range(copies)]
+        payload = sum(weight.payload_bytes for weight in groups[0])
+        flops_per_row = sum(2.0 * out_w * in_w for out_w, in_w in shapes)
+        for rows in (4, 16, 64):
+            source = torch.randn(rows, 4096, device="cuda")
+            outputs = [torch.empty(rows, out_w, device="cuda")
+                       for out_w, _ in shapes]
+
+            def one_by_one():
+                for group in groups:
+                    for weight, out in zip(group, outputs):
+                        device.linear_forward(source, weight, out=out)
+
+            def together():
+                stream = torch.cuda.current_stream().cuda_stream
+                for group in groups:
+                    library.linear_forward_group(
+                        source.data_ptr(),
+                        [(weight, None, out.data_ptr())
+                         for weight, out in zip(group, outputs)], rows, stream)
+
+            timings = {}
+            for label, body in (("one_by_one", one_by_one),
+                                ("together", together)):
+                body()
+                torch.cuda.synchronize()
+                body = capture(torch, body)
+                body()
+                timings[label] = time_region(torch, body, steps) / (
+                    steps * len(groups)) * 1e3
+            results.append({
+                "group": name, "rows": rows,
+                "one_launch_per_projection_us": timings["one_by_one"],
+                "one_launch_per_group_us": timings["together"],
+                "gb_per_s": payload / timings["together"] / 1e3,
+                "tflop_per_s": rows * flops_per_row / timings["together"] / 1e6,
+            })
+        del groups
     return results
 
 
@@ -734,6 +790,8 @@ def main():
         print(json.dumps({
             "small_batch": bench_small_batch(package, device, torch,
                                              arguments.steps),
+            "small_batch_groups": bench_small_batch_groups(
+                package, device, torch, arguments.steps),
             "small_batch_input_backward": bench_small_batch_backward(
                 package, device, torch, arguments.steps)}))
         return
@@ -797,6 +855,8 @@ def main():
                                   max(3, arguments.steps // 4))
         line["small_batch"] = bench_small_batch(package, device, torch,
                                                 max(3, arguments.steps // 4))
+        line["small_batch_groups"] = bench_small_batch_groups(
+            package, device, torch, max(3, arguments.steps // 4))
         line["large_launches"] = bench_large_launches(
             package, device, torch, max(3, arguments.steps // 2))
         line["practical_roof"] = bench_practical_roof(

@@ -94,6 +94,13 @@ constexpr std::size_t kResidentMaxRows = 64;
 bool resident_forward_supports(const LinearProblem& problem);
 hipError_t launch_resident_forward(const LinearProblem& problem,
                                    hipStream_t stream);
+// Up to kResidentGroupMax weights applied to the same activations in ONE
+// launch; every output equals, bit for bit, what launch_resident_forward
+// writes for that member alone.
+constexpr std::size_t kResidentGroupMax = 4;
+bool resident_group_supports(const LinearProblem* problems, std::size_t count);
+hipError_t launch_resident_group(const LinearProblem* problems,
+                                 std::size_t count, hipStream_t stream);
 
 constexpr std::size_t kSkinnyMaxRows = 64;
 bool skinny_forward_supports(const LinearProblem& problem);

@@ -41,6 +41,15 @@
 //     (and at the end) the workgroup meets at a barrier, adds the eight
 //     partial tiles of each parked output tile in wavefront order and writes y
 //     with bias and adapter term.  Nothing depends on scheduling.
+//   * Several weights that share x (the query, key and value projections; the
+//     gate and up projections) can run as ONE launch: their tiles, each
+//     weight's padded to a multiple of eight, are numbered one after the other
+//     and dealt exactly as one weight's tiles are, so every output is computed
+//     by the same lanes in the same order as in a launch of its own -- bit
+//     for bit the same -- while the launch, the table and the x slice are
+//     paid for once (at 16 rows of 4096 the x slice alone is a quarter of a
+//     single launch).  The member a tile belongs to is looked up per tile
+//     from the kernel arguments (scalar work, a few dozen instructions).
 
 #include "kernels.hpp"
 #include "nf4_decode.hpp"
@@ -73,13 +82,29 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_buffer(const void* base,
         const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
 }
 
+// The weights of one launch.  Tiles are numbered member after member, each
+// member's count padded to a multiple of eight; first_tile of the slots past
+// `count` is the total.
+struct ResidentMember {
+    Nf4WeightView weight;
+    const float* bias;
+    float* y;
+    unsigned output_width;
+};
+struct ResidentGroup {
+    ResidentMember member[kResidentGroupMax];
+    unsigned first_tile[kResidentGroupMax + 1];
+    unsigned count;
+};
+
 // kGroups: contraction groups per wavefront; the row width is 1024 * kGroups.
-template <int kGroups, bool kDoubleQuantized>
+// kGrouped: more than one member (otherwise member 0 is used throughout and
+// nothing is looked up per tile).
+template <int kGroups, bool kDoubleQuantized, bool kGrouped>
 __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
-    const float* __restrict__ x, Nf4WeightView weight,
-    const float* __restrict__ bias, float* __restrict__ y, unsigned rows,
-    unsigned output_width, unsigned block_shift, unsigned tile_count,
-    unsigned row_groups, unsigned iterations, LoraEpilogue lora
+    const float* __restrict__ x, ResidentGroup group, unsigned rows,
+    unsigned block_shift, unsigned row_groups, unsigned iterations,
+    LoraEpilogue lora
 ) {
     constexpr unsigned kInputWidth = 1024U * kGroups;
     constexpr int kSubChunks = 2 * kGroups;  // 16 weights each
@@ -109,21 +134,56 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
         return item / (8 * row_groups) * 8 + item % 8;
     };
 
-    const std::size_t elements =
-        static_cast<std::size_t>(output_width) * kInputWidth;  // < 2^32
-    const std::size_t block_total =
-        (elements + (std::size_t{1} << block_shift) - 1) >> block_shift;
     const __amdgpu_buffer_rsrc_t x_buffer = raw_buffer(
         x, static_cast<std::size_t>(rows) * kInputWidth * sizeof(float));
-    const __amdgpu_buffer_rsrc_t code_buffer =
-        raw_buffer(weight.codes, elements / 2);
-    const __amdgpu_buffer_rsrc_t primary_buffer = raw_buffer(
-        weight.primary_scales, block_total * (kDoubleQuantized ? 1 : 4));
-    const __amdgpu_buffer_rsrc_t secondary_buffer = raw_buffer(
-        weight.secondary_scales,
-        kDoubleQuantized
-            ? (((block_total - 1) >> weight.second_level_shift) + 1) * 4
-            : 0);
+
+    // What the loads of one member need (all of it scalar).
+    struct Source {
+        __amdgpu_buffer_rsrc_t codes, primary, secondary;
+        float offset;
+        unsigned second_level_shift;
+        unsigned output_width;
+        unsigned first_tile;
+    };
+    const auto source_of = [&](unsigned m) {
+        const ResidentMember& member = group.member[m];
+        const std::size_t elements =
+            static_cast<std::size_t>(member.output_width) *
+            kInputWidth;  // < 2^32
+        const std::size_t block_total =
+            (elements + (std::size_t{1} << block_shift) - 1) >> block_shift;
+        Source source;
+        source.codes = raw_buffer(member.weight.codes, elements / 2);
+        source.primary =
+            raw_buffer(member.weight.primary_scales,
+                       block_total * (kDoubleQuantized ? 1 : 4));
+        source.secondary = raw_buffer(
+            member.weight.secondary_scales,
+            kDoubleQuantized
+                ? (((block_total - 1) >> member.weight.second_level_shift) +
+                   1) * 4
+                : 0);
+        source.offset = member.weight.offset;
+        source.second_level_shift = member.weight.second_level_shift;
+        source.output_width = member.output_width;
+        source.first_tile = kGrouped ? group.first_tile[m] : 0U;
+        return source;
+    };
+    // The member that owns a tile (tiles past the last one: the last member,
+    // whose row check then fails).
+    const auto member_of = [&](unsigned tile) {
+        unsigned m = 0;
+        if constexpr (kGrouped) {
+#pragma unroll
+            for (unsigned next = 1; next < kResidentGroupMax; ++next) {
+                if (next < group.count && tile >= group.first_tile[next]) {
+                    m = next;
+                }
+            }
+        }
+        return m;
+    };
+    const Source only = source_of(0);  // (unused code when kGrouped)
 
     struct Codes {
         uintx4 codes[kGroups];  // 32 nibbles each
@@ -132,37 +192,45 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
     // Tiles past the workgroup's last one, and weight rows past the output
     // width, read as zeros.
     const auto load_codes = [&](Codes& staged, unsigned tile) {
-        const unsigned n = tile * kTileRows + lane_row;
-        const bool valid = tile < tile_count && n < output_width;
+        Source source = only;
+        if constexpr (kGrouped) {
+            source = source_of(member_of(tile));
+        }
+        // (a tile is never below its member's first; padding tiles and
+        // tiles past the last member fail the row check)
+        const unsigned n = (tile - source.first_tile) * kTileRows + lane_row;
+        // Real offsets stay below 2^31; lanes with nothing to read get bit 31
+        // set, which the range check rejects.  (One value, kept opaque: a
+        // select per load invites the compiler to branch around the loads,
+        // and its wait counts are exact only on straight-line code.)
+        unsigned reject = n < source.output_width ? 0U : kRejectedOffset;
+        asm volatile("" : "+v"(reject));
         const unsigned flat = n * kInputWidth + k_base;
 #pragma unroll
         for (int g = 0; g < kGroups; ++g) {
             const unsigned first = flat + kGroupWeights * g;
             staged.codes[g] = __builtin_bit_cast(
-                uintx4,
-                __builtin_amdgcn_raw_buffer_load_b128(
-                    code_buffer, valid ? first >> 1 : kRejectedOffset, 0, 0));
+                uintx4, __builtin_amdgcn_raw_buffer_load_b128(
+                            source.codes, (first >> 1) | reject, 0, 0));
             const unsigned block = first >> block_shift;
             if constexpr (!kDoubleQuantized) {
                 staged.scales[g] = __builtin_bit_cast(
                     float, __builtin_amdgcn_raw_buffer_load_b32(
-                               primary_buffer,
-                               valid ? block * 4 : kRejectedOffset, 0, 0));
+                               source.primary, (block * 4) | reject, 0, 0));
             } else {
                 const std::uint8_t scale_code =
                     __builtin_amdgcn_raw_buffer_load_b8(
-                        primary_buffer, valid ? block : kRejectedOffset, 0, 0);
+                        source.primary, block | reject, 0, 0);
                 const float second = __builtin_bit_cast(
                     float,
                     __builtin_amdgcn_raw_buffer_load_b32(
-                        secondary_buffer,
-                        valid ? (block >> weight.second_level_shift) * 4
-                              : kRejectedOffset,
+                        source.secondary,
+                        ((block >> source.second_level_shift) * 4) | reject,
                         0, 0));
                 // Lanes with nothing to read decode (0, 0.0) into the
                 // offset: finite, and never written.
                 staged.scales[g] = decode_double_quantized_scale(
-                    scale_code, second, weight.offset);
+                    scale_code, second, source.offset);
             }
         }
     };
@@ -294,31 +362,38 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
         for (unsigned index = thread; index < count * 256;
              index += kThreads) {
             const unsigned iteration = first_iteration + index / 256;
-            const unsigned m = (index % 256) / 16;
+            const unsigned m_row = (index % 256) / 16;
             const unsigned column = index % 16;
             const unsigned tile = tile_of(iteration);
-            const unsigned n = tile * kTileRows + column;
-            if (tile >= tile_count || n >= output_width || m >= rows_here) {
+            // (a wavefront's 64 outputs belong to one tile)
+            const unsigned m = kGrouped ? __builtin_amdgcn_readfirstlane(
+                                              member_of(tile))
+                                        : 0U;
+            const ResidentMember& member = group.member[m];
+            const unsigned first_tile = kGrouped ? group.first_tile[m] : 0U;
+            const unsigned n = (tile - first_tile) * kTileRows + column;
+            if (n >= member.output_width || m_row >= rows_here) {
                 continue;
             }
             const float* source =
                 reinterpret_cast<const float*>(
                     parked + (iteration % kParkTiles) * kWaves * 64 +
-                    (m / 4) * 16 + column) +
-                m % 4;
+                    (m_row / 4) * 16 + column) +
+                m_row % 4;
             float sum = 0.0F;
 #pragma unroll
             for (int w = 0; w < kWaves; ++w) {
                 sum += source[w * 64 * 4];  // wavefront order
             }
-            if (bias != nullptr) {
-                sum += bias[n];
+            if (member.bias != nullptr) {
+                sum += member.bias[n];
             }
             if (lora.reduced != nullptr) {
-                sum += lora_term(lora, row_base + m, n);
+                sum += lora_term(lora, row_base + m_row, n);
             }
-            y[static_cast<std::size_t>(row_base + m) * output_width + n] =
-                sum;
+            member.y[static_cast<std::size_t>(row_base + m_row) *
+                         member.output_width +
+                     n] = sum;
         }
         __syncthreads();  // the parking slots are free again
     };
@@ -341,16 +416,33 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
     }
 }
 
-template <int kGroups, bool kDoubleQuantized>
-hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
-    const unsigned tiles = static_cast<unsigned>(
-        (p.output_width + kTileRows - 1) / kTileRows);
+template <int kGroups, bool kDoubleQuantized, bool kGrouped>
+hipError_t launch_instance(const LinearProblem* problems, std::size_t count,
+                           hipStream_t stream) {
+    const LinearProblem& p = problems[0];
+    ResidentGroup group{};
+    unsigned tiles = 0;  // each member's padded to a multiple of eight
+    for (std::size_t m = 0; m < kResidentGroupMax; ++m) {
+        group.first_tile[m] = tiles;
+        if (m < count) {
+            const LinearProblem& member = problems[m];
+            group.member[m].weight = member.weight;
+            group.member[m].bias = member.bias;
+            group.member[m].y = member.result;
+            group.member[m].output_width =
+                static_cast<unsigned>(member.output_width);
+            tiles += static_cast<unsigned>(
+                (member.output_width + kTileRows - 1) / kTileRows + 7) / 8 * 8;
+        }
+    }
+    group.first_tile[kResidentGroupMax] = tiles;
+    group.count = static_cast<unsigned>(count);
     const unsigned row_groups =
         static_cast<unsigned>((p.rows + kTileRows - 1) / kTileRows);
-    // Work items (tile, row group), tiles padded to a multiple of eight.  One
-    // workgroup per compute unit, rounded down to a multiple of 8 x row
-    // groups so that a workgroup keeps its row group.
-    const unsigned items = (tiles + 7) / 8 * 8 * row_groups;
+    // Work items (tile, row group).  One workgroup per compute unit, rounded
+    // down to a multiple of 8 x row groups so that a workgroup keeps its row
+    // group.
+    const unsigned items = tiles * row_groups;
     const unsigned granule = 8 * row_groups;
     unsigned groups = kComputeUnits / granule * granule;
     if (groups > items) {
@@ -358,7 +450,8 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     }
     const unsigned iterations = (items + groups - 1) / groups;
     const std::size_t shared_bytes = kStagingBytes;
-    const auto kernel = resident_forward_kernel<kGroups, kDoubleQuantized>;
+    const auto kernel =
+        resident_forward_kernel<kGroups, kDoubleQuantized, kGrouped>;
     // More than the default 64 KB of LDS.
     static const hipError_t configured = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kernel),
@@ -370,16 +463,35 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
         return configured;
     }
     kernel<<<groups, kThreads, shared_bytes, stream>>>(
-        p.activations, p.weight, p.bias, p.result,
-        static_cast<unsigned>(p.rows), static_cast<unsigned>(p.output_width),
-        p.block_shift, tiles, row_groups, iterations, p.lora);
+        p.activations, group, static_cast<unsigned>(p.rows), p.block_shift,
+        row_groups, iterations, p.lora);
     return hipSuccess;
 }
 
 template <int kGroups>
-hipError_t launch_groups(const LinearProblem& p, hipStream_t stream) {
-    return p.weight.encoding == 0 ? launch_instance<kGroups, false>(p, stream)
-                                  : launch_instance<kGroups, true>(p, stream);
+hipError_t launch_groups(const LinearProblem* problems, std::size_t count,
+                         hipStream_t stream) {
+    const bool nested = problems[0].weight.encoding != 0;
+    if (count == 1) {
+        return nested ? launch_instance<kGroups, true, false>(problems, 1,
+                                                              stream)
+                      : launch_instance<kGroups, false, false>(problems, 1,
+                                                               stream);
+    }
+    return nested
+               ? launch_instance<kGroups, true, true>(problems, count, stream)
+               : launch_instance<kGroups, false, true>(problems, count,
+                                                       stream);
+}
+
+hipError_t launch_width(const LinearProblem* problems, std::size_t count,
+                        hipStream_t stream) {
+    switch (problems[0].input_width / 1024) {
+    case 1: return launch_groups<1>(problems, count, stream);
+    case 2: return launch_groups<2>(problems, count, stream);
+    case 3: return launch_groups<3>(problems, count, stream);
+    default: return launch_groups<4>(problems, count, stream);
+    }
 }
 
 }  // namespace
@@ -396,12 +508,34 @@ bool resident_forward_supports(const LinearProblem& p) {
 
 hipError_t launch_resident_forward(const LinearProblem& p,
                                    hipStream_t stream) {
-    switch (p.input_width / 1024) {
-    case 1: return launch_groups<1>(p, stream);
-    case 2: return launch_groups<2>(p, stream);
-    case 3: return launch_groups<3>(p, stream);
-    default: return launch_groups<4>(p, stream);
+    return launch_width(&p, 1, stream);
+}
+
+bool resident_group_supports(const LinearProblem* problems,
+                             std::size_t count) {
+    if (count < 1 || count > kResidentGroupMax) {
+        return false;
     }
+    const LinearProblem& first = problems[0];
+    std::size_t tiles = 0;
+    for (std::size_t m = 0; m < count; ++m) {
+        const LinearProblem& p = problems[m];
+        if (!resident_forward_supports(p) || p.lora.reduced != nullptr ||
+            p.activations != first.activations || p.rows != first.rows ||
+            p.input_width != first.input_width ||
+            p.block_shift != first.block_shift ||
+            p.weight.encoding != first.weight.encoding) {
+            return false;
+        }
+        tiles += (p.output_width + kTileRows - 1) / kTileRows + 8;
+    }
+    // tile numbers times row groups stay far inside 32 bits
+    return tiles < (1ULL << 26);
+}
+
+hipError_t launch_resident_group(const LinearProblem* problems,
+                                 std::size_t count, hipStream_t stream) {
+    return launch_width(problems, count, stream);
 }
 
 }  // namespace rthip

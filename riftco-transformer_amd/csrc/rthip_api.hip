@@ -891,6 +891,37 @@ rthip_status rthip_nf4_linear_forward_group(
             next += run;
             continue;
         }
+        // ... or that the kernel which keeps x in registers takes (two or
+        // more members for each of which that kernel is the automatic choice)
+        run = member_count - next < rthip::kResidentGroupMax
+                  ? member_count - next
+                  : rthip::kResidentGroupMax;
+        const auto resident_run = [&](uint64_t length) {
+            for (uint64_t m = 0; m < length; ++m) {
+                if (select_forward(problems[next + m]) !=
+                    RTHIP_NF4_ALGORITHM_RESIDENT) {
+                    return false;
+                }
+            }
+            return rthip::resident_group_supports(problems + next, length);
+        };
+        while (run > 1 && !resident_run(run)) {
+            --run;
+        }
+        if (run > 1) {
+            if (const hipError_t status = rthip::launch_resident_group(
+                    problems + next, run, hip_stream);
+                status != hipSuccess) {
+                return from_hip(status, "NF4 linear forward launch");
+            }
+            if (const rthip_status status =
+                    finish_launch("NF4 linear forward launch");
+                status != RTHIP_OK) {
+                return status;
+            }
+            next += run;
+            continue;
+        }
         const rthip_nf4_member& member = members[next];
         if (const rthip_status status = linear_forward_common(
                 RTHIP_NF4_ALGORITHM_AUTO, x, member.codes,

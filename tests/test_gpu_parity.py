@@ -327,12 +327,17 @@ def test_wide_rows_at_three_and_four_rows(gpu, package, library, oracle, out_w,
     ((64, 300), 8192 + 256, 128, False),       # one 512-thread team per row
     ((48, 50, 52, 54, 56, 58), 256, 64, True),  # more members than one launch
     ((130,), 512, 64, False),                  # a group of one
+    ((1000, 24, 2050), 2048, 64, True),        # tile counts padded to eight
+    ((9, 17, 300, 8, 130), 1024, 32, False),   # five members, x in registers
+    ((520, 40), 3072, 128, True),
 ])
 def test_group_of_weights_that_share_an_input(gpu, package, library, oracle,
                                               widths, in_w, block,
                                               double_quantized):
     """rthip_nf4_linear_forward_group against one call per member (bit for
-    bit) and against the CPU oracle."""
+    bit) and against the CPU oracle: up to four rows through the streaming
+    kernel, five to sixty-four through the kernel that keeps x in registers
+    (row widths of 1024...4096), anything else one launch per member."""
     weights = [oracle.quantize(helpers.normal(300 + m, (out_w, in_w), 0.02),
                                block, double_quantized, 256)
                for m, out_w in enumerate(widths)]
@@ -341,7 +346,7 @@ def test_group_of_weights_that_share_an_input(gpu, package, library, oracle,
               for m, out_w in enumerate(widths)]
     device_biases = [None if bias is None else to_device(bias)
                      for bias in biases]
-    for rows in (1, 2, 3, 4, 7):
+    for rows in (1, 2, 3, 4, 7, 16, 40, 64):
         x = helpers.normal(340 + rows, (rows, in_w), 1.0)
         x_device = to_device(x)
         together = gpu.linear_forward_group(x_device, device_weights,
@@ -351,7 +356,7 @@ def test_group_of_weights_that_share_an_input(gpu, package, library, oracle,
                                             device_biases[m]))
             helpers.assert_bit_equal(host(together[m]), alone,
                                      f"member {m} at {rows} rows")
-        if rows in (1, 4):
+        if rows in (1, 4, 16):
             for m in (0, len(weights) - 1):
                 dense = oracle.dequantize(weights[m])
                 cpu = oracle.forward(x, weights[m], biases[m])
@@ -1278,7 +1283,8 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
     """A decode loop is launch-bound and runs from a HIP graph (the benchmark
     does).  One graph holds a launch of every forward family, the partial-tile
     path of the small-batch family with its second kernel and workspace, the
-    adapter epilogue and the input backward; each of several replays, with
+    adapter epilogue, the input backward and the adapter's backward; each of
+    several replays, with
     eager launches and synchronisations in between and fresh inputs written
     into the captured buffers, must equal the eager result bit for bit."""
     import torch
@@ -1322,6 +1328,21 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
                 gpu.linear_input_backward(
                     upstream[:rows].contiguous(), device_weight,
                     algorithm=package.ALGORITHM_GEMV)
+        # the adapter's gradients (column slices summed through the
+        # workspace) and the input backward with the adapter's share of dx in
+        # its epilogue, tiled (130 rows) and small-batch (9 rows)
+        for name, rows in (("mfma", 130), ("resident", 9)):
+            x = inputs[name]
+            reduced = torch.empty((rows, 8), device="cuda")
+            library.lora_reduce(x.data_ptr(), lora_a.data_ptr(),
+                                reduced.data_ptr(), rows, 2048, 8,
+                                torch.cuda.current_stream().cuda_stream)
+            (outputs[f"adapter backward {rows}, dx"],
+             outputs[f"adapter backward {rows}, dA"],
+             outputs[f"adapter backward {rows}, dB"]) = \
+                gpu.lora_linear_backward(
+                    upstream[:rows].contiguous(), x, device_weight, lora_a,
+                    lora_b, 0.5, reduced)
         return outputs
 
     def refill(seed):
