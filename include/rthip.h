@@ -181,9 +181,11 @@ rthip_status rthip_nf4_linear_input_backward(
  * does the same with its gate and up projections).  The result is, bit for
  * bit, that of member_count calls of rthip_nf4_linear_forward; the point is
  * the launch count: for rows <= 4 up to four members run as ONE streaming
- * launch, which removes the fixed cost between decode-sized kernels.  Other
- * row counts, or members the streaming kernel cannot take, are launched one
- * by one.  The members share input_width, block_size, encoding and
+ * launch, which removes the fixed cost between decode-sized kernels, and for
+ * rows <= 64 with a row width of 1024, 2048, 3072 or 4096 up to four members
+ * run as ONE launch of the kernel that keeps x in registers, which loads x
+ * once for all of them.  Other shapes are launched one by one.  The members
+ * share input_width, block_size, encoding and
  * second_level_block; each has its own output_width, offset, bias and y.
  * `members` is a HOST array, read before the call returns.
  */
