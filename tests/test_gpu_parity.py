@@ -734,6 +734,70 @@ def test_prefill_shapes_at_full_size(gpu, package, library, oracle, out_w,
     assert abs(lhs - rhs) <= bound
 
 
+@pytest.mark.parametrize("out_w,in_w,double_quantized", [
+    (11008, 4096, True), (4096, 11008, False)])
+def test_adapter_step_at_full_size(gpu, package, library, oracle, out_w, in_w,
+                                   double_quantized):
+    """One training step of a layer with a rank-16 adapter at M = 2048: the
+    fused forward and the backward (dx, dA, dB) against fp64 products over the
+    bit-exact deq(W) computed on the device by the vendor BLAS, and a property
+    that needs no reference: for a direction (U, V) in the space of (A, B),
+    <dy, y(A + hU, B + hV) - y(A - hU, B - hV)> / 2h = <dA, U> + <dB, V>
+    exactly (y is bilinear in (A, B), so the central difference has no
+    truncation error; what is left is the rounding of the two forward
+    passes)."""
+    import torch
+    rows, rank, scale = 2048, 16, 2.0
+    dense = helpers.normal(190, (out_w, in_w), 0.02)
+    weight = oracle.quantize(dense, 64, double_quantized, 256)
+    device_weight = upload(gpu, weight)
+    deq = gpu.dequantize(device_weight).double()
+    x = to_device(helpers.normal(191, (rows, in_w), 1.0))
+    dy = to_device(helpers.normal(192, (rows, out_w), 1.0e-2))
+    lora_a = to_device(helpers.normal(193, (rank, in_w), 0.05))
+    lora_b = to_device(helpers.normal(194, (out_w, rank), 0.05))
+    y, reduced = gpu.lora_linear_forward(x, device_weight, lora_a, lora_b,
+                                         scale)
+    dx, d_a, d_b = gpu.lora_linear_backward(dy, x, device_weight, lora_a,
+                                            lora_b, scale, reduced)
+    x64, dy64 = x.double(), dy.double()
+    a64, b64 = lora_a.double(), lora_b.double()
+    reduced64 = x64 @ a64.T
+    through_b = scale * (dy64 @ b64)
+    for what, got, exact in (
+            ("y", y, x64 @ deq.T + scale * (reduced64 @ b64.T)),
+            ("dx", dx, dy64 @ deq + through_b @ a64),
+            ("dA", d_a, through_b.T @ x64),
+            ("dB", d_b, scale * (dy64.T @ reduced64))):
+        unit = float(exact.pow(2).mean().sqrt())
+        error = float((got.double() - exact).abs().max()) / unit
+        assert error <= TOLERANCE, f"{what} vs fp64: {error:.3g}"
+        del exact
+    # directional derivative of <dy, y> in (A, B), central difference in fp64
+    # arithmetic on the fp32 outputs of the forward kernel
+    u = to_device(helpers.normal(195, (rank, in_w), 0.05))
+    v = to_device(helpers.normal(196, (out_w, rank), 0.05))
+    step = 2.0 ** -6
+
+    def objective(sign):
+        shifted, _ = gpu.lora_linear_forward(
+            x, device_weight, lora_a + sign * step * u,
+            lora_b + sign * step * v, scale)
+        return float((dy64 * shifted.double()).sum())
+
+    slope = (objective(1.0) - objective(-1.0)) / (2.0 * step)
+    predicted = float((d_a.double() * u.double()).sum() +
+                      (d_b.double() * v.double()).sum())
+    # the rounding of y in the two forward passes: at most TOLERANCE of an
+    # output's size per output, signs independent, over 2h
+    y_unit = float(y.double().pow(2).mean().sqrt())
+    noise = TOLERANCE * y_unit * float(dy64.norm()) / step
+    assert abs(predicted) > 100 * noise      # the check has teeth
+    assert abs(slope - predicted) <= noise, \
+        f"slope {slope:.6g} vs <dA,U>+<dB,V> {predicted:.6g}, " \
+        f"allowed {noise:.3g}"
+
+
 def test_decode_shapes_small_batches(gpu, package, library, oracle):
     """M in {1, 4, 16, 64} on the three distinct Llama-7B shapes."""
     for name, (out_w, in_w) in (("q_proj", (4096, 4096)),
