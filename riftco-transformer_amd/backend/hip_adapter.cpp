@@ -34,8 +34,10 @@
 #include "core/backend/optim/adam/reference/update.hpp"
 #endif
 
+#include <algorithm>
 #include <array>
 #include <atomic>
+#include <cmath>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
@@ -1030,6 +1032,155 @@ void hip_quantized_linear_forward_group(
           operation);
     finish_operation(runtime,
                      "quantized-linear forward group synchronisation");
+}
+
+namespace {
+
+void require_elements(const TensorStorage& storage, std::size_t rows,
+                      std::size_t columns, std::string_view what) {
+    if (columns != 0 && rows > SIZE_MAX / columns) {
+        throw std::overflow_error("quantized-linear adapter dimensions "
+                                  "overflow");
+    }
+    if (storage.size() != rows * columns) {
+        throw std::invalid_argument(
+            "quantized-linear adapter " + std::string(what) +
+            " does not match the dimensions");
+    }
+}
+
+// The adapter's own rules (LowRankAdapter's constructor,
+// src/nn/low_rank_adapter.cpp:27-62) on what a request carries.
+void require_adapter(std::size_t rank, float scale,
+                     const QuantizedLinearDimensions& dimensions) {
+    if (dimensions.rows == 0 || dimensions.input_width == 0 ||
+        dimensions.output_width == 0) {
+        throw std::invalid_argument(
+            "quantized linear dimensions must be greater than zero");
+    }
+    if (rank == 0 ||
+        rank > std::min(dimensions.input_width, dimensions.output_width)) {
+        throw std::invalid_argument(
+            "LoRA rank must be in [1, min(input_width, output_width)]");
+    }
+    if (!std::isfinite(scale) || scale <= 0.0F) {
+        throw std::invalid_argument(
+            "LoRA alpha divided by rank must be finite and positive");
+    }
+}
+
+}  // namespace
+
+void hip_quantized_linear_adapter_forward(
+    const QuantizedLinearAdapterForwardRequest& request
+) {
+    constexpr std::string_view operation = "quantized-linear adapter forward";
+    const QuantizedLinearDimensions& d = request.dimensions;
+    require_adapter(request.rank, request.scale, d);
+    require_elements(request.input, d.rows, d.input_width, "input");
+    require_elements(request.output, d.rows, d.output_width, "output");
+    require_elements(request.lora_a, request.rank, d.input_width, "A matrix");
+    require_elements(request.lora_b, d.output_width, request.rank,
+                     "B matrix");
+    require_elements(request.reduced, d.rows, request.rank, "reduced buffer");
+    if (request.bias != nullptr) {
+        require_elements(*request.bias, 1, d.output_width, "bias");
+    }
+    const HipRuntime& runtime = require_runtime();
+    launch_pending_forwards();
+    const auto& input = require_hip_tensor(request.input, operation);
+    const auto& weight = require_hip_weight(request.weight, operation);
+    const auto& lora_a = require_hip_tensor(request.lora_a, operation);
+    const auto& lora_b = require_hip_tensor(request.lora_b, operation);
+    auto& reduced = require_hip_tensor(request.reduced, operation);
+    auto& output = require_hip_tensor(request.output, operation);
+    const float* bias = nullptr;
+    if (request.bias != nullptr) {
+        bias = require_hip_tensor(*request.bias, operation).device_for_read();
+    }
+    check(runtime,
+          runtime.nf4_lora_linear_forward(
+              input.device_for_read(),
+              static_cast<const std::uint8_t*>(
+                  weight.packed_codes_native_handle()),
+              weight.primary_scales_native_handle(),
+              static_cast<const float*>(
+                  weight.secondary_scales_native_handle()),
+              static_cast<int32_t>(weight.encoding()),
+              weight.second_level_block_size(), weight.offset(), bias,
+              lora_a.device_for_read(), lora_b.device_for_read(),
+              request.rank, request.scale, reduced.device_for_overwrite(),
+              output.device_for_overwrite(), d.rows, d.input_width,
+              d.output_width, d.block_size, nullptr),
+          operation);
+    finish_operation(runtime,
+                     "quantized-linear adapter forward synchronisation");
+}
+
+void hip_quantized_linear_adapter_backward(
+    const QuantizedLinearAdapterBackwardRequest& request
+) {
+    constexpr std::string_view operation =
+        "quantized-linear adapter backward";
+    const QuantizedLinearDimensions& d = request.dimensions;
+    require_adapter(request.rank, request.scale, d);
+    require_elements(request.upstream, d.rows, d.output_width, "upstream");
+    require_elements(request.input, d.rows, d.input_width, "input");
+    require_elements(request.reduced, d.rows, request.rank, "reduced buffer");
+    require_elements(request.lora_a, request.rank, d.input_width, "A matrix");
+    require_elements(request.lora_b, d.output_width, request.rank,
+                     "B matrix");
+    require_elements(request.input_gradient, d.rows, d.input_width,
+                     "input gradient");
+    require_elements(request.lora_a_gradient, request.rank, d.input_width,
+                     "A gradient");
+    require_elements(request.lora_b_gradient, d.output_width, request.rank,
+                     "B gradient");
+    const HipRuntime& runtime = require_runtime();
+    launch_pending_forwards();
+    const auto& upstream = require_hip_tensor(request.upstream, operation);
+    const auto& input = require_hip_tensor(request.input, operation);
+    const auto& reduced = require_hip_tensor(request.reduced, operation);
+    const auto& weight = require_hip_weight(request.weight, operation);
+    const auto& lora_a = require_hip_tensor(request.lora_a, operation);
+    const auto& lora_b = require_hip_tensor(request.lora_b, operation);
+    auto& input_gradient =
+        require_hip_tensor(request.input_gradient, operation);
+    auto& a_gradient = require_hip_tensor(request.lora_a_gradient, operation);
+    auto& b_gradient = require_hip_tensor(request.lora_b_gradient, operation);
+    // (upstream * scale) . B, [rows, rank]: lives for this call only
+    const DeviceBuffer reduced_gradient(
+        d.rows * request.rank * sizeof(float), DeviceBuffer::Kind::Pooled);
+    const float* dy = upstream.device_for_read();
+    check(runtime,
+          runtime.lora_backward(
+              dy, input.device_for_read(), reduced.device_for_read(),
+              lora_b.device_for_read(), request.rank, request.scale,
+              static_cast<float*>(reduced_gradient.get()),
+              a_gradient.device_for_overwrite(),
+              b_gradient.device_for_overwrite(), d.rows, d.input_width,
+              d.output_width, nullptr),
+          operation);
+    check(runtime,
+          runtime.nf4_lora_linear_input_backward(
+              dy,
+              static_cast<const std::uint8_t*>(
+                  weight.packed_codes_native_handle()),
+              weight.primary_scales_native_handle(),
+              static_cast<const float*>(
+                  weight.secondary_scales_native_handle()),
+              static_cast<int32_t>(weight.encoding()),
+              weight.second_level_block_size(), weight.offset(),
+              lora_a.device_for_read(),
+              static_cast<const float*>(reduced_gradient.get()), request.rank,
+              input_gradient.device_for_overwrite(), d.rows, d.input_width,
+              d.output_width, d.block_size, nullptr),
+          operation);
+    // The temporary goes back to the pool when this function returns; the
+    // kernels that read it are queued on the same (null) stream as whatever
+    // uses the memory next, so that is ordered on the device.
+    finish_operation(runtime,
+                     "quantized-linear adapter backward synchronisation");
 }
 
 std::vector<HipPackedWeight> hip_load_packed_model_state(

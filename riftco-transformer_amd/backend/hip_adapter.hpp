@@ -69,6 +69,58 @@ struct HipPackedWeightSource {
 void hip_quantized_linear_forward_group(
     std::span<const QuantizedLinearForwardRequest> requests);
 
+// Linear::forward of a layer that holds a packed weight, an optional bias and
+// a low-rank adapter (src/nn/linear.cpp:147-172 with LowRankAdapter::forward,
+// src/nn/low_rank_adapter.cpp:126-151), and the backward pass the reference's
+// autograd runs through it (src/core/autograd/operations.cpp:176-194,252-277,
+// 480-492; src/nn/quantized_linear.cpp:60-80), each as ONE call on hip
+// storage.  A maintainer wraps the pair in a custom-gradient node whose
+// closure keeps `input` and `reduced`:
+//
+//   forward   output = input.deq(W)^T (+ bias) + scale * (input.A^T).B^T,
+//             reduced = input.A^T
+//   backward  input_gradient  = upstream.deq(W) + ((upstream * scale).B).A
+//             lora_a_gradient = ((upstream * scale).B)^T . input
+//             lora_b_gradient = (upstream * scale)^T . reduced
+//
+// Gradients are written, not added to what the storages hold; the reference
+// adds them to a node's gradient afterwards (Variable::accumulate_gradient,
+// src/core/autograd/graph.cpp:218-242).  Sizes are checked against
+// `dimensions` and `rank`; a rank outside [1, min(input, output width)] or a
+// scale that is not finite and positive is refused with the messages of
+// LowRankAdapter's constructor (src/nn/low_rank_adapter.cpp:27-62).
+struct QuantizedLinearAdapterForwardRequest {
+    const TensorStorage& input;
+    const QuantizedWeightStorage& weight;
+    const TensorStorage* bias;  // [output_width] or null
+    const TensorStorage& lora_a;  // [rank, input_width]
+    const TensorStorage& lora_b;  // [output_width, rank]
+    std::size_t rank;
+    float scale;  // alpha / rank
+    TensorStorage& reduced;  // [rows, rank]
+    TensorStorage& output;   // [rows, output_width]
+    QuantizedLinearDimensions dimensions;
+};
+void hip_quantized_linear_adapter_forward(
+    const QuantizedLinearAdapterForwardRequest& request);
+
+struct QuantizedLinearAdapterBackwardRequest {
+    const TensorStorage& upstream;  // [rows, output_width]
+    const TensorStorage& input;     // [rows, input_width]
+    const TensorStorage& reduced;   // [rows, rank], from the forward
+    const QuantizedWeightStorage& weight;
+    const TensorStorage& lora_a;
+    const TensorStorage& lora_b;
+    std::size_t rank;
+    float scale;
+    TensorStorage& input_gradient;   // [rows, input_width]
+    TensorStorage& lora_a_gradient;  // [rank, input_width]
+    TensorStorage& lora_b_gradient;  // [output_width, rank]
+    QuantizedLinearDimensions dimensions;
+};
+void hip_quantized_linear_adapter_backward(
+    const QuantizedLinearAdapterBackwardRequest& request);
+
 // RIFTCO_TRANSFORMER_HIP_MERGE=1 gives callers that were NOT changed the same
 // launches: quantized_linear_forward calls of one to four rows that follow
 // each other on the same input are held back and launched together (at most

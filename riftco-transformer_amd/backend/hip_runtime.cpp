@@ -87,6 +87,12 @@ void load(HipRuntime& runtime) {
         !bind(library, "rthip_nf4_dequantize", runtime.nf4_dequantize,
               reason) ||
         !bind(library, "rthip_matmul", runtime.matmul, reason) ||
+        !bind(library, "rthip_nf4_lora_linear_forward",
+              runtime.nf4_lora_linear_forward, reason) ||
+        !bind(library, "rthip_lora_backward", runtime.lora_backward,
+              reason) ||
+        !bind(library, "rthip_nf4_lora_linear_input_backward",
+              runtime.nf4_lora_linear_input_backward, reason) ||
         !bind(library, "rthip_nf4_check_payload", runtime.nf4_check_payload,
               reason)) {
         return;

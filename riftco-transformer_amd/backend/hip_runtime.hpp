@@ -41,6 +41,11 @@ struct HipRuntime {
         nullptr;
     decltype(&rthip_nf4_dequantize) nf4_dequantize = nullptr;
     decltype(&rthip_matmul) matmul = nullptr;
+    decltype(&rthip_nf4_lora_linear_forward) nf4_lora_linear_forward =
+        nullptr;
+    decltype(&rthip_lora_backward) lora_backward = nullptr;
+    decltype(&rthip_nf4_lora_linear_input_backward)
+        nf4_lora_linear_input_backward = nullptr;
     decltype(&rthip_nf4_check_payload) nf4_check_payload = nullptr;
 };
 

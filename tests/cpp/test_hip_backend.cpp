@@ -529,6 +529,99 @@ void test_forward_group() {
     }
 }
 
+void test_adapter_layer() {
+    // A layer with a packed weight, a bias and a rank-3 adapter: the fused
+    // forward and backward of backend/hip_adapter.hpp against the CPU
+    // restatement of the reference's autograd (pinned to the compiled
+    // reference's own Linear bit for bit).
+    namespace detail = riftco_transformer::backend_detail;
+    const std::size_t out_w = 40, in_w = 256, rank = 3;
+    const float scale = 8.0F / 3.0F;
+    const auto a_values = pseudo_normal(rank * in_w, 0.05F, 71);
+    const auto b_values = pseudo_normal(out_w * rank, 0.05F, 72);
+    const auto bias_values = pseudo_normal(out_w, 0.01F, 73);
+    for (const bool double_quantized : {false, true}) {
+        const HostWeight weight =
+            quantize(pseudo_normal(out_w * in_w, 0.02F, 70), out_w, in_w, 64,
+                     double_quantized, 32);
+        const auto storage = to_hip(weight);
+        const nf4o_scales scales = weight.view();
+        for (const std::size_t rows : {std::size_t{1}, std::size_t{9}}) {
+            const auto x = pseudo_normal(rows * in_w, 1.0F, 74 + rows);
+            const auto dy = pseudo_normal(rows * out_w, 0.01F, 75 + rows);
+            std::vector<float> want_y(rows * out_w), want_dx(rows * in_w),
+                want_da(rank * in_w), want_db(out_w * rank);
+            nf4o_lora_linear_forward(
+                x.data(), weight.codes.data(), &scales, bias_values.data(),
+                a_values.data(), b_values.data(), rank, scale, want_y.data(),
+                rows, in_w, out_w, 64);
+            nf4o_lora_linear_backward(
+                dy.data(), x.data(), weight.codes.data(), &scales,
+                a_values.data(), b_values.data(), rank, scale, want_dx.data(),
+                want_da.data(), want_db.data(), rows, in_w, out_w, 64);
+
+            auto input = backend::make_tensor_storage(kHip, x);
+            auto upstream = backend::make_tensor_storage(kHip, dy);
+            auto lora_a = backend::make_tensor_storage(kHip, a_values);
+            auto lora_b = backend::make_tensor_storage(kHip, b_values);
+            auto bias = backend::make_tensor_storage(kHip, bias_values);
+            auto reduced =
+                backend::make_tensor_storage(kHip, rows * rank, 0.0F);
+            auto output =
+                backend::make_tensor_storage(kHip, rows * out_w, 0.0F);
+            const backend::QuantizedLinearDimensions dimensions{rows, in_w,
+                                                                out_w, 64};
+            detail::hip_quantized_linear_adapter_forward(
+                {*input, *storage, bias.get(), *lora_a, *lora_b, rank, scale,
+                 *reduced, *output, dimensions});
+            require_close(std::as_const(*output).data(), want_y,
+                          "adapter forward");
+            auto dx = backend::make_tensor_storage(kHip, rows * in_w, 7.0F);
+            auto da = backend::make_tensor_storage(kHip, rank * in_w, 7.0F);
+            auto db = backend::make_tensor_storage(kHip, out_w * rank, 7.0F);
+            detail::hip_quantized_linear_adapter_backward(
+                {*upstream, *input, *reduced, *storage, *lora_a, *lora_b, rank,
+                 scale, *dx, *da, *db, dimensions});
+            require_close(std::as_const(*dx).data(), want_dx,
+                          "adapter backward, input gradient");
+            require_close(std::as_const(*da).data(), want_da,
+                          "adapter backward, A gradient");
+            require_close(std::as_const(*db).data(), want_db,
+                          "adapter backward, B gradient");
+
+            // what a request may not carry
+            require_throws<std::invalid_argument>(
+                [&] {
+                    detail::hip_quantized_linear_adapter_forward(
+                        {*input, *storage, nullptr, *lora_a, *lora_b, 0,
+                         scale, *reduced, *output, dimensions});
+                },
+                "rank zero", "LoRA rank must be in");
+            require_throws<std::invalid_argument>(
+                [&] {
+                    detail::hip_quantized_linear_adapter_forward(
+                        {*input, *storage, nullptr, *lora_a, *lora_b, rank,
+                         -1.0F, *reduced, *output, dimensions});
+                },
+                "negative scale", "finite and positive");
+            require_throws<std::invalid_argument>(
+                [&] {
+                    detail::hip_quantized_linear_adapter_backward(
+                        {*upstream, *input, *reduced, *storage, *lora_a,
+                         *lora_b, rank, scale, *dx, *db, *db, dimensions});
+                },
+                "an A gradient of the wrong size", "A gradient");
+            require_throws<std::invalid_argument>(
+                [&] {
+                    detail::hip_quantized_linear_adapter_forward(
+                        {*input, *storage, lora_a.get(), *lora_a, *lora_b,
+                         rank, scale, *reduced, *output, dimensions});
+                },
+                "a bias of the wrong size", "bias");
+        }
+    }
+}
+
 void test_merged_forwards() {
     // The decoder's pattern, unchanged callers: three projections of one
     // input and then one of another, each through the dispatcher.  Results are
@@ -1102,6 +1195,7 @@ int main(int argc, char** argv) {
         test_accelerator_oracle();
         test_transformer_sized_layer();
         test_forward_group();
+        test_adapter_layer();
         test_merged_forwards();
         test_tensor_storage();
         test_dispatch_validation();
