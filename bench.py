@@ -25,6 +25,7 @@ The same JSON line carries
   small_batch_groups
                 q/k/v and gate/up at M in {4, 16, 64}: one launch per
                 projection against one launch per group
+  ragged_shapes a shape only the shape-agnostic kernels take (4097 x 4095)
   large_launches
                 M = 1 launches of 74 and 101 MB (lm_head; four gate/up weights
                 in one grouped launch)
@@ -389,6 +390,48 @@ def bench_small_batch_groups(package, device, torch, steps):
                 "tflop_per_s": rows * flops_per_row / timings["together"] / 1e6,
             })
         del groups
+    return results
+
+
+def bench_ragged(package, device, torch, steps):
+    """A shape none of the tuned families takes (row width 4095: not a
+    multiple of 16, blocks straddle rows): the shape-agnostic kernels, forward
+    and input backward, at M in {1, 16}."""
+    out_w, in_w = 4097, 4095
+    count = out_w * in_w
+    generator = torch.Generator(device="cuda")
+    generator.manual_seed(77)
+    codes = torch.randint(0, 256, ((count + 1) // 2,), dtype=torch.uint8,
+                          device="cuda", generator=generator)
+    if count % 2:
+        codes[-1] &= 0x0F        # the unused high nibble stays zero
+    scales = torch.rand(-(-count // BLOCK), device="cuda",
+                        generator=generator) * 0.03 + 0.035
+    weight = package.DeviceWeight(out_w, in_w, BLOCK, package.SCALE_FLOAT32,
+                                  codes, scales, None)
+    results = []
+    for rows in (1, 16):
+        source = torch.randn(rows, in_w, device="cuda")
+        upstream = torch.randn(rows, out_w, device="cuda") * 1.0e-2
+        target = torch.empty(rows, out_w, device="cuda")
+        gradient = torch.empty(rows, in_w, device="cuda")
+        timings = {}
+        for label, body in (
+                ("forward", lambda: device.linear_forward(source, weight,
+                                                          out=target)),
+                ("input_backward", lambda: device.linear_input_backward(
+                    upstream, weight, out=gradient))):
+            body()
+            torch.cuda.synchronize()
+            timings[label] = time_region(torch, body, steps) / steps * 1e3
+        results.append({
+            "shape": f"{out_w}x{in_w}", "rows": rows,
+            "forward_us": timings["forward"],
+            "input_backward_us": timings["input_backward"],
+            "forward_gb_per_s": weight.payload_bytes / timings["forward"] / 1e3,
+            "input_backward_gb_per_s":
+                weight.payload_bytes / timings["input_backward"] / 1e3,
+        })
     return results
 
 
@@ -788,6 +831,8 @@ def main():
 
     if arguments.small_batch_only:
         print(json.dumps({
+            "ragged_shapes": bench_ragged(package, device, torch,
+                                          arguments.steps),
             "small_batch": bench_small_batch(package, device, torch,
                                              arguments.steps),
             "small_batch_groups": bench_small_batch_groups(
@@ -857,6 +902,8 @@ def main():
                                                 max(3, arguments.steps // 4))
         line["small_batch_groups"] = bench_small_batch_groups(
             package, device, torch, max(3, arguments.steps // 4))
+        line["ragged_shapes"] = bench_ragged(package, device, torch,
+                                             max(3, arguments.steps // 4))
         line["large_launches"] = bench_large_launches(
             package, device, torch, max(3, arguments.steps // 2))
         line["practical_roof"] = bench_practical_roof(

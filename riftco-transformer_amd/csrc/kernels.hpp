@@ -38,8 +38,8 @@ struct LinearProblem {
 
 // nf4_generic.hip
 void launch_generic_forward(const LinearProblem& problem, hipStream_t stream);
-void launch_generic_input_backward(const LinearProblem& problem,
-                                   hipStream_t stream);
+hipError_t launch_generic_input_backward(const LinearProblem& problem,
+                                         hipStream_t stream);
 void launch_dequantize(const Nf4WeightView& weight, float* out,
                        std::size_t element_count, unsigned block_shift,
                        hipStream_t stream);

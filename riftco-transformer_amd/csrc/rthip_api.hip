@@ -1162,7 +1162,11 @@ static rthip_status input_backward_common(
         -> rthip_status {
     switch (algorithm) {
     case RTHIP_NF4_ALGORITHM_GENERIC:
-        rthip::launch_generic_input_backward(problem, hip_stream);
+        if (const hipError_t status =
+                rthip::launch_generic_input_backward(problem, hip_stream);
+            status != hipSuccess) {
+            return from_hip(status, "input-backward workspace allocation");
+        }
         break;
     case RTHIP_NF4_ALGORITHM_MFMA:
         if (!rthip::mfma_input_backward_supports(problem)) {
