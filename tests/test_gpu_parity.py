@@ -540,7 +540,8 @@ def test_shared_output_tiles_are_added_in_a_fixed_order(gpu, package, library,
 def test_two_host_threads_launch_on_one_stream(gpu, package, library, oracle):
     """Kernels that hand partial results to a second kernel through the
     stream's scratch buffer (the small-batch forward and input backward, the
-    tiled kernel's leftover tiles) are launched from two host threads at once
+    tiled kernel's leftover tiles, the streaming and the shape-agnostic input
+    backward, the adapter's d_reduced) are launched from two host threads at once
     on the same stream, each thread with its own input: a thread's sum kernel
     must never read the other thread's partial results.  Every output equals,
     bit for bit, the one the same call gives alone."""
@@ -552,18 +553,31 @@ def test_two_host_threads_launch_on_one_stream(gpu, package, library, oracle):
         (11008, 4096, 16, "backward"),    # row chunks
         (1000, 4096 + 256, 40, "forward"),
         (11008, 4096, 300, "forward"),    # tiled kernel, leftover tiles
+        (11008, 4096, 1, "backward"),     # streamed weight, row ranges
+        (1001, 4095, 3, "backward"),      # shape-agnostic kernel, row chunks
+        (4096, 1024, 12, "adapter"),      # d_reduced in column slices
     ]
     for out_w, in_w, rows, direction in cases:
         weight = oracle.quantize(helpers.normal(95, (out_w, in_w), 0.02), 64,
                                  False, 256)
         device_weight = upload(gpu, weight)
         width = in_w if direction == "forward" else out_w
-        other = out_w if direction == "forward" else in_w
+        other = {"forward": out_w, "backward": in_w, "adapter": 8}[direction]
         inputs = [to_device(helpers.normal(96 + t, (rows, width), 1.0))
                   for t in range(2)]
 
+        if direction == "adapter":
+            rank = 8
+            lora_b = to_device(helpers.normal(98, (out_w, rank), 0.05))
+
         def call(source, target):
-            if direction == "forward":
+            if direction == "adapter":
+                # target: d_reduced [rows, rank] (source: dy [rows, out_w])
+                library.lora_backward(source.data_ptr(), None, None,
+                                      lora_b.data_ptr(), rank, 2.0,
+                                      target.data_ptr(), None, None, rows,
+                                      in_w, out_w, stream)
+            elif direction == "forward":
                 library.linear_forward(source.data_ptr(), device_weight, None,
                                        target.data_ptr(), rows, stream)
             else:
