@@ -41,6 +41,7 @@
 // (the contraction) x 128 contiguous columns and transposes while writing LDS.
 
 #include "kernels.hpp"
+#include "launch_config.hpp"
 #include "nf4_decode.hpp"
 #include "tile_plan.hpp"
 
@@ -527,12 +528,11 @@ hipError_t launch_encoding(const LinearProblem& p, const GemmShape& shape,
         }
     }
     float* const workspace = lease.data();
-    static const hipError_t configured = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kernel),
-        hipFuncAttributeMaxDynamicSharedMemorySize,
-        static_cast<int>(kTileBytes));
-    if (configured != hipSuccess) {
-        return configured;
+    static std::atomic<std::uint64_t> served{0};
+    if (const hipError_t error = allow_dynamic_lds(
+            reinterpret_cast<const void*>(kernel), kTileBytes, served);
+        error != hipSuccess) {
+        return error;
     }
     kernel<<<plan.whole_tiles + groups, kThreads, kTileBytes, stream>>>(
         p.activations, p.weight, p.bias, p.result, workspace, shape, plan,

@@ -52,6 +52,7 @@
 //     from the kernel arguments (scalar work, a few dozen instructions).
 
 #include "kernels.hpp"
+#include "launch_config.hpp"
 #include "nf4_decode.hpp"
 #include "nf4_pair_table.hpp"
 
@@ -453,14 +454,13 @@ hipError_t launch_instance(const LinearProblem* problems, std::size_t count,
     const auto kernel =
         resident_forward_kernel<kGroups, kDoubleQuantized, kGrouped>;
     // More than the default 64 KB of LDS.
-    static const hipError_t configured = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kernel),
-        hipFuncAttributeMaxDynamicSharedMemorySize,
-        static_cast<int>(kStagingBytes));
     static_assert(kStagingBytes >=
                   kParkTiles * kWaves * 64 * sizeof(floatx4));
-    if (configured != hipSuccess) {
-        return configured;
+    static std::atomic<std::uint64_t> served{0};
+    if (const hipError_t error = allow_dynamic_lds(
+            reinterpret_cast<const void*>(kernel), kStagingBytes, served);
+        error != hipSuccess) {
+        return error;
     }
     kernel<<<groups, kThreads, shared_bytes, stream>>>(
         p.activations, group, static_cast<unsigned>(p.rows), p.block_shift,

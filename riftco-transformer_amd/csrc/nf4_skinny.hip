@@ -40,6 +40,7 @@
 //     lanes with nothing to read, so nothing in the loop is predicated.
 
 #include "kernels.hpp"
+#include "launch_config.hpp"
 #include "nf4_decode.hpp"
 #include "nf4_pair_table.hpp"
 
@@ -491,12 +492,11 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     const auto kernel =
         skinny_forward_kernel<kBlocks, kScales, kDoubleQuantized>;
     // More than the default 64 KB of LDS.
-    static const hipError_t configured = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kernel),
-        hipFuncAttributeMaxDynamicSharedMemorySize,
-        static_cast<int>(kSharedBytes));
-    if (configured != hipSuccess) {
-        return configured;
+    static std::atomic<std::uint64_t> served{0};
+    if (const hipError_t error = allow_dynamic_lds(
+            reinterpret_cast<const void*>(kernel), kSharedBytes, served);
+        error != hipSuccess) {
+        return error;
     }
     const unsigned tiles =
         static_cast<unsigned>((p.output_width + kTileN - 1) / kTileN);

@@ -42,6 +42,7 @@
 //     order.  Nothing depends on scheduling.
 
 #include "kernels.hpp"
+#include "launch_config.hpp"
 #include "nf4_decode.hpp"
 #include "backward_split.hpp"
 #include "nf4_pair_table.hpp"
@@ -391,12 +392,11 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     }
     const auto kernel = small_backward_kernel<kBlocks, kDoubleQuantized>;
     // More than the default 64 KB of LDS (table + parking space).
-    static const hipError_t configured = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kernel),
-        hipFuncAttributeMaxDynamicSharedMemorySize,
-        static_cast<int>(kParkingBytes));
-    if (configured != hipSuccess) {
-        return configured;
+    static std::atomic<std::uint64_t> served{0};
+    if (const hipError_t error = allow_dynamic_lds(
+            reinterpret_cast<const void*>(kernel), kParkingBytes, served);
+        error != hipSuccess) {
+        return error;
     }
     kernel<<<split.units_per_xcd * 8, kThreads, kParkingBytes, stream>>>(
         p.activations, p.weight, target, static_cast<unsigned>(p.rows),

@@ -39,6 +39,7 @@
 // order: no atomics, the result does not depend on timing.
 
 #include "kernels.hpp"
+#include "launch_config.hpp"
 #include "gemv_shared.hpp"
 #include "nf4_decode.hpp"
 #include "nf4_pair_table.hpp"
@@ -379,11 +380,11 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     constexpr int kSharedBytes =
         kStageBytes > kPairTableBytes ? kStageBytes : kPairTableBytes;
     static_assert(kSharedBytes <= 160 * 1024);
-    static const hipError_t configured = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(kernel),
-        hipFuncAttributeMaxDynamicSharedMemorySize, kSharedBytes);
-    if (configured != hipSuccess) {
-        return configured;
+    static std::atomic<std::uint64_t> served{0};
+    if (const hipError_t error = allow_dynamic_lds(
+            reinterpret_cast<const void*>(kernel), kSharedBytes, served);
+        error != hipSuccess) {
+        return error;
     }
     kernel<<<plan.column_groups * plan.row_ranges, kThreads, kSharedBytes,
              stream>>>(p.activations, p.weight, target,
