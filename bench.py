@@ -25,6 +25,9 @@ The same JSON line carries
   small_batch_groups
                 q/k/v and gate/up at M in {4, 16, 64}: one launch per
                 projection against one launch per group
+  mid_batch     M in {128, 192, 256, 512, 1024}: between the small-batch
+                kernels and the prefill shapes (192 is one and a half row
+                tiles of the GEMM)
   ragged_shapes a shape only the shape-agnostic kernels take (4097 x 4095)
   large_launches
                 M = 1 launches of 74 and 101 MB (lm_head; four gate/up weights
@@ -335,6 +338,37 @@ def bench_small_batch(package, device, torch, steps):
                 "shape": name, "rows": rows, "us": milliseconds * 1e3,
                 "gb_per_s": weights[0].payload_bytes / milliseconds / 1e6,
                 "tflop_per_s": 2.0 * rows * out_w * in_w / milliseconds / 1e9,
+            })
+        del weights
+    return results
+
+
+def bench_mid_batch(package, device, torch, steps):
+    """Forward at row counts between the small-batch kernels and prefill."""
+    results = []
+    for name, out_w, in_w in (LAYER_SHAPES[0], LAYER_SHAPES[4],
+                              LAYER_SHAPES[6]):
+        weights = [synthetic_weight(package, torch, out_w, in_w, False, 700 + i)
+                   for i in range(4)]
+        for rows in (128, 192, 256, 512, 1024):
+            source = torch.randn(rows, in_w, device="cuda")
+            target = torch.empty(rows, out_w, device="cuda")
+
+            def body():
+                for weight in weights:
+                    device.linear_forward(source, weight, out=target)
+
+            body()
+            torch.cuda.synchronize()
+            body = capture(torch, body)
+            body()
+            milliseconds = time_region(torch, body, steps) / (
+                steps * len(weights))
+            tflops = 2.0 * rows * out_w * in_w / milliseconds / 1e9
+            results.append({
+                "shape": name, "rows": rows, "us": milliseconds * 1e3,
+                "tflop_per_s": tflops,
+                "frac_of_fp32_mfma_peak": tflops / MFMA_FP32_PEAK_TFLOPS,
             })
         del weights
     return results
@@ -902,6 +936,8 @@ def main():
                                                 max(3, arguments.steps // 4))
         line["small_batch_groups"] = bench_small_batch_groups(
             package, device, torch, max(3, arguments.steps // 4))
+        line["mid_batch"] = bench_mid_batch(package, device, torch,
+                                            max(3, arguments.steps // 4))
         line["ragged_shapes"] = bench_ragged(package, device, torch,
                                              max(3, arguments.steps // 4))
         line["large_launches"] = bench_large_launches(
