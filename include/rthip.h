@@ -340,9 +340,10 @@ rthip_status rthip_nf4_lora_linear_input_backward_with(
 
 /* Which family AUTO selects for a shape: direction 0 = forward, 1 = input
  * backward.  Pure host computation; needs no device.  Row counts just above
- * the small-batch families' 64 (up to 112 forward, 96 backward) run as two
- * launches, the first 64 rows and the rest; the family of the first 64 rows
- * is reported then. */
+ * the small-batch families' 64 run as launches of those families on parts of
+ * 64 rows (forward: up to 112 rows, up to 192 where the register-resident
+ * kernel takes the parts; backward: up to 96); the family of the first 64
+ * rows is reported then. */
 rthip_status rthip_nf4_select_algorithm(
     int32_t direction, uint64_t rows, uint64_t input_width,
     uint64_t output_width, uint64_t block_size, int32_t* algorithm);

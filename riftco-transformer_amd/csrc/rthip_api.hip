@@ -194,10 +194,14 @@ int32_t select_forward(const rthip::LinearProblem& problem) {
     return RTHIP_NF4_ALGORITHM_GENERIC;
 }
 
-// Row counts just above the small-batch kernels' limit run as two launches
-// of those kernels (AUTO only; see linear_forward_common).
+// Row counts just above the small-batch kernels' limit run as two or three
+// launches of those kernels (AUTO only; see linear_forward_common).
 constexpr std::size_t kSplitHeadRows = 64;
 constexpr std::size_t kForwardSplitMaxRows = 112;
+// ... further up where the register-resident kernel takes the parts: the
+// tiled kernel pads 129...192 rows to two 128-row tiles, and a weight of few
+// tiles is cut along the contraction there, which costs partial tiles.
+constexpr std::size_t kResidentSplitMaxRows = 192;
 constexpr std::size_t kBackwardSplitMaxRows = 96;
 bool split_rows(std::size_t rows, std::size_t limit) {
     return rows > kSplitHeadRows && rows <= limit;
@@ -231,34 +235,48 @@ int32_t select_input_backward(const rthip::LinearProblem& problem) {
 
 // Just past the small-batch kernels' 64 rows the tiled kernel would run a
 // 128-row tile that is mostly padding (65 rows of 11008 x 4096: 117 us against
-// 57 us at 64 rows).  AUTO then sends the first 64 rows and the rest through
-// the small-batch families, one launch after the other (74 us; equal from
-// about 112 rows on).  True if `problem` is such a case; head and tail are
-// then the two problems and their families.
+// 57 us at 64 rows).  AUTO then sends the rows through the small-batch
+// families in parts of 64, one launch after the other (65 rows: 74 us; equal
+// to the tiled kernel from about 112 rows on).  Where the parts go to the
+// register-resident kernel this holds up to 192 rows (measured, split against
+// tiled: 4096 x 4096 at 128 rows 49 against 58 us, at 192 rows 74 against
+// 91 us; 11008 x 4096 at 192 rows 173 against 210 us; at 256 rows the tiled
+// kernel wins both).  True if `problem` is such a case; `part` are then the
+// problems and `family` their kernels.
+constexpr std::size_t kMaxRowParts = 3;
 struct RowSplit {
-    rthip::LinearProblem head, tail;
-    int32_t head_family, tail_family;
+    rthip::LinearProblem part[kMaxRowParts];
+    int32_t family[kMaxRowParts];
+    std::size_t count;
 };
+static_assert(kMaxRowParts * kSplitHeadRows >= kResidentSplitMaxRows);
 bool forward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
-    if (!split_rows(problem.rows, kForwardSplitMaxRows)) {
+    if (!split_rows(problem.rows, kResidentSplitMaxRows)) {
         return false;
     }
-    split->head = problem;
-    split->head.rows = kSplitHeadRows;
-    split->tail = problem;
-    split->tail.rows = problem.rows - kSplitHeadRows;
-    if (problem.activations != nullptr) {  // null: a shape query
-        split->tail.activations += kSplitHeadRows * problem.input_width;
-        split->tail.result += kSplitHeadRows * problem.output_width;
+    split->count = (problem.rows + kSplitHeadRows - 1) / kSplitHeadRows;
+    for (std::size_t index = 0; index < split->count; ++index) {
+        const std::size_t first = index * kSplitHeadRows;
+        rthip::LinearProblem& part = split->part[index];
+        part = problem;
+        part.rows = std::min(kSplitHeadRows, problem.rows - first);
+        if (problem.activations != nullptr) {  // null: a shape query
+            part.activations += first * problem.input_width;
+            part.result += first * problem.output_width;
+        }
+        if (part.lora.reduced != nullptr) {
+            part.lora.reduced += first * problem.lora.rank;
+        }
+        split->family[index] = select_forward(part);
+        // (a last part of up to four rows goes to the GEMV)
+        if (!small_batch_family(split->family[index]) &&
+            !(index + 1 == split->count && index > 0 &&
+              split->family[index] == RTHIP_NF4_ALGORITHM_GEMV)) {
+            return false;
+        }
     }
-    if (split->tail.lora.reduced != nullptr) {
-        split->tail.lora.reduced += kSplitHeadRows * problem.lora.rank;
-    }
-    split->head_family = select_forward(split->head);
-    split->tail_family = select_forward(split->tail);
-    return small_batch_family(split->head_family) &&
-           (small_batch_family(split->tail_family) ||
-            split->tail_family == RTHIP_NF4_ALGORITHM_GEMV);
+    return problem.rows <= kForwardSplitMaxRows ||
+           split->family[0] == RTHIP_NF4_ALGORITHM_RESIDENT;
 }
 // The input backward likewise up to 96 rows (11008 x 4096: 117 -> 86...100
 // us), unless dx is much wider than dy, where the tiled kernel is as fast
@@ -268,23 +286,26 @@ bool backward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
         problem.input_width > 2 * problem.output_width) {
         return false;
     }
-    split->head = problem;
-    split->head.rows = kSplitHeadRows;
-    split->tail = problem;
-    split->tail.rows = problem.rows - kSplitHeadRows;
+    rthip::LinearProblem& head = split->part[0];
+    rthip::LinearProblem& tail = split->part[1];
+    split->count = 2;
+    head = problem;
+    head.rows = kSplitHeadRows;
+    tail = problem;
+    tail.rows = problem.rows - kSplitHeadRows;
     if (problem.activations != nullptr) {  // null: a shape query
-        split->tail.activations += kSplitHeadRows * problem.output_width;
-        split->tail.result += kSplitHeadRows * problem.input_width;
+        tail.activations += kSplitHeadRows * problem.output_width;
+        tail.result += kSplitHeadRows * problem.input_width;
     }
-    if (split->tail.lora.reduced != nullptr) {
-        split->tail.lora.reduced += kSplitHeadRows * problem.lora.rank;
+    if (tail.lora.reduced != nullptr) {
+        tail.lora.reduced += kSplitHeadRows * problem.lora.rank;
     }
-    split->head_family = select_input_backward(split->head);
-    split->tail_family = select_input_backward(split->tail);
+    split->family[0] = select_input_backward(head);
+    split->family[1] = select_input_backward(tail);
     // (a tail of up to four rows goes to the streaming family)
-    return split->head_family == RTHIP_NF4_ALGORITHM_SKINNY &&
-           (split->tail_family == RTHIP_NF4_ALGORITHM_SKINNY ||
-            split->tail_family == RTHIP_NF4_ALGORITHM_GEMV);
+    return split->family[0] == RTHIP_NF4_ALGORITHM_SKINNY &&
+           (split->family[1] == RTHIP_NF4_ALGORITHM_SKINNY ||
+            split->family[1] == RTHIP_NF4_ALGORITHM_GEMV);
 }
 
 // ---- the entry point that allocates nothing ------------------------------
@@ -475,11 +496,11 @@ rthip_status rthip_nf4_select_algorithm(
     RowSplit split;
     if (direction == 0) {
         *algorithm = forward_row_split(problem, &split)
-                         ? split.head_family
+                         ? split.family[0]
                          : select_forward(problem);
     } else if (direction == 1) {
         *algorithm = backward_row_split(problem, &split)
-                         ? split.head_family
+                         ? split.family[0]
                          : select_input_backward(problem);
     } else {
         return fail(RTHIP_INVALID_ARGUMENT,
@@ -619,15 +640,12 @@ rthip_status linear_forward_common(
     if (algorithm == RTHIP_NF4_ALGORITHM_AUTO) {
         RowSplit split;
         if (forward_row_split(problem, &split)) {
-            if (const rthip_status status =
-                    launch(split.head_family, split.head);
-                status != RTHIP_OK) {
-                return status;
-            }
-            if (const rthip_status status =
-                    launch(split.tail_family, split.tail);
-                status != RTHIP_OK) {
-                return status;
+            for (std::size_t index = 0; index < split.count; ++index) {
+                if (const rthip_status status =
+                        launch(split.family[index], split.part[index]);
+                    status != RTHIP_OK) {
+                    return status;
+                }
             }
             return finish_launch("NF4 linear forward launch");
         }
@@ -1223,15 +1241,12 @@ static rthip_status input_backward_common(
     if (algorithm == RTHIP_NF4_ALGORITHM_AUTO) {
         RowSplit split;
         if (backward_row_split(problem, &split)) {
-            if (const rthip_status status =
-                    launch(split.head_family, split.head);
-                status != RTHIP_OK) {
-                return status;
-            }
-            if (const rthip_status status =
-                    launch(split.tail_family, split.tail);
-                status != RTHIP_OK) {
-                return status;
+            for (std::size_t index = 0; index < split.count; ++index) {
+                if (const rthip_status status =
+                        launch(split.family[index], split.part[index]);
+                    status != RTHIP_OK) {
+                    return status;
+                }
             }
             return finish_launch("NF4 linear input-backward launch");
         }

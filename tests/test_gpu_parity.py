@@ -217,7 +217,7 @@ def test_llama_rows_against_golden(gpu, package, library, oracle, name,
 
 
 @pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 16, 64, 65, 67, 96, 97, 112,
-                                  113, 130])
+                                  113, 128, 130, 131, 190, 192, 193])
 @pytest.mark.parametrize("double_quantized", [False, True])
 def test_row_counts_across_the_gemv_mfma_crossover(
         gpu, package, library, oracle, rows, double_quantized):
@@ -832,7 +832,7 @@ def test_decode_shapes_small_batches(gpu, package, library, oracle):
     (768, 256, 64, 8, (1, 16)),         # the tiny parity layer
     (33, 33, 32, 1, (2,)),              # shape-agnostic kernels, rank one
     (1000, 1600, 64, 2, (1, 5, 70)),    # rank that is not a multiple of 4
-    (4096, 4096, 64, 16, (1, 4, 64, 100, 300)),  # 100: two launches
+    (4096, 4096, 64, 16, (1, 4, 64, 100, 150, 300)),  # 100: two launches, 150: three
     (512, 2048, 128, 100, (3, 40)),     # more than one 64-row adapter chunk
 ])
 @pytest.mark.parametrize("double_quantized", [False, True])
@@ -1375,10 +1375,11 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
     # name -> (rows, pinned family or None for the automatic choice)
     launches = {"gemv": (2, None), "resident": (9, None),
                 "resident, three row groups": (40, None),
-                "skinny": (40, package.ALGORITHM_SKINNY), "mfma": (130, None)}
+                "skinny": (40, package.ALGORITHM_SKINNY),
+                "resident, three launches": (130, None), "mfma": (200, None)}
     inputs = {name: torch.zeros((rows, 2048), device="cuda")
               for name, (rows, _) in launches.items()}
-    upstream = torch.zeros((130, 1000), device="cuda")
+    upstream = torch.zeros((200, 1000), device="cuda")
     for name, (rows, family) in launches.items():
         if family is None:
             assert package.ALGORITHM_NAMES[library.select_algorithm(
@@ -1408,8 +1409,8 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
                     algorithm=package.ALGORITHM_GEMV)
         # the adapter's gradients (column slices summed through the
         # workspace) and the input backward with the adapter's share of dx in
-        # its epilogue, tiled (130 rows) and small-batch (9 rows)
-        for name, rows in (("mfma", 130), ("resident", 9)):
+        # its epilogue, tiled (200 rows) and small-batch (9 rows)
+        for name, rows in (("mfma", 200), ("resident", 9)):
             x = inputs[name]
             reduced = torch.empty((rows, 8), device="cuda")
             library.lora_reduce(x.data_ptr(), lora_a.data_ptr(),
@@ -1427,7 +1428,7 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
         for index, x in enumerate(inputs.values()):
             x.copy_(to_device(helpers.normal(seed + index, tuple(x.shape),
                                              1.0)))
-        upstream.copy_(to_device(helpers.normal(seed + 9, (130, 1000),
+        upstream.copy_(to_device(helpers.normal(seed + 9, (200, 1000),
                                                 1.0e-2)))
 
     refill(170)
