@@ -86,9 +86,9 @@ enum {
      * input backward: the packed weight is walked row by row as it lies in
      * memory, a lane owning eight of its columns */
     RTHIP_NF4_ALGORITHM_SKINNY = 4,
-    /* up to 64 rows (forward) with a row width of 1024..4096: like SKINNY, but
-     * x stays in registers, 16 rows per workgroup, and the wavefronts split
-     * the contraction axis */
+    /* up to 128 rows (forward) with a row width of 1024..4096: like SKINNY,
+     * but x stays in registers, 16 rows per workgroup, and the wavefronts
+     * split the contraction axis */
     RTHIP_NF4_ALGORITHM_RESIDENT = 5
 };
 
@@ -182,7 +182,7 @@ rthip_status rthip_nf4_linear_input_backward(
  * bit, that of member_count calls of rthip_nf4_linear_forward; the point is
  * the launch count: for rows <= 4 up to four members run as ONE streaming
  * launch, which removes the fixed cost between decode-sized kernels, and for
- * rows <= 64 with a row width of 1024, 2048, 3072 or 4096 up to four members
+ * rows <= 128 with a row width of 1024, 2048, 3072 or 4096 up to four members
  * run as ONE launch of the kernel that keeps x in registers, which loads x
  * once for all of them.  Other shapes are launched one by one.  The members
  * share input_width, block_size, encoding and
@@ -340,10 +340,11 @@ rthip_status rthip_nf4_lora_linear_input_backward_with(
 
 /* Which family AUTO selects for a shape: direction 0 = forward, 1 = input
  * backward.  Pure host computation; needs no device.  Row counts just above
- * the small-batch families' 64 run as launches of those families on parts of
- * 64 rows (forward: up to 112 rows, up to 192 where the register-resident
- * kernel takes the parts; backward: up to 96); the family of the first 64
- * rows is reported then. */
+ * the small-batch families' 64 run as two launches of those families, the
+ * first 64 rows and the rest (forward: up to 112 rows; backward: up to 96).
+ * Where the register-resident kernel takes the rows, 81...128 are one launch
+ * of it and 129...224 two, 128 rows and the rest.  The family of the first
+ * part is reported. */
 rthip_status rthip_nf4_select_algorithm(
     int32_t direction, uint64_t rows, uint64_t input_width,
     uint64_t output_width, uint64_t block_size, int32_t* algorithm);

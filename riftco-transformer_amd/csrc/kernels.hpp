@@ -89,8 +89,8 @@ hipError_t release_stream_workspaces(hipStream_t stream, bool every_stream);
 // operands.  Shapes whose output tiles are shared between workgroups use a
 // per-stream workspace that is allocated on first use, so the launcher can
 // fail.
-// nf4_resident.hip: up to 64 rows in groups of 16, x resident in registers
-constexpr std::size_t kResidentMaxRows = 64;
+// nf4_resident.hip: up to 128 rows in groups of 16, x resident in registers
+constexpr std::size_t kResidentMaxRows = 128;
 bool resident_forward_supports(const LinearProblem& problem);
 hipError_t launch_resident_forward(const LinearProblem& problem,
                                    hipStream_t stream);

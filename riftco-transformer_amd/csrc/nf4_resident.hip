@@ -1,4 +1,4 @@
-// Forward product for up to 64 rows when a row of the weight is short enough
+// Forward product for up to 128 rows when a row of the weight is short enough
 // for x to live in registers (row width 1024, 2048, 3072 or 4096):
 //     y[r, o] = sum_i x[r, i] * codebook[code(o, i)] * scale(o, i / B)
 // restating reference_quantized_linear_forward
@@ -31,7 +31,7 @@
 //     ones.
 //   * Tiles are dealt round-robin to one persistent workgroup per compute
 //     unit; the codes of tile t + 1 are requested before tile t is computed.
-//   * More than 16 rows of x are handled as up to four row groups of 16: a
+//   * More than 16 rows of x are handled as up to eight row groups of 16: a
 //     workgroup holds ONE row group for its whole life, and the work items
 //     (tile, row group) are numbered so that the row groups of a tile go to
 //     workgroups eight apart in the grid -- the same XCD, in the same round of

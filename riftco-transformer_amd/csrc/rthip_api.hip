@@ -194,14 +194,18 @@ int32_t select_forward(const rthip::LinearProblem& problem) {
     return RTHIP_NF4_ALGORITHM_GENERIC;
 }
 
-// Row counts just above the small-batch kernels' limit run as two or three
-// launches of those kernels (AUTO only; see linear_forward_common).
+// Row counts just above the small-batch kernels' limit run as two launches
+// of those kernels (AUTO only; see linear_forward_common).
 constexpr std::size_t kSplitHeadRows = 64;
 constexpr std::size_t kForwardSplitMaxRows = 112;
-// ... further up where the register-resident kernel takes the parts: the
-// tiled kernel pads 129...192 rows to two 128-row tiles, and a weight of few
-// tiles is cut along the contraction there, which costs partial tiles.
-constexpr std::size_t kResidentSplitMaxRows = 192;
+// ... further up where the register-resident kernel takes the parts, in
+// parts of its 128 rows: the tiled kernel pads 129...192 rows to two 128-row
+// tiles, and a weight of few tiles is cut along the contraction there, which
+// costs partial tiles.
+constexpr std::size_t kResidentSplitMaxRows = 224;
+// Up to here the resident kernel's parts are 64 rows and the rest: a fifth
+// row group that is nearly empty costs a whole round of matrix instructions.
+constexpr std::size_t kResidentSmallPartMaxRows = 80;
 constexpr std::size_t kBackwardSplitMaxRows = 96;
 bool split_rows(std::size_t rows, std::size_t limit) {
     return rows > kSplitHeadRows && rows <= limit;
@@ -235,31 +239,53 @@ int32_t select_input_backward(const rthip::LinearProblem& problem) {
 
 // Just past the small-batch kernels' 64 rows the tiled kernel would run a
 // 128-row tile that is mostly padding (65 rows of 11008 x 4096: 117 us against
-// 57 us at 64 rows).  AUTO then sends the rows through the small-batch
-// families in parts of 64, one launch after the other (65 rows: 74 us; equal
-// to the tiled kernel from about 112 rows on).  Where the parts go to the
-// register-resident kernel this holds up to 192 rows (measured, split against
-// tiled: 4096 x 4096 at 128 rows 49 against 58 us, at 192 rows 74 against
-// 91 us; 11008 x 4096 at 192 rows 173 against 210 us; at 256 rows the tiled
-// kernel wins both).  True if `problem` is such a case; `part` are then the
-// problems and `family` their kernels.
-constexpr std::size_t kMaxRowParts = 3;
+// 57 us at 64 rows).  AUTO then sends the first 64 rows and the rest through
+// the small-batch families, one launch after the other (65 rows: 74 us; equal
+// to the tiled kernel from about 112 rows on).  Where the register-resident
+// kernel takes the rows this goes on to 224: it runs 81...128 rows as ONE
+// launch of up to eight row groups (65...80 as 64 and the rest), and 129...224
+// as 128 and the rest.  Measured against the tiled kernel: 4096 x 4096 at 128
+// rows 42 against 59 us, at 192 rows 67 against 92 us; 11008 x 4096 107
+// against 115 us and 164 against 208 us; at 256 rows the tiled kernel is as
+// fast or faster (88 against 89 us, 215 against 212 us; nested scales 95
+// against 93 and 234 against 222).
+// True if `problem` is such a case; `part` are then the problems and `family`
+// their kernels.
+constexpr std::size_t kMaxRowParts = 2;
 struct RowSplit {
     rthip::LinearProblem part[kMaxRowParts];
     int32_t family[kMaxRowParts];
     std::size_t count;
 };
-static_assert(kMaxRowParts * kSplitHeadRows >= kResidentSplitMaxRows);
+static_assert(kMaxRowParts * rthip::kResidentMaxRows >= kResidentSplitMaxRows &&
+              kMaxRowParts * kSplitHeadRows >= kForwardSplitMaxRows);
 bool forward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
-    if (!split_rows(problem.rows, kResidentSplitMaxRows)) {
+    if (problem.rows <= kSplitHeadRows) {
         return false;
     }
-    split->count = (problem.rows + kSplitHeadRows - 1) / kSplitHeadRows;
+    rthip::LinearProblem head = problem;
+    head.rows = kSplitHeadRows;
+    const bool resident =
+        select_forward(head) == RTHIP_NF4_ALGORITHM_RESIDENT;
+    std::size_t part_rows = kSplitHeadRows;
+    if (resident) {
+        if (problem.rows > kResidentSplitMaxRows ||
+            (problem.rows > kResidentSmallPartMaxRows &&
+             problem.rows <= rthip::kResidentMaxRows)) {
+            return false;  // (the second: one launch takes them all)
+        }
+        if (problem.rows > rthip::kResidentMaxRows) {
+            part_rows = rthip::kResidentMaxRows;
+        }
+    } else if (problem.rows > kForwardSplitMaxRows) {
+        return false;
+    }
+    split->count = (problem.rows + part_rows - 1) / part_rows;
     for (std::size_t index = 0; index < split->count; ++index) {
-        const std::size_t first = index * kSplitHeadRows;
+        const std::size_t first = index * part_rows;
         rthip::LinearProblem& part = split->part[index];
         part = problem;
-        part.rows = std::min(kSplitHeadRows, problem.rows - first);
+        part.rows = std::min(part_rows, problem.rows - first);
         if (problem.activations != nullptr) {  // null: a shape query
             part.activations += first * problem.input_width;
             part.result += first * problem.output_width;
@@ -270,13 +296,12 @@ bool forward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
         split->family[index] = select_forward(part);
         // (a last part of up to four rows goes to the GEMV)
         if (!small_batch_family(split->family[index]) &&
-            !(index + 1 == split->count && index > 0 &&
+            !(index > 0 &&
               split->family[index] == RTHIP_NF4_ALGORITHM_GEMV)) {
             return false;
         }
     }
-    return problem.rows <= kForwardSplitMaxRows ||
-           split->family[0] == RTHIP_NF4_ALGORITHM_RESIDENT;
+    return true;
 }
 // The input backward likewise up to 96 rows (11008 x 4096: 117 -> 86...100
 // us), unless dx is much wider than dy, where the tiled kernel is as fast

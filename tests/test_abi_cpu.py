@@ -56,15 +56,16 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(fwd, 8, 3072, 1000, 32) == package.ALGORITHM_RESIDENT
     assert select(fwd, 17, 4096, 4096, 64) == package.ALGORITHM_RESIDENT
     assert select(fwd, 64, 4096, 11008, 64) == package.ALGORITHM_RESIDENT
-    # 65...112 rows: parts of 64 rows as small-batch launches (the family of
-    # the first part is reported), the tiled GEMM after that; where the parts
-    # go to the register-resident kernel, up to 192 rows
+    # 65...112 rows: the first 64 and the rest as two small-batch launches
+    # (the family of the first part is reported), the tiled GEMM after that;
+    # the register-resident kernel takes up to 128 rows in one launch and
+    # 129...224 as 128 and the rest
     assert select(fwd, 65, 4096, 11008, 64) == package.ALGORITHM_RESIDENT
     assert select(fwd, 112, 11008, 4096, 64) == package.ALGORITHM_SKINNY
     assert select(fwd, 113, 11008, 4096, 64) == package.ALGORITHM_MFMA
-    assert select(fwd, 113, 4096, 11008, 64) == package.ALGORITHM_RESIDENT
-    assert select(fwd, 192, 4096, 4096, 64) == package.ALGORITHM_RESIDENT
-    assert select(fwd, 193, 4096, 11008, 64) == package.ALGORITHM_MFMA
+    assert select(fwd, 128, 4096, 11008, 64) == package.ALGORITHM_RESIDENT
+    assert select(fwd, 224, 4096, 4096, 64) == package.ALGORITHM_RESIDENT
+    assert select(fwd, 225, 4096, 11008, 64) == package.ALGORITHM_MFMA
     assert select(fwd, 16, 11008, 4096, 64) == package.ALGORITHM_SKINNY
     assert select(fwd, 16, 5120, 4096, 64) == package.ALGORITHM_SKINNY
     # (row width a multiple of 32 but not of 64 -> tiled GEMM)

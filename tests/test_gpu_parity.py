@@ -216,8 +216,9 @@ def test_llama_rows_against_golden(gpu, package, library, oracle, name,
                                     weight_rms) <= TOLERANCE + own
 
 
-@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 16, 64, 65, 67, 96, 97, 112,
-                                  113, 128, 130, 131, 190, 192, 193])
+@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 16, 64, 65, 67, 80, 81, 96,
+                                  112, 113, 128, 129, 131, 190, 193, 224,
+                                  225])
 @pytest.mark.parametrize("double_quantized", [False, True])
 def test_row_counts_across_the_gemv_mfma_crossover(
         gpu, package, library, oracle, rows, double_quantized):
@@ -282,8 +283,8 @@ def test_small_batch_work_split(gpu, package, library, oracle, out_w, in_w,
 ])
 def test_resident_small_batch_family(gpu, package, library, oracle, out_w,
                                      in_w, block, second, double_quantized):
-    """Up to 64 rows, in row groups of 16, with x resident in registers: row
-    counts from the GEMV's to the family's limit (one to four row groups, full
+    """Up to 128 rows, in row groups of 16, with x resident in registers: row
+    counts from the GEMV's to the family's limit (one to eight row groups, full
     and partly empty), with bias, against the oracle, fp64 and the other
     families (check_layer runs each that accepts the shape)."""
     dense = helpers.normal(73, (out_w, in_w), 0.02)
@@ -292,7 +293,9 @@ def test_resident_small_batch_family(gpu, package, library, oracle, out_w,
     assert library.select_algorithm(package.FORWARD, 64, in_w, out_w,
                                     block) == package.ALGORITHM_RESIDENT
     bias = helpers.normal(74, (out_w,), 0.01)
-    for rows in (1, 5, 16, 17, 33, 48, 64):
+    assert library.select_algorithm(package.FORWARD, 128, in_w, out_w,
+                                    block) == package.ALGORITHM_RESIDENT
+    for rows in (1, 5, 16, 17, 33, 48, 64, 65, 81, 100, 128):
         x = helpers.normal(75 + rows, (rows, in_w), 1.0)
         dy = helpers.normal(76 + rows, (rows, out_w), 1.0e-2)
         check_layer(gpu, package, library, oracle, weight, x, dy, bias=bias,
@@ -346,7 +349,7 @@ def test_group_of_weights_that_share_an_input(gpu, package, library, oracle,
               for m, out_w in enumerate(widths)]
     device_biases = [None if bias is None else to_device(bias)
                      for bias in biases]
-    for rows in (1, 2, 3, 4, 7, 16, 40, 64):
+    for rows in (1, 2, 3, 4, 7, 16, 40, 64, 70, 128):
         x = helpers.normal(340 + rows, (rows, in_w), 1.0)
         x_device = to_device(x)
         together = gpu.linear_forward_group(x_device, device_weights,
@@ -832,7 +835,7 @@ def test_decode_shapes_small_batches(gpu, package, library, oracle):
     (768, 256, 64, 8, (1, 16)),         # the tiny parity layer
     (33, 33, 32, 1, (2,)),              # shape-agnostic kernels, rank one
     (1000, 1600, 64, 2, (1, 5, 70)),    # rank that is not a multiple of 4
-    (4096, 4096, 64, 16, (1, 4, 64, 100, 150, 300)),  # 100: two launches, 150: three
+    (4096, 4096, 64, 16, (1, 4, 64, 70, 100, 150, 300)),  # 70, 150: two launches
     (512, 2048, 128, 100, (3, 40)),     # more than one 64-row adapter chunk
 ])
 @pytest.mark.parametrize("double_quantized", [False, True])
@@ -1376,10 +1379,10 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
     launches = {"gemv": (2, None), "resident": (9, None),
                 "resident, three row groups": (40, None),
                 "skinny": (40, package.ALGORITHM_SKINNY),
-                "resident, three launches": (130, None), "mfma": (200, None)}
+                "resident, two launches": (130, None), "mfma": (300, None)}
     inputs = {name: torch.zeros((rows, 2048), device="cuda")
               for name, (rows, _) in launches.items()}
-    upstream = torch.zeros((200, 1000), device="cuda")
+    upstream = torch.zeros((300, 1000), device="cuda")
     for name, (rows, family) in launches.items():
         if family is None:
             assert package.ALGORITHM_NAMES[library.select_algorithm(
@@ -1409,8 +1412,8 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
                     algorithm=package.ALGORITHM_GEMV)
         # the adapter's gradients (column slices summed through the
         # workspace) and the input backward with the adapter's share of dx in
-        # its epilogue, tiled (200 rows) and small-batch (9 rows)
-        for name, rows in (("mfma", 200), ("resident", 9)):
+        # its epilogue, tiled (300 rows) and small-batch (9 rows)
+        for name, rows in (("mfma", 300), ("resident", 9)):
             x = inputs[name]
             reduced = torch.empty((rows, 8), device="cuda")
             library.lora_reduce(x.data_ptr(), lora_a.data_ptr(),
@@ -1428,7 +1431,7 @@ def test_every_family_replays_from_a_graph(gpu, package, library, oracle):
         for index, x in enumerate(inputs.values()):
             x.copy_(to_device(helpers.normal(seed + index, tuple(x.shape),
                                              1.0)))
-        upstream.copy_(to_device(helpers.normal(seed + 9, (200, 1000),
+        upstream.copy_(to_device(helpers.normal(seed + 9, (300, 1000),
                                                 1.0e-2)))
 
     refill(170)
