@@ -341,7 +341,8 @@ rthip_status rthip_nf4_lora_linear_input_backward_with(
 /* Which family AUTO selects for a shape: direction 0 = forward, 1 = input
  * backward.  Pure host computation; needs no device.  Row counts just above
  * the small-batch families' 64 run as two launches of those families, the
- * first 64 rows and the rest (forward: up to 112 rows; backward: up to 96).
+ * first 64 rows and the rest (forward: up to 112 rows; backward: up to 96,
+ * and up to 192 in three parts where output_width >= 2 * input_width).
  * Where the register-resident kernel takes the rows, 81...128 are one launch
  * of it and 129...224 two, 128 rows and the rest.  The family of the first
  * part is reported. */

@@ -251,14 +251,14 @@ int32_t select_input_backward(const rthip::LinearProblem& problem) {
 // against 93 and 234 against 222).
 // True if `problem` is such a case; `part` are then the problems and `family`
 // their kernels.
-constexpr std::size_t kMaxRowParts = 2;
+constexpr std::size_t kMaxRowParts = 3;
 struct RowSplit {
     rthip::LinearProblem part[kMaxRowParts];
     int32_t family[kMaxRowParts];
     std::size_t count;
 };
-static_assert(kMaxRowParts * rthip::kResidentMaxRows >= kResidentSplitMaxRows &&
-              kMaxRowParts * kSplitHeadRows >= kForwardSplitMaxRows);
+static_assert(2 * rthip::kResidentMaxRows >= kResidentSplitMaxRows &&
+              2 * kSplitHeadRows >= kForwardSplitMaxRows);
 bool forward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
     if (problem.rows <= kSplitHeadRows) {
         return false;
@@ -305,32 +305,44 @@ bool forward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
 }
 // The input backward likewise up to 96 rows (11008 x 4096: 117 -> 86...100
 // us), unless dx is much wider than dy, where the tiled kernel is as fast
-// (4096 x 11008: 117 against 113...132 us).
+// (4096 x 11008: 117 against 113...132 us).  Where dy is at least twice as
+// wide as dx (11008 x 4096) parts of 64 rows win up to 192 rows: the tiled
+// kernel pads 129...192 rows to two row tiles of a long contraction (97 rows
+// 110 -> 98 us, 192 rows 202 -> 168 us; a tie at 128; 4096 x 4096 gains
+// nothing there).
+constexpr std::size_t kLongBackwardSplitMaxRows = 192;
+static_assert(kMaxRowParts * kSplitHeadRows >= kLongBackwardSplitMaxRows);
 bool backward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
-    if (!split_rows(problem.rows, kBackwardSplitMaxRows) ||
+    const std::size_t limit =
+        problem.output_width >= 2 * problem.input_width
+            ? kLongBackwardSplitMaxRows
+            : kBackwardSplitMaxRows;
+    if (!split_rows(problem.rows, limit) ||
         problem.input_width > 2 * problem.output_width) {
         return false;
     }
-    rthip::LinearProblem& head = split->part[0];
-    rthip::LinearProblem& tail = split->part[1];
-    split->count = 2;
-    head = problem;
-    head.rows = kSplitHeadRows;
-    tail = problem;
-    tail.rows = problem.rows - kSplitHeadRows;
-    if (problem.activations != nullptr) {  // null: a shape query
-        tail.activations += kSplitHeadRows * problem.output_width;
-        tail.result += kSplitHeadRows * problem.input_width;
+    split->count = (problem.rows + kSplitHeadRows - 1) / kSplitHeadRows;
+    for (std::size_t index = 0; index < split->count; ++index) {
+        const std::size_t first = index * kSplitHeadRows;
+        rthip::LinearProblem& part = split->part[index];
+        part = problem;
+        part.rows = std::min(kSplitHeadRows, problem.rows - first);
+        if (problem.activations != nullptr) {  // null: a shape query
+            part.activations += first * problem.output_width;
+            part.result += first * problem.input_width;
+        }
+        if (part.lora.reduced != nullptr) {
+            part.lora.reduced += first * problem.lora.rank;
+        }
+        split->family[index] = select_input_backward(part);
+        // (a last part of up to four rows goes to the streaming family)
+        if (split->family[index] != RTHIP_NF4_ALGORITHM_SKINNY &&
+            !(index > 0 &&
+              split->family[index] == RTHIP_NF4_ALGORITHM_GEMV)) {
+            return false;
+        }
     }
-    if (tail.lora.reduced != nullptr) {
-        tail.lora.reduced += kSplitHeadRows * problem.lora.rank;
-    }
-    split->family[0] = select_input_backward(head);
-    split->family[1] = select_input_backward(tail);
-    // (a tail of up to four rows goes to the streaming family)
-    return split->family[0] == RTHIP_NF4_ALGORITHM_SKINNY &&
-           (split->family[1] == RTHIP_NF4_ALGORITHM_SKINNY ||
-            split->family[1] == RTHIP_NF4_ALGORITHM_GEMV);
+    return true;
 }
 
 // ---- the entry point that allocates nothing ------------------------------

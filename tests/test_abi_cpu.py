@@ -85,10 +85,14 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(bwd, 5, 4096, 11008, 64) == package.ALGORITHM_SKINNY
     assert select(bwd, 64, 11008, 4096, 64) == package.ALGORITHM_SKINNY
     assert select(bwd, 16, 40, 768, 32) == package.ALGORITHM_SKINNY
-    # 65...96 rows: two launches of it, unless dx is much wider than dy
+    # 65...96 rows: two launches of it, unless dx is much wider than dy;
+    # up to 192 rows (three launches) where dy is at least twice as wide
     assert select(bwd, 65, 4096, 11008, 64) == package.ALGORITHM_SKINNY
     assert select(bwd, 96, 4096, 4096, 64) == package.ALGORITHM_SKINNY
-    assert select(bwd, 97, 4096, 11008, 64) == package.ALGORITHM_MFMA
+    assert select(bwd, 97, 4096, 4096, 64) == package.ALGORITHM_MFMA
+    assert select(bwd, 97, 4096, 11008, 64) == package.ALGORITHM_SKINNY
+    assert select(bwd, 192, 4096, 11008, 64) == package.ALGORITHM_SKINNY
+    assert select(bwd, 193, 4096, 11008, 64) == package.ALGORITHM_MFMA
     assert select(bwd, 65, 11008, 4096, 64) == package.ALGORITHM_MFMA
     assert select(bwd, 16, 36, 768, 32) == package.ALGORITHM_GENERIC
     # the reference's edge layout -> shape-agnostic kernels

@@ -229,6 +229,21 @@ def test_row_counts_across_the_gemv_mfma_crossover(
     check_layer(gpu, package, library, oracle, weight, x, dy)
 
 
+@pytest.mark.parametrize("rows", [97, 128, 129, 192, 193])
+def test_row_counts_where_the_upstream_is_much_wider(gpu, package, library,
+                                                      oracle, rows):
+    """An input backward whose dy is at least twice as wide as dx runs up to
+    192 rows as parts of 64 through the small-batch kernel."""
+    assert library.select_algorithm(
+        package.INPUT_BACKWARD, rows, 512, 1152, 64) == (
+            package.ALGORITHM_SKINNY if rows <= 192 else package.ALGORITHM_MFMA)
+    weight = oracle.quantize(helpers.normal(54, (1152, 512), 0.02), 64, True,
+                             256)
+    x = helpers.normal(55 + rows, (rows, 512), 1.0)
+    dy = helpers.normal(56 + rows, (rows, 1152), 1.0e-2)
+    check_layer(gpu, package, library, oracle, weight, x, dy, oracle_rows=4)
+
+
 @pytest.mark.parametrize("out_w,in_w,block,second", [
     (96, 160, 32, 32),      # narrow rows, tiles mostly empty
     (200, 352, 32, 64),     # output width not a multiple of the tile
@@ -903,6 +918,7 @@ def adapter_backward_exact(dy, x, deq, lora_a, lora_b, lora_scale):
     (4096, 4096, 64, 16, (1, 3, 64, 80, 300)),  # 80: two launches
     (512, 2048, 128, 100, (3, 40)),     # more than one chunk of the rank
     (4096, 11008, 64, 24, (2, 17)),     # dx wider than dy, rank 24
+    (2304, 1024, 64, 8, (100, 150)),    # dy much wider: three launches at 150
 ])
 @pytest.mark.parametrize("double_quantized", [False, True])
 def test_lora_linear_backward(gpu, package, library, oracle, out_w, in_w,
