@@ -344,8 +344,10 @@ rthip_status rthip_nf4_lora_linear_input_backward_with(
  * first 64 rows and the rest (forward: up to 112 rows; backward: up to 96,
  * and up to 192 in three parts where output_width >= 2 * input_width).
  * Where the register-resident kernel takes the rows, 81...128 are one launch
- * of it and 129...224 two, 128 rows and the rest.  The family of the first
- * part is reported. */
+ * of it and 129...224 two, 128 rows and the rest.  Larger row counts that end
+ * 1...64 rows past a multiple of 128 run as a tiled launch for the whole
+ * 128-row tiles and a small-batch launch for the rest, in both directions.
+ * The family of the first part is reported. */
 rthip_status rthip_nf4_select_algorithm(
     int32_t direction, uint64_t rows, uint64_t input_width,
     uint64_t output_width, uint64_t block_size, int32_t* algorithm);

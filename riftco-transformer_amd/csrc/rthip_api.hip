@@ -259,7 +259,25 @@ struct RowSplit {
 };
 static_assert(2 * rthip::kResidentMaxRows >= kResidentSplitMaxRows &&
               2 * kSplitHeadRows >= kForwardSplitMaxRows);
-bool forward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
+// Rows [first, first + rows) of `problem` as a problem of their own.
+rthip::LinearProblem row_part(const rthip::LinearProblem& problem,
+                              std::size_t first, std::size_t rows,
+                              bool forward) {
+    rthip::LinearProblem part = problem;
+    part.rows = rows;
+    if (problem.activations != nullptr) {  // null: a shape query
+        part.activations +=
+            first * (forward ? problem.input_width : problem.output_width);
+        part.result +=
+            first * (forward ? problem.output_width : problem.input_width);
+    }
+    if (part.lora.reduced != nullptr) {
+        part.lora.reduced += first * problem.lora.rank;
+    }
+    return part;
+}
+bool forward_small_split(const rthip::LinearProblem& problem,
+                         RowSplit* split) {
     if (problem.rows <= kSplitHeadRows) {
         return false;
     }
@@ -283,17 +301,10 @@ bool forward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
     split->count = (problem.rows + part_rows - 1) / part_rows;
     for (std::size_t index = 0; index < split->count; ++index) {
         const std::size_t first = index * part_rows;
-        rthip::LinearProblem& part = split->part[index];
-        part = problem;
-        part.rows = std::min(part_rows, problem.rows - first);
-        if (problem.activations != nullptr) {  // null: a shape query
-            part.activations += first * problem.input_width;
-            part.result += first * problem.output_width;
-        }
-        if (part.lora.reduced != nullptr) {
-            part.lora.reduced += first * problem.lora.rank;
-        }
-        split->family[index] = select_forward(part);
+        split->part[index] =
+            row_part(problem, first,
+                     std::min(part_rows, problem.rows - first), true);
+        split->family[index] = select_forward(split->part[index]);
         // (a last part of up to four rows goes to the GEMV)
         if (!small_batch_family(split->family[index]) &&
             !(index > 0 &&
@@ -312,7 +323,8 @@ bool forward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
 // nothing there).
 constexpr std::size_t kLongBackwardSplitMaxRows = 192;
 static_assert(kMaxRowParts * kSplitHeadRows >= kLongBackwardSplitMaxRows);
-bool backward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
+bool backward_small_split(const rthip::LinearProblem& problem,
+                          RowSplit* split) {
     const std::size_t limit =
         problem.output_width >= 2 * problem.input_width
             ? kLongBackwardSplitMaxRows
@@ -324,17 +336,10 @@ bool backward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
     split->count = (problem.rows + kSplitHeadRows - 1) / kSplitHeadRows;
     for (std::size_t index = 0; index < split->count; ++index) {
         const std::size_t first = index * kSplitHeadRows;
-        rthip::LinearProblem& part = split->part[index];
-        part = problem;
-        part.rows = std::min(kSplitHeadRows, problem.rows - first);
-        if (problem.activations != nullptr) {  // null: a shape query
-            part.activations += first * problem.output_width;
-            part.result += first * problem.input_width;
-        }
-        if (part.lora.reduced != nullptr) {
-            part.lora.reduced += first * problem.lora.rank;
-        }
-        split->family[index] = select_input_backward(part);
+        split->part[index] =
+            row_part(problem, first,
+                     std::min(kSplitHeadRows, problem.rows - first), false);
+        split->family[index] = select_input_backward(split->part[index]);
         // (a last part of up to four rows goes to the streaming family)
         if (split->family[index] != RTHIP_NF4_ALGORITHM_SKINNY &&
             !(index > 0 &&
@@ -343,6 +348,43 @@ bool backward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
         }
     }
     return true;
+}
+
+// The tiled kernel works in row tiles of 128.  A row count that ends up to 64
+// rows past a multiple of 128 would pay a whole tile row for them (11008 x
+// 4096: ~93 us, whatever the count); AUTO gives those last rows to the
+// small-batch families instead, after the tiled launch for the rows before
+// them.  Measured, forward / input backward, nested scales: 272 rows of
+// 11008 x 4096 320 -> 243 / 315 -> 237 us, 320 rows 319 -> 283 / 318 -> 273
+// us, 2080 rows 1682 -> 1618 / 1649 -> 1594 us; 4096 x 4096 at 272 rows
+// 144 -> 116 / 138 -> 112 us; with 94 rows left over both ways are even, so
+// from 65 on the tile row stays.
+constexpr std::size_t kTileRows = 128;
+constexpr std::size_t kTailSplitMaxRows = 64;
+bool tail_split(const rthip::LinearProblem& problem, bool forward,
+                RowSplit* split) {
+    const auto select = forward ? select_forward : select_input_backward;
+    const std::size_t tail = problem.rows % kTileRows;
+    if (problem.rows <= kTileRows || tail == 0 || tail > kTailSplitMaxRows ||
+        select(problem) != RTHIP_NF4_ALGORITHM_MFMA) {
+        return false;
+    }
+    split->count = 2;
+    split->part[0] = row_part(problem, 0, problem.rows - tail, forward);
+    split->part[1] = row_part(problem, problem.rows - tail, tail, forward);
+    split->family[0] = select(split->part[0]);
+    split->family[1] = select(split->part[1]);
+    return split->family[0] == RTHIP_NF4_ALGORITHM_MFMA &&
+           (small_batch_family(split->family[1]) ||
+            split->family[1] == RTHIP_NF4_ALGORITHM_GEMV);
+}
+bool forward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
+    return forward_small_split(problem, split) ||
+           tail_split(problem, true, split);
+}
+bool backward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
+    return backward_small_split(problem, split) ||
+           tail_split(problem, false, split);
 }
 
 // ---- the entry point that allocates nothing ------------------------------

@@ -218,7 +218,7 @@ def test_llama_rows_against_golden(gpu, package, library, oracle, name,
 
 @pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 16, 64, 65, 67, 80, 81, 96,
                                   112, 113, 128, 129, 131, 190, 193, 224,
-                                  225])
+                                  225, 257, 300, 320, 321])
 @pytest.mark.parametrize("double_quantized", [False, True])
 def test_row_counts_across_the_gemv_mfma_crossover(
         gpu, package, library, oracle, rows, double_quantized):
@@ -471,9 +471,10 @@ def test_small_batch_input_backward(gpu, package, library, oracle, out_w, in_w,
                 host(gpu.linear_input_backward(dy_device, device_weight)),
                 first, f"{rows} rows, launch {launch}")
     # 65...96 rows run as two launches of this kernel (unless dx is much
-    # wider than dy), more rows go to the tiled kernel
+    # wider than dy; up to 192 rows where dy is at least twice as wide as
+    # dx), more rows go to the tiled kernel
     assert library.select_algorithm(
-        package.INPUT_BACKWARD, 97, in_w, out_w,
+        package.INPUT_BACKWARD, 97 if out_w < 2 * in_w else 193, in_w, out_w,
         block) != package.ALGORITHM_SKINNY
     rows = 80
     x = helpers.normal(84 + rows, (rows, in_w), 1.0)
