@@ -25,9 +25,9 @@ The same JSON line carries
   small_batch_groups
                 q/k/v and gate/up at M in {4, 16, 64}: one launch per
                 projection against one launch per group
-  mid_batch     M in {128, 192, 256, 512, 1024}: between the small-batch
+  mid_batch     M in {128, 192, 256, 272, 512, 1024}: between the small-batch
                 kernels and the prefill shapes (192 is one and a half row
-                tiles of the GEMM)
+                tiles of the GEMM, 272 two and sixteen rows)
   ragged_shapes a shape only the shape-agnostic kernels take (4097 x 4095)
   large_launches
                 M = 1 launches of 74 and 101 MB (lm_head; four gate/up weights
@@ -350,7 +350,7 @@ def bench_mid_batch(package, device, torch, steps):
                               LAYER_SHAPES[6]):
         weights = [synthetic_weight(package, torch, out_w, in_w, False, 700 + i)
                    for i in range(4)]
-        for rows in (128, 192, 256, 512, 1024):
+        for rows in (128, 192, 256, 272, 512, 1024):
             source = torch.randn(rows, in_w, device="cuda")
             target = torch.empty(rows, out_w, device="cuda")
 
