@@ -585,11 +585,15 @@ std::size_t held_rows(const LinearProblem& p) {
 }
 
 // A thread's register-resident slice of x is held_rows x segments x 16
-// values; beyond 8 x 16 it no longer fits.  Two teams of 256 threads per
-// workgroup measured best; rows too wide for that get one team of 512.
+// values; beyond 8 x 16 it no longer fits, and a thread takes at most four
+// segments of a row.  Two teams of 256 threads per workgroup measured best;
+// rows too wide for that get one team of 512 (three and four rows of x from
+// 8192 weights per row on, one and two rows from 16384 to 32768).
 constexpr std::size_t kMaxHeldSegments = 8;
+constexpr std::size_t kMaxSegments = 4;
 bool wide_team(const LinearProblem& p) {
-    return held_rows(p) * segments_per_thread(p, 256) > kMaxHeldSegments;
+    return held_rows(p) * segments_per_thread(p, 256) > kMaxHeldSegments ||
+           segments_per_thread(p, 256) > kMaxSegments;
 }
 
 // The weights of one launch: `count` problems that share activations, row
@@ -673,10 +677,17 @@ template <int kX, bool kDoubleQuantized, bool kGrouped>
 void launch_segments(const Launch& launch, hipStream_t stream) {
     const LinearProblem& p = launch.problems[0];
     if (wide_team(p)) {
-        // four x rows and a row wider than 8192: two segments per thread of a
-        // 512-thread team
+        // one 512-thread team per weight row: four x rows and a row wider
+        // than 8192 (two segments per thread), one or two x rows and a row
+        // wider than 16384 (three or four)
         if constexpr (kX == 4) {
             launch_instance<kX, 2, kDoubleQuantized, kGrouped, true>(launch,
+                                                                     stream);
+        } else if (segments_per_thread(p, 512) == 3) {
+            launch_instance<kX, 3, kDoubleQuantized, kGrouped, true>(launch,
+                                                                     stream);
+        } else {
+            launch_instance<kX, 4, kDoubleQuantized, kGrouped, true>(launch,
                                                                      stream);
         }
         return;
@@ -731,13 +742,14 @@ void launch_encoding(const Launch& launch, hipStream_t stream) {
 
 bool gemv_forward_supports(const LinearProblem& p) {
     constexpr std::size_t kMaxWidth =
-        static_cast<std::size_t>(kSegment) * 256 * 4;
+        static_cast<std::size_t>(kSegment) * 512 * kMaxSegments;
     return p.rows >= 1 && p.rows <= kGemvMaxRows &&
            // the register-resident x slice must fit, with two teams of 256
-           // threads or, for three and four rows, one team of 512
+           // threads or one team of 512
            (!wide_team(p) ||
-            (held_rows(p) == 4 && held_rows(p) * segments_per_thread(p, 512) <=
-                                      kMaxHeldSegments)) &&
+            (segments_per_thread(p, 512) >= 2 &&
+             held_rows(p) * segments_per_thread(p, 512) <=
+                 kMaxHeldSegments)) &&
            p.input_width % kSegment == 0 && p.input_width <= kMaxWidth &&
            // rows start on block boundaries (scalar row offset into scales)
            p.input_width % (std::size_t{1} << p.block_shift) == 0 &&

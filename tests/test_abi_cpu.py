@@ -44,6 +44,11 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(fwd, 3, 11008, 4096, 64) == package.ALGORITHM_GEMV
     assert select(fwd, 4, 16384, 4096, 64) == package.ALGORITHM_GEMV
     assert select(fwd, 4, 16384 + 64, 4096, 64) == package.ALGORITHM_SKINNY
+    # one and two rows of up to 32768 weights: the same one-team form
+    assert select(fwd, 1, 28672, 8192, 64) == package.ALGORITHM_GEMV
+    assert select(fwd, 2, 32768, 1024, 64) == package.ALGORITHM_GEMV
+    assert select(fwd, 3, 28672, 8192, 64) == package.ALGORITHM_SKINNY
+    assert select(fwd, 1, 32768 + 64, 1024, 64) == package.ALGORITHM_SKINNY
     # prefill / training -> MFMA GEMM, both directions
     assert select(fwd, 2048, 4096, 11008, 64) == package.ALGORITHM_MFMA
     # small batches -> weights decoded straight into MFMA operands
