@@ -584,16 +584,21 @@ std::size_t held_rows(const LinearProblem& p) {
     return p.rows == 3 ? 4 : p.rows;
 }
 
-// A thread's register-resident slice of x is held_rows x segments x 16
-// values; beyond 8 x 16 it no longer fits, and a thread takes at most four
-// segments of a row.  Two teams of 256 threads per workgroup measured best;
-// rows too wide for that get one team of 512 (three and four rows of x from
-// 8192 weights per row on, one and two rows from 16384 to 32768).
-constexpr std::size_t kMaxHeldSegments = 8;
-constexpr std::size_t kMaxSegments = 4;
+// What a thread keeps in registers grows with both the x rows it holds (its
+// slice of x: held rows x segments x 16 values) and the segments it takes of a
+// weight row (the looked-up levels of two rows: 32 values per segment).  These
+// combinations fit the 256 registers without spills: one x row with up to four
+// segments, two with up to three, four with up to two.
+constexpr bool fits_registers(std::size_t held, std::size_t segments) {
+    return segments >= 1 && (held == 1   ? segments <= 4
+                             : held == 2 ? segments <= 3
+                                         : segments <= 2);
+}
+// Two teams of 256 threads per workgroup measured best; rows too wide for
+// that get one team of 512 (half the segments per thread): four rows of x
+// from 8192 weights per row on, two from 12288, one from 16384 to 32768.
 bool wide_team(const LinearProblem& p) {
-    return held_rows(p) * segments_per_thread(p, 256) > kMaxHeldSegments ||
-           segments_per_thread(p, 256) > kMaxSegments;
+    return !fits_registers(held_rows(p), segments_per_thread(p, 256));
 }
 
 // The weights of one launch: `count` problems that share activations, row
@@ -673,22 +678,35 @@ void launch_instance(const Launch& launch, hipStream_t stream) {
         batch_count, iterations, first.lora);
 }
 
+// One instance per (x rows, segments) pair that fits; the others are never
+// compiled.
+template <int kX, int kSegments, bool kDoubleQuantized, bool kGrouped,
+          bool kWide>
+void launch_fitting(const Launch& launch, hipStream_t stream) {
+    if constexpr (fits_registers(kX, kSegments)) {
+        launch_instance<kX, kSegments, kDoubleQuantized, kGrouped, kWide>(
+            launch, stream);
+    }
+}
+
 template <int kX, bool kDoubleQuantized, bool kGrouped>
 void launch_segments(const Launch& launch, hipStream_t stream) {
     const LinearProblem& p = launch.problems[0];
     if (wide_team(p)) {
-        // one 512-thread team per weight row: four x rows and a row wider
-        // than 8192 (two segments per thread), one or two x rows and a row
-        // wider than 16384 (three or four)
-        if constexpr (kX == 4) {
-            launch_instance<kX, 2, kDoubleQuantized, kGrouped, true>(launch,
-                                                                     stream);
-        } else if (segments_per_thread(p, 512) == 3) {
-            launch_instance<kX, 3, kDoubleQuantized, kGrouped, true>(launch,
-                                                                     stream);
-        } else {
-            launch_instance<kX, 4, kDoubleQuantized, kGrouped, true>(launch,
-                                                                     stream);
+        // one 512-thread team per weight row
+        switch (segments_per_thread(p, 512)) {
+        case 2:
+            launch_fitting<kX, 2, kDoubleQuantized, kGrouped, true>(launch,
+                                                                    stream);
+            break;
+        case 3:
+            launch_fitting<kX, 3, kDoubleQuantized, kGrouped, true>(launch,
+                                                                    stream);
+            break;
+        default:
+            launch_fitting<kX, 4, kDoubleQuantized, kGrouped, true>(launch,
+                                                                    stream);
+            break;
         }
         return;
     }
@@ -709,13 +727,16 @@ void launch_segments(const Launch& launch, hipStream_t stream) {
         launch_instance<kX, 1, kDoubleQuantized, kGrouped>(launch, stream);
         break;
     case 2:
-        launch_instance<kX, 2, kDoubleQuantized, kGrouped>(launch, stream);
+        launch_fitting<kX, 2, kDoubleQuantized, kGrouped, false>(launch,
+                                                                 stream);
         break;
     case 3:
-        launch_instance<kX, 3, kDoubleQuantized, kGrouped>(launch, stream);
+        launch_fitting<kX, 3, kDoubleQuantized, kGrouped, false>(launch,
+                                                                 stream);
         break;
     default:
-        launch_instance<kX, 4, kDoubleQuantized, kGrouped>(launch, stream);
+        launch_fitting<kX, 4, kDoubleQuantized, kGrouped, false>(launch,
+                                                                 stream);
         break;
     }
 }
@@ -742,14 +763,13 @@ void launch_encoding(const Launch& launch, hipStream_t stream) {
 
 bool gemv_forward_supports(const LinearProblem& p) {
     constexpr std::size_t kMaxWidth =
-        static_cast<std::size_t>(kSegment) * 512 * kMaxSegments;
+        static_cast<std::size_t>(kSegment) * 512 * 4;
     return p.rows >= 1 && p.rows <= kGemvMaxRows &&
-           // the register-resident x slice must fit, with two teams of 256
-           // threads or one team of 512
+           // the registers must hold a thread's share, with two teams of 256
+           // threads or one team of 512 (then at least two segments each)
            (!wide_team(p) ||
             (segments_per_thread(p, 512) >= 2 &&
-             held_rows(p) * segments_per_thread(p, 512) <=
-                 kMaxHeldSegments)) &&
+             fits_registers(held_rows(p), segments_per_thread(p, 512)))) &&
            p.input_width % kSegment == 0 && p.input_width <= kMaxWidth &&
            // rows start on block boundaries (scalar row offset into scales)
            p.input_width % (std::size_t{1} << p.block_shift) == 0 &&

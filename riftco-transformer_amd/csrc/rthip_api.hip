@@ -378,9 +378,36 @@ bool tail_split(const rthip::LinearProblem& problem, bool forward,
            (small_batch_family(split->family[1]) ||
             split->family[1] == RTHIP_NF4_ALGORITHM_GEMV);
 }
+// Two to four rows of x against weight rows too wide for the GEMV to hold
+// that many rows of x in registers (from 16384 weights on) run as two GEMV
+// launches of fewer rows where that covers them: the small-batch kernel, the
+// only other taker, needs 80 us for 8192 x 28672 where one row through the
+// GEMV takes 27.
+bool wide_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
+    if (problem.rows < 2 || problem.rows > rthip::kGemvMaxRows ||
+        select_forward(problem) == RTHIP_NF4_ALGORITHM_GEMV) {
+        return false;
+    }
+    for (std::size_t head = 2; head >= 1; --head) {
+        if (head >= problem.rows || problem.rows > 2 * head) {
+            continue;
+        }
+        split->count = 2;
+        split->part[0] = row_part(problem, 0, head, true);
+        split->part[1] = row_part(problem, head, problem.rows - head, true);
+        split->family[0] = select_forward(split->part[0]);
+        split->family[1] = select_forward(split->part[1]);
+        if (split->family[0] == RTHIP_NF4_ALGORITHM_GEMV &&
+            split->family[1] == RTHIP_NF4_ALGORITHM_GEMV) {
+            return true;
+        }
+    }
+    return false;
+}
 bool forward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
     return forward_small_split(problem, split) ||
-           tail_split(problem, true, split);
+           tail_split(problem, true, split) ||
+           wide_row_split(problem, split);
 }
 bool backward_row_split(const rthip::LinearProblem& problem, RowSplit* split) {
     return backward_small_split(problem, split) ||

@@ -43,11 +43,15 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(fwd, 2, 11008, 4096, 64) == package.ALGORITHM_GEMV
     assert select(fwd, 3, 11008, 4096, 64) == package.ALGORITHM_GEMV
     assert select(fwd, 4, 16384, 4096, 64) == package.ALGORITHM_GEMV
-    assert select(fwd, 4, 16384 + 64, 4096, 64) == package.ALGORITHM_SKINNY
-    # one and two rows of up to 32768 weights: the same one-team form
+    assert select(fwd, 5, 16384 + 64, 4096, 64) == package.ALGORITHM_SKINNY
+    # one row of up to 32768 weights, two of up to 24576: the same one-team
+    # form; more rows as two launches where two launches cover them
     assert select(fwd, 1, 28672, 8192, 64) == package.ALGORITHM_GEMV
+    assert select(fwd, 2, 24576, 1024, 64) == package.ALGORITHM_GEMV
     assert select(fwd, 2, 32768, 1024, 64) == package.ALGORITHM_GEMV
+    assert select(fwd, 4, 24576, 1024, 64) == package.ALGORITHM_GEMV
     assert select(fwd, 3, 28672, 8192, 64) == package.ALGORITHM_SKINNY
+    assert select(fwd, 5, 24576, 8192, 64) == package.ALGORITHM_SKINNY
     assert select(fwd, 1, 32768 + 64, 1024, 64) == package.ALGORITHM_SKINNY
     # prefill / training -> MFMA GEMM, both directions
     assert select(fwd, 2048, 4096, 11008, 64) == package.ALGORITHM_MFMA

@@ -338,25 +338,27 @@ def test_wide_rows_at_three_and_four_rows(gpu, package, library, oracle, out_w,
                     oracle_rows=2)
 
 
-@pytest.mark.parametrize("out_w,in_w,block,double_quantized", [
-    (8192 // 16, 28672, 64, False),  # a 70B feed-forward width, 3.5 segments
-    (130, 16384 + 64, 64, True),     # just past four segments per 256 threads
-    (65, 32768, 64, True),           # the widest row
+@pytest.mark.parametrize("out_w,in_w,block,double_quantized,gemv_rows", [
+    (8192 // 16, 28672, 64, False, (1, 2)),  # a 70B feed-forward width
+    (130, 16384 + 64, 64, True, (1, 2, 3, 4)),  # just past 4 x 256 segments
+    (200, 13824, 128, True, (1, 2, 3, 4)),   # a 13B feed-forward width
+    (65, 32768, 64, True, (1, 2)),           # the widest row
 ])
-def test_rows_wider_than_16384_at_one_and_two_rows(gpu, package, library,
-                                                    oracle, out_w, in_w,
-                                                    block, double_quantized):
-    """Rows of 16385...32768 weights with one or two x rows run the GEMV with
-    one 512-thread team per weight row (three or four segments per thread);
-    three and four x rows of such a width go to the small-batch kernel."""
+def test_rows_wider_than_12288(gpu, package, library, oracle, out_w, in_w,
+                               block, double_quantized, gemv_rows):
+    """Rows too wide for two 256-thread teams to hold their share in registers
+    run the GEMV with one 512-thread team per weight row: two x rows from
+    12289 weights on, one from 16385 to 32768.  Row counts the GEMV cannot
+    hold at such a width run as two launches of fewer rows where that covers
+    them (the family reported is still the GEMV), else through the
+    small-batch kernel."""
     weight = oracle.quantize(helpers.normal(87, (out_w, in_w), 0.02), block,
                              double_quantized, 256)
     bias = helpers.normal(88, (out_w,), 0.01)
-    assert library.select_algorithm(package.FORWARD, 3, in_w, out_w,
-                                    block) != package.ALGORITHM_GEMV
-    for rows in (1, 2):
-        assert library.select_algorithm(package.FORWARD, rows, in_w, out_w,
-                                        block) == package.ALGORITHM_GEMV
+    for rows in (1, 2, 3, 4):
+        assert (library.select_algorithm(package.FORWARD, rows, in_w, out_w,
+                                         block) == package.ALGORITHM_GEMV) == \
+            (rows in gemv_rows)
         x = helpers.normal(89 + rows, (rows, in_w), 1.0)
         dy = helpers.normal(90 + rows, (rows, out_w), 1.0e-2)
         check_layer(gpu, package, library, oracle, weight, x, dy, bias=bias,
