@@ -471,15 +471,18 @@ def bench_ragged(package, device, torch, steps):
 
 def bench_large_launches(package, device, torch, steps):
     """M = 1 launches that move more bytes than one projection: the lm_head of
-    the same model (32000 x 4096) and gate/up of two layers in one grouped
-    launch.  They show the rate the GEMV streams at once a launch's fixed cost
+    the same model (32000 x 4096), gate/up of two layers in one grouped
+    launch, and the feed-forward projections of a 70B model (117 MB each; the
+    second has rows of 28672 weights).  They show the rate the GEMV streams at once a launch's fixed cost
     (about 3 us) is spread over enough bytes."""
     library = package.load_library()
     results = []
-    x = torch.randn(1, 4096, device="cuda")
     cases = [("lm_head 32000x4096", [(32000, 4096)]),
-             ("4 x 11008x4096 in one launch", [(11008, 4096)] * 4)]
+             ("4 x 11008x4096 in one launch", [(11008, 4096)] * 4),
+             ("70B feed-forward 28672x8192", [(28672, 8192)]),
+             ("70B feed-forward 8192x28672", [(8192, 28672)])]
     for name, shapes in cases:
+        x = torch.randn(1, shapes[0][1], device="cuda")
         copies = 6  # 6 x >= 74 MB: beyond the last-level cache
         groups = [[synthetic_weight(package, torch, out_w, in_w, False,
                                     900 + 10 * copy + index)
