@@ -30,8 +30,9 @@ The same JSON line carries
                 tiles of the GEMM, 272 two and sixteen rows)
   ragged_shapes a shape only the shape-agnostic kernels take (4097 x 4095)
   large_launches
-                M = 1 launches of 74 and 101 MB (lm_head; four gate/up weights
-                in one grouped launch)
+                M = 1 launches of 74 to 117 MB (lm_head; four gate/up weights
+                in one grouped launch; the feed-forward projections of a 70B
+                model)
   practical_roof
                 a plain streaming read of the same sizes, one launch per
                 buffer, and an empty launch: what the device gives a kernel
