@@ -102,7 +102,9 @@ def test_select_algorithm_is_pure_host_logic(package, library):
     assert select(bwd, 97, 4096, 11008, 64) == package.ALGORITHM_SKINNY
     assert select(bwd, 192, 4096, 11008, 64) == package.ALGORITHM_SKINNY
     assert select(bwd, 193, 4096, 11008, 64) == package.ALGORITHM_MFMA
-    assert select(bwd, 65, 11008, 4096, 64) == package.ALGORITHM_MFMA
+    # (dx much wider than dy: only while the rest fits the streaming kernel)
+    assert select(bwd, 68, 11008, 4096, 64) == package.ALGORITHM_SKINNY
+    assert select(bwd, 69, 11008, 4096, 64) == package.ALGORITHM_MFMA
     assert select(bwd, 16, 36, 768, 32) == package.ALGORITHM_GENERIC
     # the reference's edge layout -> shape-agnostic kernels
     assert select(fwd, 2, 33, 33, 32) == package.ALGORITHM_GENERIC

@@ -503,10 +503,11 @@ def test_small_batch_input_backward(gpu, package, library, oracle, out_w, in_w,
     assert library.select_algorithm(
         package.INPUT_BACKWARD, 97 if out_w < 2 * in_w else 193, in_w, out_w,
         block) != package.ALGORITHM_SKINNY
-    rows = 80
-    x = helpers.normal(84 + rows, (rows, in_w), 1.0)
-    dy = helpers.normal(85 + rows, (rows, out_w), 1.0e-2)
-    check_layer(gpu, package, library, oracle, weight, x, dy, oracle_rows=2)
+    for rows in (66, 80):
+        x = helpers.normal(84 + rows, (rows, in_w), 1.0)
+        dy = helpers.normal(85 + rows, (rows, out_w), 1.0e-2)
+        check_layer(gpu, package, library, oracle, weight, x, dy,
+                    oracle_rows=2)
 
 
 @pytest.mark.parametrize("out_w,in_w,block,second,double_quantized", [
