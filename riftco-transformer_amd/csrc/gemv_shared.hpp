@@ -70,6 +70,59 @@ __device__ __forceinline__ float sum_over_rows(float value) {
     return value + twin;
 }
 
+template <int kXor, int kHalf, int kValues>
+__device__ __forceinline__ void transposed_step(float (&values)[kValues],
+                                                unsigned lane) {
+    if constexpr (kHalf >= 1) {
+        // Lanes with bit kXor set keep the upper half of the values and hand
+        // the lower half to their partner, and vice versa.
+        const bool upper = (lane & kXor) != 0;
+#pragma unroll
+        for (int j = 0; j < kHalf; ++j) {
+            float low = values[j];
+            float high = values[j + kHalf];
+            // Keep the two operands as plain registers: without this the
+            // selects below are rewritten into a dynamically indexed read of
+            // `values`, which costs a compare/select chain over the array.
+            asm volatile("" : "+v"(low), "+v"(high));
+            const float keep = upper ? high : low;
+            const float send = upper ? low : high;
+            values[j] = keep + dpp_xor<kXor>(send);
+        }
+    } else {
+        values[0] += dpp_xor<kXor>(values[0]);
+    }
+}
+
+// Sum over each 16-lane DPP row of kValues per-lane values.  On return every
+// lane holds the row total of value `slot_of_lane(lane)`.
+template <int kValues>
+__device__ __forceinline__ float transposed_row_sum(float (&values)[kValues],
+                                                    unsigned lane) {
+    static_assert((kValues & (kValues - 1)) == 0 && kValues <= kRowLanes);
+    transposed_step<1, kValues / 2>(values, lane);
+    transposed_step<2, kValues / 4>(values, lane);
+    transposed_step<4, kValues / 8>(values, lane);
+    transposed_step<8, kValues / 16>(values, lane);
+    return values[0];
+}
+
+// Which value a lane ends up holding after transposed_row_sum: lane bit s
+// selected the upper half at step s.
+template <int kValues>
+__device__ __forceinline__ unsigned slot_of_lane(unsigned lane) {
+    unsigned slot = 0;
+    unsigned bit = 1;
+#pragma unroll
+    for (int half = kValues / 2; half >= 1; half /= 2) {
+        if (lane & bit) {
+            slot += half;
+        }
+        bit *= 2;
+    }
+    return slot;
+}
+
 // One weight of a launch.  A launch covers up to kGemvGroupMax weights that
 // are applied to the same x (the q/k/v or gate/up projections of a layer):
 // their row batches are numbered one member after the other, and member m owns

@@ -57,6 +57,14 @@ constexpr std::size_t kGemvGroupMax = 4;
 bool gemv_group_supports(const LinearProblem* problems, std::size_t count);
 void launch_gemv_group(const LinearProblem* problems, std::size_t count,
                        hipStream_t stream);
+// nf4_gemv1.hip -- the same product for ONE row of x (the decode step of a
+// model), built around the launch's start and the bytes in flight: `count`
+// weights that gemv_group_supports accepts, each of which
+// gemv1_forward_supports accepts.  launch_gemv_forward / launch_gemv_group
+// route here by themselves.
+bool gemv1_forward_supports(const LinearProblem& problem);
+void launch_gemv1_forward(const LinearProblem* problems, std::size_t count,
+                          hipStream_t stream);
 
 // workspace.hip -- scratch memory shared by the kernels that pass partial
 // results between workgroups; one fixed-size buffer per (device, stream),

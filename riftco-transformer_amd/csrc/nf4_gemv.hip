@@ -84,60 +84,6 @@ constexpr unsigned kParkedValues = 512;
 #define RTHIP_GEMV_DEPTH 2
 #endif
 
-template <int kXor, int kHalf, int kValues>
-__device__ __forceinline__ void transposed_step(float (&values)[kValues],
-                                                unsigned lane) {
-    if constexpr (kHalf >= 1) {
-        // Lanes with bit kXor set keep the upper half of the values and hand
-        // the lower half to their partner, and vice versa.
-        const bool upper = (lane & kXor) != 0;
-#pragma unroll
-        for (int j = 0; j < kHalf; ++j) {
-            float low = values[j];
-            float high = values[j + kHalf];
-            // Keep the two operands as plain registers: without this the
-            // selects below are rewritten into a dynamically indexed read of
-            // `values`, which costs a compare/select chain over the array.
-            asm volatile("" : "+v"(low), "+v"(high));
-            const float keep = upper ? high : low;
-            const float send = upper ? low : high;
-            values[j] = keep + dpp_xor<kXor>(send);
-        }
-    } else {
-        values[0] += dpp_xor<kXor>(values[0]);
-    }
-}
-
-// Sum over each 16-lane DPP row of kValues per-lane values.  On return every
-// lane holds the row total of value `slot_of_lane(lane)`.
-template <int kValues>
-__device__ __forceinline__ float transposed_row_sum(float (&values)[kValues],
-                                                    unsigned lane) {
-    static_assert((kValues & (kValues - 1)) == 0 && kValues <= kRowLanes);
-    transposed_step<1, kValues / 2>(values, lane);
-    transposed_step<2, kValues / 4>(values, lane);
-    transposed_step<4, kValues / 8>(values, lane);
-    transposed_step<8, kValues / 16>(values, lane);
-    return values[0];
-}
-
-// Which value a lane ends up holding after transposed_row_sum: lane bit s
-// selected the upper half at step s.
-template <int kValues>
-__device__ __forceinline__ unsigned slot_of_lane(unsigned lane) {
-    unsigned slot = 0;
-    unsigned bit = 1;
-#pragma unroll
-    for (int half = kValues / 2; half >= 1; half /= 2) {
-        if (lane & bit) {
-            slot += half;
-        }
-        bit *= 2;
-    }
-    return slot;
-}
-
-
 // Shared scale loads per batch (nested scale encoding): a load covers 64
 // (row, block) pairs and a wavefront's part of a row spans at most 32 blocks
 // (block size 32), so two-row batches need one load and four-row batches two.
@@ -781,6 +727,10 @@ bool gemv_forward_supports(const LinearProblem& p) {
 }
 
 void launch_gemv_forward(const LinearProblem& p, hipStream_t stream) {
+    if (gemv1_forward_supports(p)) {  // one row of x: the kernel of its own
+        launch_gemv1_forward(&p, 1, stream);
+        return;
+    }
     launch_encoding<false>(Launch{&p, 1}, stream);
 }
 
@@ -809,8 +759,29 @@ void launch_gemv_group(const LinearProblem* problems, std::size_t count,
                        hipStream_t stream) {
     if (count == 1) {
         launch_gemv_forward(problems[0], stream);
-    } else {
-        launch_encoding<true>(Launch{problems, count}, stream);
+        return;
+    }
+    // Members that the one-row kernel takes go to it together, the others
+    // stay with this file's kernel: either way a member's output is what its
+    // launch alone writes, bit for bit.
+    LinearProblem one_row[kGemvGroupMax];
+    LinearProblem other[kGemvGroupMax];
+    std::size_t one_row_count = 0;
+    std::size_t other_count = 0;
+    for (std::size_t m = 0; m < count; ++m) {
+        if (gemv1_forward_supports(problems[m])) {
+            one_row[one_row_count++] = problems[m];
+        } else {
+            other[other_count++] = problems[m];
+        }
+    }
+    if (one_row_count != 0) {
+        launch_gemv1_forward(one_row, one_row_count, stream);
+    }
+    if (other_count == 1) {
+        launch_encoding<false>(Launch{other, 1}, stream);
+    } else if (other_count > 1) {
+        launch_encoding<true>(Launch{other, other_count}, stream);
     }
 }
 
