@@ -63,12 +63,11 @@ __device__ __forceinline__ void load_codebook_to_lds(float* table) {
 // the add into one fused multiply-add, and plain operators are used because
 // only code written inside this scope is covered by it.  Division of fp32 is
 // correctly rounded in HIP by default.
-__device__ __forceinline__ float decode_double_quantized_scale(
-    std::uint8_t scale_code, float second_level, float offset
+// The part after the division: factor = (float)(code - 128) / 127.0F.
+__device__ __forceinline__ float double_quantized_scale_from_factor(
+    float factor, float second_level, float offset
 ) {
 #pragma clang fp contract(off)
-    const int centered = static_cast<int>(scale_code) - 128;
-    const float factor = static_cast<float>(centered) / 127.0F;
     const float delta = second_level * factor;
     constexpr float kMaxFinite = 0x1.fffffep+127F;
     if (delta > 0.0F && offset > kMaxFinite - delta) {
@@ -76,6 +75,15 @@ __device__ __forceinline__ float decode_double_quantized_scale(
     }
     const float reconstructed = offset + delta;
     return reconstructed > 0.0F ? reconstructed : 0.0F;
+}
+
+__device__ __forceinline__ float decode_double_quantized_scale(
+    std::uint8_t scale_code, float second_level, float offset
+) {
+#pragma clang fp contract(off)
+    const int centered = static_cast<int>(scale_code) - 128;
+    const float factor = static_cast<float>(centered) / 127.0F;
+    return double_quantized_scale_from_factor(factor, second_level, offset);
 }
 
 template <bool kDoubleQuantized>

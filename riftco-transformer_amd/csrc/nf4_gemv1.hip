@@ -33,12 +33,16 @@
 // Work split.  One persistent workgroup per CU; batch b of kRows consecutive
 // weight rows goes to workgroup b % gridDim.x.  Requests: batch 0, then x,
 // then -- after the table build -- the further batches of the ring; batch
-// i + kDepth - 1 is requested when batch i is about to be multiplied.  The
-// memory system serves a burst from all CUs at once badly (the first bytes of
-// a launch that requests 64 KB per CU up front arrive later than the LAST
-// bytes of one that requests 16 KB at a time), so the ring is shallow.  The
-// step exists in two compiled copies, with and without a batch left to
-// request: the compiler's wait counts are exact only along straight-line code.
+// i + kDepth - 1 is requested when batch i is about to be multiplied.  A
+// compute unit keeps about 32 KB of loads in flight (the size of its vector
+// L1: beyond that the issue of further loads blocks), and the memory system
+// serves a burst from all CUs at once badly -- the first bytes of a launch
+// that requests 64 KB per CU up front arrive later than the LAST bytes of one
+// that requests 16 KB at a time -- so a batch is 9 to 25 KB per CU and the ring
+// is two deep.  The step exists in two compiled copies, with and without a
+// batch left to request, and nothing on the vector ALU stands between a
+// step's start and its loads (see load_batch): the compiler's wait counts are
+// exact only along straight-line code.
 //
 // Decode is the (low nibble, high nibble) pair table in LDS of nf4_gemv.hip
 // (which serves two to four rows of x and block sizes other than 64).  Row
@@ -107,8 +111,11 @@ struct RowBatch {
     float offset;  // of the member the batch belongs to (uniform)
 };
 
+// kWholeGroups (nested scales): every batch starts on a second-level group
+// boundary, so a lane's second-level scale sits at a fixed offset from the
+// batch's first one.
 template <int kSegments, int kRows, int kDepth, int kLook,
-          bool kDoubleQuantized, int kMembers>
+          bool kDoubleQuantized, bool kWholeGroups, int kMembers>
 __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
     // The first 14 dwords are preloaded into scalar registers when the
     // wavefront is created (the file is compiled with
@@ -128,6 +135,11 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
     static_assert(kRows == 8 || kRows == 4 || kRows == 2);
     __shared__ __attribute__((aligned(256))) char table[kPairTableBytes];
     __shared__ float partial[kMaxIterations][kWaves][kRows];
+    // Nested scales: (code - 128) / 127 for every scale code, so that a
+    // scale costs its lane one LDS read, a multiply and an add instead of a
+    // correctly rounded division (the same quotients, hence the same scales
+    // bit for bit as decode_double_quantized_scale).
+    __shared__ float factor[kDoubleQuantized ? 256 : 1];
 
     const unsigned thread = threadIdx.x;
     const unsigned lane = thread % kWave;
@@ -151,6 +163,13 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
         code_offset[j] = kept * (kSegment / 2);
         scale_offset[j] = (my_row * row_blocks + kept / kBlockLanes) *
                           (kDoubleQuantized ? 1U : 4U);
+    }
+    // (nested scales, whole groups) of this lane's second-level scale, from
+    // the batch's first one, in bytes
+    unsigned second_offset[kSegments];
+#pragma unroll
+    for (int j = 0; j < kSegments; ++j) {
+        second_offset[j] = (scale_offset[j] >> second_level_shift) * 4;
     }
 
     // The member whose batches are being REQUESTED.  A workgroup's batch
@@ -221,7 +240,21 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
                     primary_buffer, scale_offset[j], 0, 0);
             }
         }
-        if constexpr (kDoubleQuantized) {
+        if constexpr (kDoubleQuantized && kWholeGroups) {
+            const unsigned second_start =
+                min((first_block >> second_level_shift) * 4,
+                    member.secondary_bytes);
+            const __amdgpu_buffer_rsrc_t secondary_buffer = make_buffer(
+                reinterpret_cast<const char*>(member.secondary_scales) +
+                    second_start,
+                member.secondary_bytes - second_start);
+#pragma unroll
+            for (int j = 0; j < kSegments; ++j) {
+                batch.scales[j] = __builtin_bit_cast(
+                    float, __builtin_amdgcn_raw_buffer_load_b32(
+                               secondary_buffer, second_offset[j], 0, 0));
+            }
+        } else if constexpr (kDoubleQuantized) {
             // The second-level scale's index needs a shift of the block
             // number, a vector instruction: its result is kept alive past
             // the load, so it cannot share a register with the load's
@@ -277,6 +310,12 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
     }
 
     build_pair_table<kThreads>(table);
+    if constexpr (kDoubleQuantized) {
+        if (thread < 256) {
+            factor[thread] =
+                static_cast<float>(static_cast<int>(thread) - 128) / 127.0F;
+        }
+    }
 
 #pragma unroll
     for (int d = 1; d < kDepth - 1; ++d) {
@@ -350,8 +389,8 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
             transposed_step<4, kRows / 8>(acc[j], lane);
             float scale = current.scales[j];
             if constexpr (kDoubleQuantized) {
-                scale = decode_double_quantized_scale(
-                    static_cast<std::uint8_t>(current.scale_codes[j]), scale,
+                scale = double_quantized_scale_from_factor(
+                    factor[current.scale_codes[j] & 0xFFU], scale,
                     current.offset);
             }
             total += acc[j][0] * scale;
@@ -363,6 +402,9 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
         }
     };
 
+    // The ring is walked with static slot numbers.  The last kDepth - 1 steps
+    // have nothing left to request; they run the copy of the step that issues
+    // no loads.
     for (unsigned iteration = 0; iteration < iterations;
          iteration += kDepth) {
 #pragma unroll
@@ -487,14 +529,27 @@ void launch_instance(const LinearProblem* problems, std::size_t count,
     }
     const unsigned iterations = (batch_count + blocks - 1) / blocks;
     const OneRowSource& head = sources[0];
-    gemv1_forward_kernel<kSegments, kRows, kDepth, kLook, kDoubleQuantized,
-                         kMembers>
-        <<<blocks, kThreads, 0, stream>>>(
-            first.activations, head.codes, head.primary_scales,
-            static_cast<unsigned>(first.input_width), head.code_bytes,
-            head.primary_bytes, iterations, head.secondary_scales,
-            head.secondary_bytes, head.offset,
-            first.weight.second_level_shift, batch_count, rest, first.lora);
+    const auto launch = [&](auto whole_groups) {
+        gemv1_forward_kernel<kSegments, kRows, kDepth, kLook, kDoubleQuantized,
+                             decltype(whole_groups)::value, kMembers>
+            <<<blocks, kThreads, 0, stream>>>(
+                first.activations, head.codes, head.primary_scales,
+                static_cast<unsigned>(first.input_width), head.code_bytes,
+                head.primary_bytes, iterations, head.secondary_scales,
+                head.secondary_bytes, head.offset,
+                first.weight.second_level_shift, batch_count, rest,
+                first.lora);
+    };
+    if constexpr (kDoubleQuantized) {
+        const std::size_t batch_blocks =
+            kRows * (first.input_width >> kBlockShift);
+        if (batch_blocks % (std::size_t{1} << first.weight.second_level_shift)
+            == 0) {
+            launch(std::true_type{});
+            return;
+        }
+    }
+    launch(std::false_type{});
 }
 
 template <bool kDoubleQuantized, int kMembers>
