@@ -380,7 +380,8 @@ rthip_status rthip_nf4_dequantize(
  *   secondary_scales    float [ceil(blocks / second_level_block)]
  *   fp32_scale_scratch  float [blocks]: receives the plain block scales
  *   host_offset         HOST pointer that receives the offset
- * Unlike the compute entry points this one returns after the work is done:
+ * Unlike the compute entry points this one returns after the work is done
+ * (it waits for `stream`, so it cannot be recorded into a graph):
  * a non-finite source value is reported as RTHIP_INVALID_ARGUMENT ("NF4 source
  * values must be finite") and a non-finite scale mean as RTHIP_OVERFLOW, the
  * two exceptions the reference throws (:189-191, :224-227).
@@ -401,7 +402,8 @@ rthip_status rthip_nf4_quantize(
  * check; this call reads
  *   codes [ceil(element_count / 2)], primary_scales [blocks] (float or uint8),
  *   secondary_scales [ceil(blocks / second_level_block)] (nested only)
- * and returns, after the work is done, RTHIP_OK or RTHIP_INVALID_ARGUMENT
+ * and returns, after the work is done (it waits for `stream`, so it cannot
+ * be recorded into a graph), RTHIP_OK or RTHIP_INVALID_ARGUMENT
  * with the message of the exception the reference would throw first:
  * a non-zero unused high nibble, a negative or non-finite offset,
  * second-level scale or decoded block scale, or a block with an fp32 scale of
@@ -431,7 +433,12 @@ rthip_status rthip_probe_empty_launch(void* stream);
  * allocated by the first call on a stream that needs one): the buffer of
  * `stream` on the current device, or of every stream when every_stream != 0.
  * Waits for the device to finish with them; a later call allocates afresh.
- * No counterpart in the reference (its backends allocate per call).
+ * A graph that was captured on such a stream keeps the address of the buffer
+ * it was recorded with: do not release while such a graph may still be
+ * replayed.  With every_stream != 0 the call also unbinds the static array of
+ * rthip_nf4_linear_input_backward_no_alloc from its stream (after that stream
+ * has finished).  No counterpart in the reference (its backends allocate per
+ * call).
  */
 rthip_status rthip_release_workspaces(void* stream, int32_t every_stream);
 
@@ -448,9 +455,15 @@ rthip_status rthip_release_workspaces(void* stream, int32_t every_stream);
  * partial sums -- chunks x rows x input_width x 4 bytes, chunks <= 16 --
  * exceed that size is refused with RTHIP_UNSUPPORTED and a message that
  * names both sizes.  It calls no hipMalloc, hipFree or allocating library
- * routine.  Every call on a GPU shares that GPU's array: calls that overlap
- * on one GPU (two streams, or two graphs replayed at once) race; calls on
- * one stream are ordered and safe.
+ * routine.  Every call on a GPU shares that GPU's array, and calls that
+ * overlap on the GPU would race on it, so the array is bound to the stream of
+ * the first call on that GPU: calls on that stream, from any number of host
+ * threads, are ordered and safe (a thread holds the array until both of its
+ * launches are enqueued); a call on ANOTHER stream is refused with
+ * RTHIP_UNSUPPORTED until rthip_release_workspaces(stream, 1) has unbound the
+ * array.  What the library cannot see stays the caller's to avoid: two graphs
+ * that were captured on the bound stream and are replayed at the same time on
+ * different streams.
  */
 #define RTHIP_NO_ALLOC_SCRATCH_BYTES (24u << 20)
 rthip_status rthip_nf4_linear_input_backward_no_alloc(

@@ -95,7 +95,7 @@ bool environment_flag(const char* name) noexcept {
     return value != nullptr && std::strcmp(value, "1") == 0;
 }
 
-// Decode-sized forwards that RIFTCO_TRANSFORMER_HIP_MERGE=1 holds back (see
+// Decode-sized forwards that are held back to be merged (see
 // PendingForwards below) name device memory by address, so they have to be
 // launched before any of that memory changes hands or is looked at.
 void launch_pending_forwards();
@@ -274,15 +274,21 @@ private:
 };
 
 // The reference contract is that an adapter has finished writing its output
-// when it returns (docs/BACKENDS_AND_PYTHON.md:168), and that is the default
-// here: every launch is followed by a synchronisation.  Host code can only
-// see a hip tensor through data(), which copies from the device with a call
-// that itself waits for the default stream, so the synchronisation per
-// operation is not needed for correctness; RIFTCO_TRANSFORMER_HIP_ASYNC=1
-// drops it, and operations then queue behind each other on the device.
-// (Errors of a queued kernel surface at the next synchronising call.)
+// when it returns (docs/BACKENDS_AND_PYTHON.md:168).  Host code can only see
+// a hip tensor through data(), which copies from the device with a call that
+// itself waits for the default stream, so a synchronisation per operation is
+// not needed for correctness, and by default there is none: operations queue
+// behind each other on the device, and decode-sized forwards that share their
+// input are merged (below).  RIFTCO_TRANSFORMER_HIP_MERGE=0 restores one
+// launch per call, each followed by a synchronisation (unless
+// RIFTCO_TRANSFORMER_HIP_ASYNC=1 keeps the queued execution).  Errors of a
+// queued kernel surface at the next synchronising call.
 bool merge_requested() noexcept {
-    static const bool merge = environment_flag("RIFTCO_TRANSFORMER_HIP_MERGE");
+    // on unless RIFTCO_TRANSFORMER_HIP_MERGE=0
+    static const bool merge = [] {
+        const char* value = std::getenv("RIFTCO_TRANSFORMER_HIP_MERGE");
+        return value == nullptr || std::strcmp(value, "0") != 0;
+    }();
     return merge;
 }
 
@@ -294,11 +300,12 @@ void finish_operation(const HipRuntime& runtime, std::string_view operation) {
     }
 }
 
-// RIFTCO_TRANSFORMER_HIP_MERGE=1 (which implies the queued execution of
-// RIFTCO_TRANSFORMER_HIP_ASYNC=1).  A decoder calls the query, key and value
+// Merged forwards (the default; RIFTCO_TRANSFORMER_HIP_MERGE=0 turns them
+// off), which imply the queued execution of RIFTCO_TRANSFORMER_HIP_ASYNC=1.
+// A decoder calls the query, key and value
 // projections -- and gate and up -- one after the other on the same input
 // (src/model/decoder_only_transformer.cpp:406-419), each through
-// quantized_linear_forward.  At one to four rows a launch costs about as much
+// quantized_linear_forward.  At up to 128 rows a launch costs about as much
 // as the bytes it reads, so consecutive forwards that share their input are
 // held back here and go out together through rthip_nf4_linear_forward_group,
 // whose outputs are bit for bit those of separate launches.
@@ -312,7 +319,8 @@ void finish_operation(const HipRuntime& runtime, std::string_view operation) {
 // An error of a held-back launch is reported by the call that launches it.
 class PendingForwards final {
 public:
-    static constexpr std::size_t kMaximumRows = 4;  // the decode kernel's range
+    // the range of the kernels that take several weights per launch
+    static constexpr std::size_t kMaximumRows = 128;
     static constexpr std::size_t kCapacity = 4;     // weights per launch
 
     struct Shape {

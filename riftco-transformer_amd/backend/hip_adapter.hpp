@@ -121,14 +121,15 @@ struct QuantizedLinearAdapterBackwardRequest {
 void hip_quantized_linear_adapter_backward(
     const QuantizedLinearAdapterBackwardRequest& request);
 
-// RIFTCO_TRANSFORMER_HIP_MERGE=1 gives callers that were NOT changed the same
-// launches: quantized_linear_forward calls of one to four rows that follow
-// each other on the same input are held back and launched together (at most
-// four weights per launch) as soon as a call arrives that does not belong to
-// them, another operation of the adapter runs, host code reads a tensor, or a
-// device buffer is released.  It implies RIFTCO_TRANSFORMER_HIP_ASYNC=1.
+// Callers that were NOT changed get the same launches: quantized_linear_forward
+// calls of up to 128 rows that follow each other on the same input are held
+// back and launched together (at most four weights per launch) as soon as a
+// call arrives that does not belong to them, another operation of the adapter
+// runs, host code reads a tensor, or a device buffer is released.  This is
+// the default and implies the queued execution of
+// RIFTCO_TRANSFORMER_HIP_ASYNC=1; RIFTCO_TRANSFORMER_HIP_MERGE=0 turns it off.
 // requests: forwards that went through the merge; launches: kernel launches
-// they became.  Both stay zero while the option is off.
+// they became.  Both stay zero while merging is off.
 struct HipForwardMergeStatistics {
     std::uint64_t requests = 0;
     std::uint64_t launches = 0;

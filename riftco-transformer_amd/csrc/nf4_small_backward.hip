@@ -434,6 +434,12 @@ bool small_input_backward_supports(const LinearProblem& p) {
            // bit 31 of a byte offset means "rejected"
            p.rows * p.output_width * sizeof(float) < (1ULL << 31) &&
            p.rows * p.input_width * sizeof(float) < (1ULL << 32) &&
+           // with an adapter term the partial sums always pass through the
+           // workspace, even where the weight rows are a single chunk
+           (p.lora.reduced == nullptr ||
+            p.rows * p.input_width * sizeof(float) <=
+                (p.scratch != nullptr ? p.scratch_bytes
+                                      : kStreamWorkspaceBytes)) &&
            reinterpret_cast<std::uintptr_t>(p.weight.codes) % 4 == 0 &&
            reinterpret_cast<std::uintptr_t>(p.activations) % 16 == 0 &&
            reinterpret_cast<std::uintptr_t>(p.result) % 4 == 0;

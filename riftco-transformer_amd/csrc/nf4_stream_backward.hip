@@ -422,6 +422,10 @@ bool stream_input_backward_supports(const LinearProblem& p) {
            p.output_width * p.input_width < (1ULL << 32) &&
            p.rows * p.output_width * sizeof(float) < (1ULL << 31) &&
            p.rows * p.input_width * sizeof(float) < (1ULL << 31) &&
+           // with an adapter term the partial sums always pass through the
+           // stream workspace, even where the weight is a single range
+           (p.lora.reduced == nullptr ||
+            p.rows * p.input_width * sizeof(float) <= kStreamWorkspaceBytes) &&
            reinterpret_cast<std::uintptr_t>(p.weight.codes) % 8 == 0 &&
            reinterpret_cast<std::uintptr_t>(p.activations) % 16 == 0 &&
            reinterpret_cast<std::uintptr_t>(p.result) % 4 == 0;

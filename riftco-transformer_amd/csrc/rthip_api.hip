@@ -430,21 +430,40 @@ static __device__ __align__(256) float
 
 constexpr int kMaxScratchDevices = 64;
 
-// The device address of `scratch` on the current device (looked up once per
-// device, with that device current).
-rthip_status static_scratch(float** out) {
-    static std::mutex guard;
-    static float* address[kMaxScratchDevices] = {};
+// The array of one device: its address there (looked up once, with that
+// device current), the stream its users are bound to, and the exclusive right
+// to enqueue launches that use it.
+struct StaticScratch {
+    std::mutex busy;
+    float* address = nullptr;
+    bool bound = false;
+    hipStream_t stream = nullptr;
+};
+StaticScratch* static_scratch_of_device(int device) {
+    static StaticScratch all[kMaxScratchDevices];
+    return device >= 0 && device < kMaxScratchDevices ? &all[device] : nullptr;
+}
+
+// Leases the current device's array for launches on `stream`; the caller
+// holds `lock` until its last launch is enqueued, so that two threads cannot
+// interleave their partial-sum and sum launches.  The array is bound to the
+// first stream that uses it: launches on one stream are ordered, launches on
+// two are not, and nothing here could wait for the other stream without a
+// call that may not be made under graph capture.  A call on another stream
+// is refused until rthip_release_workspaces has unbound the array.
+rthip_status lease_static_scratch(hipStream_t stream, float** out,
+                                  std::unique_lock<std::mutex>* lock) {
     int device = 0;
     if (const hipError_t error = hipGetDevice(&device); error != hipSuccess) {
         return from_hip(error, "current device query");
     }
-    if (device < 0 || device >= kMaxScratchDevices) {
+    StaticScratch* const entry = static_scratch_of_device(device);
+    if (entry == nullptr) {
         return fail(RTHIP_UNSUPPORTED, "device ordinal %d is out of range",
                     device);
     }
-    const std::lock_guard<std::mutex> lock(guard);
-    if (address[device] == nullptr) {
+    std::unique_lock<std::mutex> held(entry->busy);
+    if (entry->address == nullptr) {
         float* found = nullptr;
         if (const hipError_t error = hipGetSymbolAddress(
                 reinterpret_cast<void**>(&found), HIP_SYMBOL(scratch));
@@ -455,9 +474,40 @@ rthip_status static_scratch(float** out) {
             return fail(RTHIP_RUNTIME_ERROR,
                         "static scratch address lookup returned null");
         }
-        address[device] = found;
+        entry->address = found;
     }
-    *out = address[device];
+    if (entry->bound && entry->stream != stream) {
+        return fail(RTHIP_UNSUPPORTED,
+                    "the device's static scratch array is in use by another "
+                    "stream: calls that share it must be on one stream "
+                    "(rthip_release_workspaces unbinds it)");
+    }
+    entry->bound = true;
+    entry->stream = stream;
+    *out = entry->address;
+    *lock = std::move(held);
+    return RTHIP_OK;
+}
+
+// After the device has finished with the current device's array, lets the
+// next caller bind it to a stream of its choice.
+rthip_status unbind_static_scratch() {
+    int device = 0;
+    if (const hipError_t error = hipGetDevice(&device); error != hipSuccess) {
+        return from_hip(error, "current device query");
+    }
+    StaticScratch* const entry = static_scratch_of_device(device);
+    if (entry == nullptr) {
+        return RTHIP_OK;
+    }
+    const std::lock_guard<std::mutex> held(entry->busy);
+    if (entry->bound) {
+        if (const hipError_t error = hipStreamSynchronize(entry->stream);
+            error != hipSuccess) {
+            return from_hip(error, "static scratch release");
+        }
+        entry->bound = false;
+    }
     return RTHIP_OK;
 }
 
@@ -695,8 +745,9 @@ rthip_status linear_forward_common(
         if (!rthip::gemv_forward_supports(problem)) {
             return fail(RTHIP_UNSUPPORTED,
                         "the GEMV family needs rows <= %zu, a row width that "
-                        "is a multiple of 16 and at most 16384, and aligned "
-                        "pointers",
+                        "is a multiple of 16 and of the block size and at "
+                        "most 32768 (one row of x), 24576 (two) or 16384 "
+                        "(three and four), and aligned pointers",
                         rthip::kGemvMaxRows);
         }
         rthip::launch_gemv_forward(problem, hip_stream);
@@ -1392,7 +1443,9 @@ rthip_status rthip_nf4_linear_input_backward_no_alloc(
         return status;
     }
     float* partial_sums = nullptr;
-    if (const rthip_status status = static_scratch(&partial_sums);
+    std::unique_lock<std::mutex> lease;  // until both launches are enqueued
+    if (const rthip_status status = lease_static_scratch(
+            static_cast<hipStream_t>(stream), &partial_sums, &lease);
         status != RTHIP_OK) {
         return status;
     }
@@ -1430,6 +1483,12 @@ rthip_status rthip_probe_empty_launch(void* stream) {
 rthip_status rthip_release_workspaces(void* stream, int32_t every_stream) {
     if (const rthip_status status = require_device(); status != RTHIP_OK) {
         return status;
+    }
+    if (every_stream != 0) {
+        if (const rthip_status status = unbind_static_scratch();
+            status != RTHIP_OK) {
+            return status;
+        }
     }
     return from_hip(
         rthip::release_stream_workspaces(static_cast<hipStream_t>(stream),
@@ -1522,8 +1581,8 @@ rthip_status rthip_nf4_quantize(
     }
     const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
     // [0]: status bits, [1]: the offset (a float): the first status word of
-    // the stream workspace, cleared by a kernel (no allocation per call, and
-    // no memset node if the stream is being captured).
+    // the stream workspace, cleared by a kernel (no allocation per call).
+    // The call waits for the stream below, so it cannot be captured.
     rthip::WorkspaceLease lease;
     if (const hipError_t error =
             rthip::lease_stream_workspace(hip_stream, &lease);

@@ -55,6 +55,9 @@ hipError_t lease_stream_workspace(hipStream_t stream, WorkspaceLease* lease) {
     Registry& all = registry();
     Workspace* workspace = nullptr;
     {
+        // `busy` is taken while `guard` is still held (the order in which
+        // release_stream_workspaces takes them): a release that runs between
+        // the lookup and the lease cannot free the buffer under the caller.
         const std::pair<int, hipStream_t> key(device, stream);
         const std::lock_guard<std::mutex> lock(all.guard);
         const auto found = all.buffers.find(key);
@@ -84,8 +87,8 @@ hipError_t lease_stream_workspace(hipStream_t stream, WorkspaceLease* lease) {
                 return restored;
             }
         }
+        lease->lock_ = std::unique_lock<std::mutex>(workspace->busy);
     }
-    lease->lock_ = std::unique_lock<std::mutex>(workspace->busy);
     lease->data_ = workspace->data;
     return hipSuccess;
 }

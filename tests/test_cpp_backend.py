@@ -47,8 +47,9 @@ def test_adapter_on_the_host_only_runtime():
     {"RIFTCO_TRANSFORMER_HIP_POOL": "0"},
     {"RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
     {"RIFTCO_TRANSFORMER_HIP_POOL": "0", "RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
-    {"RIFTCO_TRANSFORMER_HIP_MERGE": "1"},
-    {"RIFTCO_TRANSFORMER_HIP_POOL": "0", "RIFTCO_TRANSFORMER_HIP_MERGE": "1"},
+    {"RIFTCO_TRANSFORMER_HIP_MERGE": "0"},
+    {"RIFTCO_TRANSFORMER_HIP_POOL": "0", "RIFTCO_TRANSFORMER_HIP_MERGE": "0"},
+    {"RIFTCO_TRANSFORMER_HIP_ASYNC": "1", "RIFTCO_TRANSFORMER_HIP_MERGE": "0"},
 ])
 def test_adapter_options_on_the_host_only_runtime(options):
     """Without the buffer pool, without the per-operation synchronise, and
@@ -87,7 +88,7 @@ def run_sanitized(program, runtime, **environment):
     {"FAKE_RTHIP_CAN_FAIL": "1"},
     {"RIFTCO_TRANSFORMER_HIP_POOL": "0"},
     {"RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
-    {"RIFTCO_TRANSFORMER_HIP_MERGE": "1"},
+    {"RIFTCO_TRANSFORMER_HIP_MERGE": "0"},
     {"FAKE_RTHIP_NO_BAR": "1"},
 ])
 def test_adapter_under_address_and_undefined_behaviour_sanitizers(options):
@@ -109,7 +110,7 @@ def test_adapter_under_address_and_undefined_behaviour_sanitizers(options):
     {},
     {"RIFTCO_TRANSFORMER_HIP_POOL": "0"},
     {"RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
-    {"RIFTCO_TRANSFORMER_HIP_MERGE": "1"},
+    {"RIFTCO_TRANSFORMER_HIP_MERGE": "0"},
 ])
 def test_adapter_from_four_threads_under_thread_sanitizer(options):
     """tests/cpp/test_threads.cpp: four threads share a weight, an input and
@@ -237,7 +238,7 @@ def test_adapter_on_the_real_library():
 @pytest.mark.parametrize("options", [
     {"RIFTCO_TRANSFORMER_HIP_POOL": "0"},
     {"RIFTCO_TRANSFORMER_HIP_ASYNC": "1"},
-    {"RIFTCO_TRANSFORMER_HIP_MERGE": "1"},
+    {"RIFTCO_TRANSFORMER_HIP_MERGE": "0"},
 ])
 def test_adapter_options_on_the_real_library(options):
     """The pool switched off, and operations queued without a synchronise per

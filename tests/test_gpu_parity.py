@@ -588,7 +588,8 @@ def test_two_host_threads_launch_on_one_stream(gpu, package, library, oracle):
     """Kernels that hand partial results to a second kernel through the
     stream's scratch buffer (the small-batch forward and input backward, the
     tiled kernel's leftover tiles, the streaming and the shape-agnostic input
-    backward, the adapter's d_reduced) are launched from two host threads at once
+    backward, the adapter's d_reduced, the input backward that keeps its partial
+    sums in the library's static array) are launched from two host threads at once
     on the same stream, each thread with its own input: a thread's sum kernel
     must never read the other thread's partial results.  Every output equals,
     bit for bit, the one the same call gives alone."""
@@ -603,13 +604,15 @@ def test_two_host_threads_launch_on_one_stream(gpu, package, library, oracle):
         (11008, 4096, 1, "backward"),     # streamed weight, row ranges
         (1001, 4095, 3, "backward"),      # shape-agnostic kernel, row chunks
         (4096, 1024, 12, "adapter"),      # d_reduced in column slices
+        (4096, 1024, 64, "no_alloc"),     # row chunks in the static array
     ]
     for out_w, in_w, rows, direction in cases:
         weight = oracle.quantize(helpers.normal(95, (out_w, in_w), 0.02), 64,
                                  False, 256)
         device_weight = upload(gpu, weight)
         width = in_w if direction == "forward" else out_w
-        other = {"forward": out_w, "backward": in_w, "adapter": 8}[direction]
+        other = {"forward": out_w, "backward": in_w, "adapter": 8,
+                 "no_alloc": in_w}[direction]
         inputs = [to_device(helpers.normal(96 + t, (rows, width), 1.0))
                   for t in range(2)]
 
@@ -627,6 +630,10 @@ def test_two_host_threads_launch_on_one_stream(gpu, package, library, oracle):
             elif direction == "forward":
                 library.linear_forward(source.data_ptr(), device_weight, None,
                                        target.data_ptr(), rows, stream)
+            elif direction == "no_alloc":
+                library.linear_input_backward_no_alloc(
+                    source.data_ptr(), device_weight, target.data_ptr(), rows,
+                    stream)
             else:
                 library.linear_input_backward(source.data_ptr(),
                                               device_weight,

@@ -74,3 +74,38 @@ def test_no_alloc_input_backward_matches_the_allocating_entry_point(
         library.linear_input_backward_no_alloc(
             dy_device.data_ptr(), big, got.data_ptr(), 65,
             torch.cuda.current_stream().cuda_stream)
+
+
+def test_no_alloc_array_is_bound_to_one_stream(gpu, package, library, oracle):
+    """Calls that overlap on the GPU would race on the one static array, so
+    it is bound to the stream of the first call: another stream is refused
+    until rthip_release_workspaces has unbound it."""
+    import torch
+    out_w, in_w, rows = 4096, 1024, 64
+    weight = oracle.quantize(helpers.normal(320, (out_w, in_w), 0.02), 64,
+                             False, 256)
+    device_weight = upload(gpu, weight)
+    dy_device = torch.from_numpy(
+        helpers.normal(321, (rows, out_w), 1.0e-2)).cuda()
+    first = torch.empty(rows, in_w, device="cuda")
+    main = torch.cuda.current_stream().cuda_stream
+    library.linear_input_backward_no_alloc(dy_device.data_ptr(),
+                                           device_weight, first.data_ptr(),
+                                           rows, main)
+    other = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    second = torch.empty(rows, in_w, device="cuda")
+    with pytest.raises(package.Unsupported) as refused:
+        library.linear_input_backward_no_alloc(
+            dy_device.data_ptr(), device_weight, second.data_ptr(), rows,
+            other.cuda_stream)
+    assert "another stream" in str(refused.value)
+    library.release_workspaces(0, True)  # unbinds (after the stream is done)
+    library.linear_input_backward_no_alloc(dy_device.data_ptr(),
+                                           device_weight, second.data_ptr(),
+                                           rows, other.cuda_stream)
+    torch.cuda.synchronize()
+    helpers.assert_bit_equal(second.cpu().numpy(), first.cpu().numpy(),
+                             "the same call on the newly bound stream")
+    # back to the stream the other tests use
+    library.release_workspaces(0, True)
