@@ -1,6 +1,6 @@
 """Benchmark of the packed NF4 linear path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--full]
 
 Headline workload (the configuration the metric is quoted on): decode GEMV,
 M = 1, the seven Llama-7B projection shapes per layer (q/k/v/o 4096x4096,
@@ -8,48 +8,41 @@ gate/up 11008x4096, down 4096x11008), NF4 block 64 with fp32 absmax scales, no
 bias.  One step = one token through all 7 projections of L layers, every layer
 holding its own packed weights, so the working set (L x 113.8 MB) is far
 larger than the 256 MB last-level cache and every step streams it from HBM.
-`value` = algorithmic bytes (packed codes + scale payload) per second with
-everything resident in HBM before the timed region.
+Projections that read the same activations (q/k/v; gate/up) go out in ONE
+launch through rthip_nf4_linear_forward_group -- four launches per layer, as
+the backend adapter issues them for unchanged callers -- and
+--one-launch-per-projection times the seven-launch form instead (both are in
+the line either way, see roofline.decode_steps).  `value` = algorithmic bytes
+(packed codes + scale payload) per second with everything resident in HBM
+before the timed region.
 
-The same JSON line carries
-  roofline      HBM roofline of the GEMV kernel (bytes per launch / average
-                launch duration from HIP events on the launch stream)
-  decode_double_quantized_scales
-                the decode step again with the nested scale encoding
-  decode_shared_input_groups
-                the decode step with q/k/v and gate/up launched together
-                through rthip_nf4_linear_forward_group
-  gemm          M = 2048 forward and input-backward GEMMs (prefill / training
-                shapes) with their fp32-MFMA rooflines
-  small_batch   M in {1, 4, 16, 64} on the three distinct shapes
-  small_batch_groups
-                q/k/v and gate/up at M in {4, 16, 64}: one launch per
-                projection against one launch per group
-  mid_batch     M in {128, 192, 256, 272, 512, 1024}: between the small-batch
-                kernels and the prefill shapes (192 is one and a half row
-                tiles of the GEMM, 272 two and sixteen rows)
-  ragged_shapes a shape only the shape-agnostic kernels take (4097 x 4095)
-  large_launches
-                M = 1 launches of 74 to 117 MB (lm_head; four gate/up weights
-                in one grouped launch; the feed-forward projections of a 70B
-                model)
-  practical_roof
-                a plain streaming read of the same sizes, one launch per
-                buffer, and an empty launch: what the device gives a kernel
-                that only reads, beside the 8 TB/s of the data sheet
-  small_batch_input_backward
-                the input backward at M in {1, 16, 64}, nested scales
-  lora          the fused bias + rank-16 adapter forward beside the plain one,
-                and the backward pass with the adapter (d_reduced, dA, dB and
-                the adapter's share of dx) beside the plain input backward
-  matmul        dense fp32 matmul at layer and adapter shapes
-  quantizer     the device quantizer on one 11008 x 4096 weight (wall clock,
-                the call returns after the work is done)
+Everything that the metric names is inside `roofline`, so that a reader of
+that object alone can recompute it:
+  roofline      HBM roofline of the dominant decode kernel (bytes per launch /
+                average launch duration from HIP events on the launch stream;
+                traffic from the tracked rocprofv3 counter summary, refused
+                when that summary was taken with other kernel instances than
+                this build launches)
+    .decode_steps   the decode step four ways: launches per shared input or per
+                    projection, fp32 or nested (double-quantised) scales
+    .gemm           M = 2048 forward and input-backward GEMMs (prefill /
+                    training shapes, both scale encodings) against the fp32
+                    MFMA peak
+    .small_batch    M in {1, 4, 16, 64} on the three distinct shapes
+    .large_launches M = 1 launches of 74 to 117 MB (lm_head; four gate/up
+                    weights in one launch; a 70B model's feed-forward shapes)
+    .practical_roof a plain streaming read of the same sizes, one launch per
+                    buffer, and an empty launch: what the device gives a kernel
+                    that only reads, beside the 8 TB/s of the data sheet
   cpu_baseline  the reference CPU backend (kind "reference": oracle/_ref, built
                 in the build container from the reference's own sources and
                 shipped prebuilt; kind "port": the C restatement, where that
                 library is absent) timed on this host, single thread, on one
                 layer; host_cpu names the processor
+With --full the line also carries
+  small_batch_groups, mid_batch (M in {128 ... 1024}), ragged_shapes (4097 x
+  4095), small_batch_input_backward, lora (fused adapter forward and
+  backward), matmul (dense fp32) and quantizer.
 
 Packed payloads are synthetic: uniformly random nibbles (NF4 codes of normal
 weights are close to uniform by construction) and block scales drawn around
@@ -203,6 +196,14 @@ def bench_decode(package, device, torch, layers, steps, warmup, use_graph,
                          for item in dominant for member in item[1])
     average_us = dominant_ms * 1e3 / (steps * len(dominant))
     achieved = dominant_bytes * steps / (dominant_ms / 1e3) / 1e9
+    # the kernel instances of those launches, as a profiler prints them
+    encoding = weights[0].encoding
+    instances = sorted({
+        library.forward_kernel_name(
+            1, 4096, [member[0].output_width for member in item[1]], BLOCK,
+            encoding, SECOND_LEVEL_BLOCK if double_quantized else 0)
+        for item in dominant})
+    traffic, traffic_source = profiled_traffic(grouped, instances)
     return {
         "value": gbs,
         "ms_per_step": milliseconds / steps,
@@ -212,10 +213,8 @@ def bench_decode(package, device, torch, layers, steps, warmup, use_graph,
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": profiled_traffic(grouped)[0],
-            "traffic_source": profiled_traffic(grouped)[1],
-            "kernel": "gemv_forward_kernel<rows=1, K=4096%s>" % (
-                ", grouped" if grouped else ""),
+            "traffic": traffic, "traffic_source": traffic_source,
+            "kernel": ", ".join(instances),
             "bytes_per_launch": dominant_bytes / len(dominant),
             "avg_launch_us": average_us,
         },
@@ -226,18 +225,18 @@ TRAFFIC_PROFILE = os.path.join(ROOT, "profiles",
                                "decode_gemv_hbm_traffic_pmc.txt")
 
 
-def profiled_traffic(grouped):
+def profiled_traffic(grouped, instances):
     """HBM bytes per launch of the dominant kernel as the tracked rocprofv3
     counter summary has them (a counter run cannot be nested inside this
-    timing run): FETCH_SIZE and WRITE_SIZE averages of the K = 4096 GEMV
-    instantiation, each scaled by what the same counter read for torch's
+    timing run): FETCH_SIZE and WRITE_SIZE averages of the kernel instances
+    in `instances` (the names this build reports for the launches that were
+    timed), each scaled by what the same counter read for torch's
     2^28-element copy (2^20 KiB read, 2^20 KiB written).  Returns (bytes,
-    where it came from), or (None, why not) when the summary cannot be read
-    -- a kernel whose template arguments changed since it was profiled shows
-    up here as "no row", not as a stale figure."""
+    where it came from), or (None, why not): a summary that was taken with
+    other instances than this build launches has no row for them and is
+    refused, not quoted."""
     section = ("projections that share x in one launch" if grouped
                else "one launch per projection")
-    grouped_flag = "true>" if grouped else "false>"
     try:
         with open(TRAFFIC_PROFILE) as handle:
             text = handle.read()
@@ -245,9 +244,13 @@ def profiled_traffic(grouped):
         return None, "no profile: %s" % error
     if section not in text:
         return None, "the profile has no section '%s'" % section
-    body = text[text.index(section):]
-    if not grouped and "projections that share x" in body:
-        body = body[:body.index("projections that share x")]
+    body = text[text.index(section) + len(section):]
+    for other in ("projections that share x in one launch",
+                  "one launch per projection"):
+        if other != section and other in body:
+            body = body[:body.index(other)]
+    if not instances or "" in instances:
+        return None, "the timed launches are not served by the decode kernel"
     readings = {}
     for line in body.splitlines():
         fields = line.split()
@@ -255,17 +258,31 @@ def profiled_traffic(grouped):
             if counter not in fields:
                 continue
             average = float(fields[fields.index(counter) + 2])
+            calls = float(fields[fields.index(counter) + 1])
             if line.startswith("at::native::vectorized_elementwise_kernel"):
-                readings[counter, "copy"] = average
-            elif (line.startswith("rthip::gemv_forward_kernel<1, 1,") and
-                  line.split(">")[0].endswith(grouped_flag[:-1])):
-                readings[counter, "kernel"] = average
+                # the 2^28-element copy is the largest of torch's launches
+                if average >= readings.get((counter, "copy"), (0.0, 0))[0]:
+                    readings[counter, "copy"] = (average, calls)
+            for name in instances:
+                if ("rthip::" + name) in line.replace(
+                        "(anonymous namespace)::", ""):
+                    total, count = readings.get((counter, "kernel"), (0, 0))
+                    readings[counter, "kernel"] = (total + average * calls,
+                                                   count + calls)
+                    readings[counter, name] = True
+    missing = [name for name in instances
+               if (("FETCH_SIZE", name) not in readings or
+                   ("WRITE_SIZE", name) not in readings)]
+    if missing:
+        return None, ("the profile was taken with other kernel instances: "
+                      "no row for %s" % ", ".join(missing))
     try:
-        kib = sum(readings[counter, "kernel"] * 2.0 ** 20 /
-                  readings[counter, "copy"]
+        kib = sum(readings[counter, "kernel"][0] /
+                  readings[counter, "kernel"][1] * 2.0 ** 20 /
+                  readings[counter, "copy"][0]
                   for counter in ("FETCH_SIZE", "WRITE_SIZE"))
-    except KeyError as missing:
-        return None, "the profile has no row for %s" % (missing.args[0],)
+    except KeyError as missing_row:
+        return None, "the profile has no row for %s" % (missing_row.args[0],)
     return int(kib * 1024), (
         "profiles/decode_gemv_hbm_traffic_pmc.txt: rocprofv3 --pmc "
         "FETCH_SIZE / WRITE_SIZE per dispatch, each scaled by its reading "
@@ -792,6 +809,18 @@ def cpu_baseline(budget_seconds=12.0):
     }
 
 
+def rounded(value, digits=4):
+    """Floats to `digits` significant digits, recursively: keeps the line
+    short enough to be read where only its tail is kept."""
+    if isinstance(value, float):
+        return float("%.*g" % (digits, value))
+    if isinstance(value, dict):
+        return {key: rounded(item, digits) for key, item in value.items()}
+    if isinstance(value, list):
+        return [rounded(item, digits) for item in value]
+    return value
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -801,6 +830,11 @@ def main():
     parser.add_argument("--skip-extras", action="store_true",
                         help="only the headline decode workload")
     parser.add_argument("--skip-cpu", action="store_true")
+    parser.add_argument("--full", action="store_true",
+                        help="also the sections off the metric: mid-size "
+                             "batches, ragged shapes, the adapter, dense "
+                             "matmul, the quantizer, small-batch groups and "
+                             "input backward")
     parser.add_argument("--gemm-only", action="store_true",
                         help="run only the M = 2048 GEMM section (for "
                              "rocprofv3 counter runs)")
@@ -812,15 +846,16 @@ def main():
                              "and backward (for rocprofv3 kernel traces)")
     parser.add_argument("--practical-roof-only", action="store_true",
                         help="run only the streaming-read and empty-launch "
-                             "probes (for rocprofv3 kernel traces)")
+                             "probes and a 1 GiB elementwise copy beside "
+                             "them (for rocprofv3 kernel traces)")
     parser.add_argument("--traffic-calibration", action="store_true",
                         help="for rocprofv3 --pmc runs: a 1 GiB elementwise "
                              "copy of known traffic, then one decode step "
                              "launched kernel by kernel, nothing else")
-    parser.add_argument("--shared-input-groups", action="store_true",
+    parser.add_argument("--one-launch-per-projection", action="store_true",
                         help="headline decode step (and the traffic "
-                             "calibration) with q/k/v and gate/up launched "
-                             "together: 4 launches per layer instead of 7")
+                             "calibration) with one launch per projection, "
+                             "7 per layer, instead of one per shared input")
     parser.add_argument("--no-graph", action="store_true",
                         help="launch the decode kernels one by one from "
                              "Python instead of replaying a HIP graph")
@@ -835,10 +870,27 @@ def main():
     library = package.load_library()
     if not torch.cuda.is_available() or not library.is_available():
         sys.exit("bench.py: no usable MI355X: " + library.last_error())
+    grouped = not arguments.one_launch_per_projection
 
     if arguments.practical_roof_only:
-        print(json.dumps({"practical_roof": bench_practical_roof(
-            package, torch, arguments.steps)}))
+        # torch's elementwise kernel beside the probes, in the same trace: it
+        # reads 2^30 B and writes 2^30 B per call
+        source = torch.zeros(2 ** 28, device="cuda")
+        target = torch.empty_like(source)
+        for _ in range(5):
+            torch.add(source, 1.0, out=target)
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        for _ in range(10):
+            torch.add(source, 1.0, out=target)
+        torch.cuda.synchronize()
+        copy_ms = (time.perf_counter() - begin) * 100.0
+        del source, target
+        print(json.dumps({
+            "elementwise_copy_1gib": {
+                "ms": copy_ms, "read_plus_write_gb_per_s": 2 ** 31 / copy_ms / 1e6},
+            "practical_roof": bench_practical_roof(package, torch,
+                                                   arguments.steps)}))
         return
 
     if arguments.traffic_calibration:
@@ -850,7 +902,7 @@ def main():
             torch.add(source, 1.0, out=target)
         torch.cuda.synchronize()
         bench_decode(package, device, torch, arguments.layers, 1, 0, False,
-                     grouped=arguments.shared_input_groups)
+                     grouped=grouped)
         print(json.dumps({"traffic_calibration": "done",
                           "copy_bytes_read": 2 ** 30,
                           "copy_bytes_written": 2 ** 30}))
@@ -879,10 +931,28 @@ def main():
                 package, device, torch, arguments.steps)}))
         return
 
-    decode = bench_decode(package, device, torch, arguments.layers,
-                          arguments.steps, arguments.warmup,
-                          not arguments.no_graph,
-                          grouped=arguments.shared_input_groups)
+    def decode_step(grouped_launches, double_quantized, steps):
+        result = bench_decode(package, device, torch, arguments.layers, steps,
+                              arguments.warmup, not arguments.no_graph,
+                              double_quantized=double_quantized,
+                              grouped=grouped_launches)
+        summary = {
+            "launches": ("per_shared_input" if grouped_launches
+                         else "per_projection"),
+            "scales": "double_quantized" if double_quantized else "fp32",
+            "launches_per_step": result["launches_per_step"],
+            "bytes_per_step": result["bytes_per_step"],
+            "ms_per_step": result["ms_per_step"],
+            "gb_per_s": result["value"],
+            "frac_of_hbm_peak": result["value"] / HBM_PEAK_GBS,
+            "dominant_kernel": result["roofline"]["kernel"],
+            "dominant_kernel_frac": result["roofline"]["frac"],
+            "dominant_kernel_us": result["roofline"]["avg_launch_us"],
+        }
+        return result, summary
+
+    decode, headline_summary = decode_step(grouped, False, arguments.steps)
+    roofline = decode["roofline"]
     line = {
         "metric": "NF4 linear: HBM GB/s at M=1, TFLOP/s at M=2048, % of "
                   "MI355X roofline",
@@ -898,7 +968,7 @@ def main():
                         "%d layers x 7 projections per step%s" % (
                             arguments.layers,
                             ", projections that share their input launched "
-                            "together" if arguments.shared_input_groups
+                            "together (4 launches per layer)" if grouped
                             else ", one launch per projection"),
             "layers": arguments.layers,
             "bytes_per_step": decode["bytes_per_step"],
@@ -906,58 +976,51 @@ def main():
             "launch": "per-kernel" if arguments.no_graph else "hip-graph",
             "device": library.device_description(),
         },
-        "roofline": decode["roofline"],
+        "roofline": roofline,
     }
+    del decode
+    roofline["decode_steps"] = [headline_summary]
     if not arguments.skip_extras:
-        del decode
-        # The same decode step with the reference's double-quantised scale
-        # encoding (3.36 GB of packed payload per step instead of 3.64).
-        nested = bench_decode(package, device, torch, arguments.layers,
-                              max(3, arguments.steps // 2), arguments.warmup,
-                              not arguments.no_graph, double_quantized=True)
-        line["decode_double_quantized_scales"] = {
-            "value": nested["value"], "unit": "GB/s",
-            "ms_per_step": nested["ms_per_step"],
-            "bytes_per_step": nested["bytes_per_step"],
-        }
-        del nested
-        # The same step with projections that share their input launched
-        # together (q/k/v and gate/up): 4 launches per layer instead of 7.
-        together = bench_decode(package, device, torch, arguments.layers,
-                                max(3, arguments.steps // 2),
-                                arguments.warmup, not arguments.no_graph,
-                                grouped=True)
-        line["decode_shared_input_groups"] = {
-            "value": together["value"], "unit": "GB/s",
-            "ms_per_step": together["ms_per_step"],
-            "launches_per_step": together["launches_per_step"],
-            "roofline": together["roofline"],
-        }
-        del together
-        line["gemm"] = bench_gemm(package, device, torch,
-                                  max(3, arguments.steps // 4))
-        line["small_batch"] = bench_small_batch(package, device, torch,
-                                                max(3, arguments.steps // 4))
-        line["small_batch_groups"] = bench_small_batch_groups(
-            package, device, torch, max(3, arguments.steps // 4))
-        line["mid_batch"] = bench_mid_batch(package, device, torch,
-                                            max(3, arguments.steps // 4))
-        line["ragged_shapes"] = bench_ragged(package, device, torch,
-                                             max(3, arguments.steps // 4))
-        line["large_launches"] = bench_large_launches(
-            package, device, torch, max(3, arguments.steps // 2))
-        line["practical_roof"] = bench_practical_roof(
-            package, torch, max(3, arguments.steps // 2))
-        line["small_batch_input_backward"] = bench_small_batch_backward(
-            package, device, torch, max(3, arguments.steps // 4))
-        line["lora"] = bench_lora(package, device, torch,
-                                  max(3, arguments.steps // 4))
-        line["matmul"] = bench_matmul(package, device, torch,
-                                      max(3, arguments.steps // 4))
-        line["quantizer"] = bench_quantizer(package, device, torch)
+        fewer = max(3, arguments.steps // 2)
+        few = max(3, arguments.steps // 4)
+        # The decode step the other three ways: the other launch grouping,
+        # and both with the reference's double-quantised scale encoding
+        # (3.34 GB of packed payload per step instead of 3.64).
+        for grouped_launches, double_quantized in (
+                (not grouped, False), (grouped, True), (not grouped, True)):
+            result, summary = decode_step(grouped_launches, double_quantized,
+                                          fewer)
+            del result
+            roofline["decode_steps"].append(summary)
+        roofline["gemm"] = [
+            {"direction": case["direction"],
+             "weight": "%dx%d" % (case["output_width"], case["input_width"]),
+             "rows": case["rows"], "scales": case["scales"], "ms": case["ms"],
+             "tflop_per_s": case["roofline"]["achieved"],
+             "frac_of_fp32_mfma_peak": case["roofline"]["frac"]}
+            for case in bench_gemm(package, device, torch, few)]
+        roofline["small_batch"] = bench_small_batch(package, device, torch,
+                                                    few)
+        roofline["large_launches"] = [
+            {"launch": case["launch"], "bytes": case["bytes"],
+             "us": case["us"], "gb_per_s": case["roofline"]["achieved"],
+             "frac_of_hbm_peak": case["roofline"]["frac"]}
+            for case in bench_large_launches(package, device, torch, fewer)]
+        roofline["practical_roof"] = bench_practical_roof(package, torch,
+                                                          fewer)
+        if arguments.full:
+            line["small_batch_groups"] = bench_small_batch_groups(
+                package, device, torch, few)
+            line["mid_batch"] = bench_mid_batch(package, device, torch, few)
+            line["ragged_shapes"] = bench_ragged(package, device, torch, few)
+            line["small_batch_input_backward"] = bench_small_batch_backward(
+                package, device, torch, few)
+            line["lora"] = bench_lora(package, device, torch, few)
+            line["matmul"] = bench_matmul(package, device, torch, few)
+            line["quantizer"] = bench_quantizer(package, device, torch)
     if not arguments.skip_cpu:
         line["cpu_baseline"] = cpu_baseline()
-    print(json.dumps(line))
+    print(json.dumps(rounded(line, 5)))
 
 
 if __name__ == "__main__":

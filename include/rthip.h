@@ -41,7 +41,7 @@ extern "C" {
 #endif
 
 #define RTHIP_ABI_VERSION_MAJOR 1u
-#define RTHIP_ABI_VERSION_MINOR 7u
+#define RTHIP_ABI_VERSION_MINOR 8u
 
 typedef int32_t rthip_status;
 
@@ -351,6 +351,19 @@ rthip_status rthip_nf4_lora_linear_input_backward_with(
 rthip_status rthip_nf4_select_algorithm(
     int32_t direction, uint64_t rows, uint64_t input_width,
     uint64_t output_width, uint64_t block_size, int32_t* algorithm);
+
+/* The kernel instance that rthip_nf4_linear_forward (member_count == 1) or
+ * rthip_nf4_linear_forward_group launches for weights of these output widths
+ * when the one-row decode kernel serves the call, as a profiler prints it
+ * without its namespace ("gemv1_forward_kernel<1, 8, 2, 4, false, false,
+ * 4>"); an empty string where another family serves it.  For tools that have
+ * to tell whether a stored profile still describes the kernels a build
+ * launches.  Pure host computation; needs no device.  No counterpart in the
+ * reference. */
+rthip_status rthip_nf4_forward_kernel_name(
+    uint64_t rows, uint64_t input_width, const uint64_t* output_widths,
+    uint64_t member_count, uint64_t block_size, int32_t encoding,
+    uint64_t second_level_block, char* name, uint64_t capacity);
 
 /*
  * out[j] = scale(j / block_size) * codebook[code(j)] for j < element_count.

@@ -143,6 +143,9 @@ _PROTOTYPES = {
                                         _u64, _u64, _ptr]),
     "rthip_nf4_select_algorithm": (
         _i32, [_i32, _u64, _u64, _u64, _u64, ctypes.POINTER(_i32)]),
+    "rthip_nf4_forward_kernel_name": (
+        _i32, [_u64, _u64, ctypes.POINTER(_u64), _u64, _u64, _i32, _u64,
+               ctypes.c_char_p, _u64]),
     "rthip_nf4_dequantize": (_i32, _WEIGHT + [_ptr, _u64, _u64, _ptr]),
     "rthip_nf4_quantize": (
         _i32, [_ptr, _u64, _u64, _i32, _u64, _ptr, _ptr, _ptr, _ptr,
@@ -272,6 +275,19 @@ class Library:
             direction, rows, input_width, output_width, block_size,
             ctypes.byref(algorithm)))
         return algorithm.value
+
+    def forward_kernel_name(self, rows: int, input_width: int, output_widths,
+                            block_size: int, encoding: int,
+                            second_level_block: int = 0) -> str:
+        """The one-row decode kernel instance a forward of these weights
+        launches, as a profiler prints it ("" where another family serves
+        the call)."""
+        widths = (_u64 * len(output_widths))(*output_widths)
+        name = ctypes.create_string_buffer(160)
+        self._check(self._lib.rthip_nf4_forward_kernel_name(
+            rows, input_width, widths, len(output_widths), block_size,
+            encoding, second_level_block, name, len(name)))
+        return name.value.decode()
 
     def linear_forward(self, x_ptr: int, weight: DeviceWeight,
                        bias_ptr: Optional[int], y_ptr: int, rows: int,

@@ -65,6 +65,10 @@ void launch_gemv_group(const LinearProblem* problems, std::size_t count,
 bool gemv1_forward_supports(const LinearProblem& problem);
 void launch_gemv1_forward(const LinearProblem* problems, std::size_t count,
                           hipStream_t stream);
+// The name of the instance that launch would run, as a profiler prints it
+// without its namespace ("gemv1_forward_kernel<1, 8, 2, 4, false, false, 4>").
+void gemv1_kernel_name(const LinearProblem* problems, std::size_t count,
+                       char* name, std::size_t capacity);
 
 // workspace.hip -- scratch memory shared by the kernels that pass partial
 // results between workgroups; one fixed-size buffer per (device, stream),

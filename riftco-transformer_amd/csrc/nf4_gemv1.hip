@@ -57,6 +57,7 @@
 #include "nf4_pair_table.hpp"
 #include "gemv_shared.hpp"
 
+#include <cstdio>
 #include <type_traits>
 
 namespace rthip {
@@ -472,9 +473,17 @@ std::size_t segments_per_thread(const LinearProblem& p) {
     return (p.input_width / kSegment + kThreads - 1) / kThreads;
 }
 
+// What to do with the instance that serves a call: launch it, or only write
+// its name (as a profiler prints it) into `name`.
+struct Request {
+    hipStream_t stream;
+    char* name;
+    std::size_t capacity;
+};
+
 template <int kSegments, bool kDoubleQuantized, int kMembers>
 void launch_instance(const LinearProblem* problems, std::size_t count,
-                     hipStream_t stream) {
+                     const Request& request) {
     constexpr int kDepth = RTHIP_GEMV1_DEPTH;
     // A compute unit keeps about 32 KB of loads in flight (its vector L1):
     // a batch should stay well below that, so wider rows take fewer of them.
@@ -530,9 +539,18 @@ void launch_instance(const LinearProblem* problems, std::size_t count,
     const unsigned iterations = (batch_count + blocks - 1) / blocks;
     const OneRowSource& head = sources[0];
     const auto launch = [&](auto whole_groups) {
+        constexpr bool kWhole = decltype(whole_groups)::value;
+        if (request.name != nullptr) {
+            std::snprintf(request.name, request.capacity,
+                          "gemv1_forward_kernel<%d, %d, %d, %d, %s, %s, %d>",
+                          kSegments, kRows, kDepth, kLook,
+                          kDoubleQuantized ? "true" : "false",
+                          kWhole ? "true" : "false", kMembers);
+            return;
+        }
         gemv1_forward_kernel<kSegments, kRows, kDepth, kLook, kDoubleQuantized,
-                             decltype(whole_groups)::value, kMembers>
-            <<<blocks, kThreads, 0, stream>>>(
+                             kWhole, kMembers>
+            <<<blocks, kThreads, 0, request.stream>>>(
                 first.activations, head.codes, head.primary_scales,
                 static_cast<unsigned>(first.input_width), head.code_bytes,
                 head.primary_bytes, iterations, head.secondary_scales,
@@ -554,7 +572,7 @@ void launch_instance(const LinearProblem* problems, std::size_t count,
 
 template <bool kDoubleQuantized, int kMembers>
 void launch_segments(const LinearProblem* problems, std::size_t count,
-                     hipStream_t stream) {
+                     const Request& stream) {
     switch (segments_per_thread(problems[0])) {
     case 1:
         launch_instance<1, kDoubleQuantized, kMembers>(problems, count, stream);
@@ -570,7 +588,7 @@ void launch_segments(const LinearProblem* problems, std::size_t count,
 
 template <int kMembers>
 void launch_encoding(const LinearProblem* problems, std::size_t count,
-                     hipStream_t stream) {
+                     const Request& stream) {
     if (problems[0].weight.encoding == 0) {
         launch_segments<false, kMembers>(problems, count, stream);
     } else {
@@ -596,11 +614,23 @@ bool gemv1_forward_supports(const LinearProblem& p) {
 
 void launch_gemv1_forward(const LinearProblem* problems, std::size_t count,
                           hipStream_t stream) {
+    const Request request{stream, nullptr, 0};
     if (count == 1) {
-        launch_encoding<1>(problems, count, stream);
+        launch_encoding<1>(problems, count, request);
     } else {
         launch_encoding<static_cast<int>(kGemvGroupMax)>(problems, count,
-                                                         stream);
+                                                         request);
+    }
+}
+
+void gemv1_kernel_name(const LinearProblem* problems, std::size_t count,
+                       char* name, std::size_t capacity) {
+    const Request request{nullptr, name, capacity};
+    if (count == 1) {
+        launch_encoding<1>(problems, count, request);
+    } else {
+        launch_encoding<static_cast<int>(kGemvGroupMax)>(problems, count,
+                                                         request);
     }
 }
 

@@ -1456,6 +1456,59 @@ rthip_status rthip_nf4_linear_input_backward_no_alloc(
         kStaticScratchBytes, rthip::LoraEpilogue{});
 }
 
+rthip_status rthip_nf4_forward_kernel_name(
+    uint64_t rows, uint64_t input_width, const uint64_t* output_widths,
+    uint64_t member_count, uint64_t block_size, int32_t encoding,
+    uint64_t second_level_block, char* name, uint64_t capacity
+) {
+    if (output_widths == nullptr || name == nullptr || capacity == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "output widths and the name buffer must not be null");
+    }
+    if (member_count == 0 || member_count > rthip::kGemvGroupMax) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "between 1 and %zu weights share a launch",
+                    rthip::kGemvGroupMax);
+    }
+    name[0] = '\0';
+    // stand-ins for device memory: only their alignment is looked at
+    alignas(256) static const float activations[4] = {};
+    alignas(256) static const std::uint8_t payload[16] = {};
+    alignas(256) static float results[rthip::kGemvGroupMax][4];
+    rthip::LinearProblem problems[rthip::kGemvGroupMax];
+    for (uint64_t m = 0; m < member_count; ++m) {
+        rthip::LinearProblem& problem = problems[m];
+        problem = rthip::LinearProblem{};
+        if (const rthip_status status = check_dimensions(
+                rows, input_width, output_widths[m], block_size,
+                &problem.block_shift);
+            status != RTHIP_OK) {
+            return status;
+        }
+        if (const rthip_status status = make_weight_view(
+                payload, payload,
+                encoding == RTHIP_NF4_SCALE_FLOAT32 ? nullptr : activations,
+                encoding, second_level_block, 0.0F, &problem.weight);
+            status != RTHIP_OK) {
+            return status;
+        }
+        problem.activations = activations;
+        problem.result = results[m];
+        problem.rows = rows;
+        problem.input_width = input_width;
+        problem.output_width = output_widths[m];
+        if (!rthip::gemv1_forward_supports(problem)) {
+            return RTHIP_OK;  // another family: no name
+        }
+    }
+    if (member_count > 1 &&
+        !rthip::gemv_group_supports(problems, member_count)) {
+        return RTHIP_OK;
+    }
+    rthip::gemv1_kernel_name(problems, member_count, name, capacity);
+    return RTHIP_OK;
+}
+
 rthip_status rthip_probe_streaming_read(const void* data, uint64_t bytes,
                                         void* stream) {
     if (data == nullptr || bytes == 0 || bytes % 16 != 0 ||
