@@ -115,7 +115,9 @@ struct RowBatch {
 // kWholeGroups (nested scales): every batch starts on a second-level group
 // boundary, so a lane's second-level scale sits at a fixed offset from the
 // batch's first one.
-template <int kSegments, int kRows, int kDepth, int kLook,
+// kX: rows of x held per thread (1, 2 or 4; three rows run as four with an
+// empty fourth).
+template <int kX, int kSegments, int kRows, int kDepth, int kLook,
           bool kDoubleQuantized, bool kWholeGroups, int kMembers>
 __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
     // The first 14 dwords are preloaded into scalar registers when the
@@ -128,14 +130,15 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
     const float* __restrict__ secondary_scales, unsigned secondary_bytes,
     float offset_of_scales,
     // read from memory
-    unsigned second_level_shift, unsigned batch_count,
+    unsigned second_level_shift, unsigned batch_count, unsigned x_rows,
     const OneRowRest<kMembers> rest, const LoraEpilogue lora
 ) {
     constexpr bool kGrouped = kMembers > 1;
-    constexpr unsigned kMaxIterations = kParkedRows / kRows;
+    constexpr unsigned kMaxIterations = kParkedRows / (kRows * kX);
     static_assert(kRows == 8 || kRows == 4 || kRows == 2);
+    static_assert(kX == 1 || kX == 2 || kX == 4);
     __shared__ __attribute__((aligned(256))) char table[kPairTableBytes];
-    __shared__ float partial[kMaxIterations][kWaves][kRows];
+    __shared__ float partial[kMaxIterations][kWaves][kRows][kX];
     // Nested scales: (code - 128) / 127 for every scale code, so that a
     // scale costs its lane one LDS read, a multiply and an add instead of a
     // correctly rounded division (the same quotients, hence the same scales
@@ -289,24 +292,30 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
     load_batch(ring[0], first_batch);
 
     // This thread's slice of x, resident for the whole kernel; stripes past
-    // the row end read as zero (range check).
-    const __amdgpu_buffer_rsrc_t x_buffer =
-        make_buffer(x, input_width * 4U);
-    float xs[kSegments][kSegment];
+    // the row end and rows past x_rows read as zero (range check).
+    float xs[kX][kSegments][kSegment];
 #pragma unroll
-    for (int j = 0; j < kSegments; ++j) {
-        const unsigned first = (thread + kThreads * j) * (kSegment * 4);
+    for (int r = 0; r < kX; ++r) {
+        const bool row_exists = static_cast<unsigned>(r) < x_rows;
+        const __amdgpu_buffer_rsrc_t x_buffer = make_buffer(
+            x + (row_exists ? static_cast<unsigned>(r) * input_width : 0U),
+            row_exists ? input_width * 4U : 0U);
 #pragma unroll
-        for (int q = 0; q < kSegment / 4; ++q) {
-            // (the whole vector is cast at once: a bit cast of ONE element
-            // of an ext-vector reads element 0 whatever the element is)
-            const float4_vec v = __builtin_bit_cast(
-                float4_vec, __builtin_amdgcn_raw_buffer_load_b128(
-                                x_buffer, first + q * 16, 0, 0));
-            xs[j][4 * q + 0] = v.x;
-            xs[j][4 * q + 1] = v.y;
-            xs[j][4 * q + 2] = v.z;
-            xs[j][4 * q + 3] = v.w;
+        for (int j = 0; j < kSegments; ++j) {
+            const unsigned first = (thread + kThreads * j) * (kSegment * 4);
+#pragma unroll
+            for (int q = 0; q < kSegment / 4; ++q) {
+                // (the whole vector is cast at once: a bit cast of ONE
+                // element of an ext-vector reads element 0 whatever the
+                // element is)
+                const float4_vec v = __builtin_bit_cast(
+                    float4_vec, __builtin_amdgcn_raw_buffer_load_b128(
+                                    x_buffer, first + q * 16, 0, 0));
+                xs[r][j][4 * q + 0] = v.x;
+                xs[r][j][4 * q + 1] = v.y;
+                xs[r][j][4 * q + 2] = v.z;
+                xs[r][j][4 * q + 3] = v.w;
+            }
         }
     }
 
@@ -356,7 +365,7 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
         for (int row = 0; row < kLook - 1; ++row) {
             look_up(row);
         }
-        float acc[kSegments][kRows];
+        float acc[kX][kSegments][kRows];
 #pragma unroll
         for (int row = 0; row < kRows; ++row) {
             if (row + kLook - 1 < kRows) {
@@ -365,41 +374,60 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < kSegments; ++j) {
-                float even = 0.0F;
-                float odd = 0.0F;
+                float even[kX];
+                float odd[kX];
+#pragma unroll
+                for (int r = 0; r < kX; ++r) {
+                    even[r] = 0.0F;
+                    odd[r] = 0.0F;
+                }
 #pragma unroll
                 for (int p = 0; p < 4; ++p) {
                     const float2 pair = levels[row % kLook][j][p];
-                    even += xs[j][2 * p] * pair.x;
-                    odd += xs[j][2 * p + 1] * pair.y;
+#pragma unroll
+                    for (int r = 0; r < kX; ++r) {
+                        even[r] += xs[r][j][2 * p] * pair.x;
+                        odd[r] += xs[r][j][2 * p + 1] * pair.y;
+                    }
                 }
-                acc[j][row] = even + odd;
+#pragma unroll
+                for (int r = 0; r < kX; ++r) {
+                    acc[r][j][row] = even[r] + odd[r];
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
 
         // Block sums (8 lanes), times the block's scale, then the stripes, the
         // 16-lane DPP row and the wavefront's four rows.
-        float total = 0.0F;
+        float scale[kSegments];
 #pragma unroll
         for (int j = 0; j < kSegments; ++j) {
-            // after log2(kRows) transposed steps a lane holds ONE row's sum
-            // over kRows lanes; plain steps take it to the block's 8 lanes
-            transposed_step<1, kRows / 2>(acc[j], lane);
-            transposed_step<2, kRows / 4>(acc[j], lane);
-            transposed_step<4, kRows / 8>(acc[j], lane);
-            float scale = current.scales[j];
+            scale[j] = current.scales[j];
             if constexpr (kDoubleQuantized) {
-                scale = double_quantized_scale_from_factor(
-                    factor[current.scale_codes[j] & 0xFFU], scale,
+                scale[j] = double_quantized_scale_from_factor(
+                    factor[current.scale_codes[j] & 0xFFU], scale[j],
                     current.offset);
             }
-            total += acc[j][0] * scale;
         }
-        total += dpp_xor<8>(total);
-        total = sum_over_rows(total);
-        if (lane < kRows) {
-            partial[iteration][wave][my_row] = total;
+#pragma unroll
+        for (int r = 0; r < kX; ++r) {
+            float total = 0.0F;
+#pragma unroll
+            for (int j = 0; j < kSegments; ++j) {
+                // after log2(kRows) transposed steps a lane holds ONE row's
+                // sum over kRows lanes; plain steps take it to the block's 8
+                // lanes
+                transposed_step<1, kRows / 2>(acc[r][j], lane);
+                transposed_step<2, kRows / 4>(acc[r][j], lane);
+                transposed_step<4, kRows / 8>(acc[r][j], lane);
+                total += acc[r][j][0] * scale[j];
+            }
+            total += dpp_xor<8>(total);
+            total = sum_over_rows(total);
+            if (lane < kRows) {
+                partial[iteration][wave][my_row][r] = total;
+            }
         }
     };
 
@@ -425,10 +453,11 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
     // has been parked.  The eight wavefront partials of a row are added in
     // wavefront order.
     __syncthreads();
-    for (unsigned index = thread; index < iterations * kRows;
+    for (unsigned index = thread; index < iterations * kRows * kX;
          index += kThreads) {
-        const unsigned iteration = index / kRows;
-        const unsigned value = index % kRows;
+        const unsigned iteration = index / (kRows * kX);
+        const unsigned value = index / kX % kRows;
+        const unsigned r = index % kX;
         const unsigned batch_index = first_batch + iteration * stride;
         // the member's target per lane: a chain of selects over kernel
         // arguments
@@ -442,19 +471,20 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
             }
         }
         const unsigned o = (batch_index - target.first_batch) * kRows + value;
-        if (batch_index < batch_count && o < target.output_width) {
+        if (batch_index < batch_count && o < target.output_width &&
+            r < x_rows) {
             float sum = 0.0F;
 #pragma unroll
             for (int w = 0; w < kWaves; ++w) {
-                sum += partial[iteration][w][value];
+                sum += partial[iteration][w][value][r];
             }
             if (target.bias != nullptr) {
                 sum += target.bias[o];
             }
             if (!kGrouped && lora.reduced != nullptr) {
-                sum += lora_term(lora, 0, o);
+                sum += lora_term(lora, r, o);
             }
-            target.y[o] = sum;
+            target.y[r * target.output_width + o] = sum;
         }
     }
 }
@@ -481,16 +511,20 @@ struct Request {
     std::size_t capacity;
 };
 
-template <int kSegments, bool kDoubleQuantized, int kMembers>
+template <int kX, int kSegments, bool kDoubleQuantized, int kMembers>
 void launch_instance(const LinearProblem* problems, std::size_t count,
                      const Request& request) {
     constexpr int kDepth = RTHIP_GEMV1_DEPTH;
     // A compute unit keeps about 32 KB of loads in flight (its vector L1):
     // a batch should stay well below that, so wider rows take fewer of them.
+    // (With four rows of x and three stripes the thread's slice of x alone
+    // is 96 registers: two weight rows per batch.)
     constexpr int kRows =
-        kSegments == 1 ? 8 : (kSegments == 2 ? 4 : RTHIP_GEMV1_WIDE_ROWS);
-    constexpr int kLook = kSegments == 1 ? RTHIP_GEMV1_LOOK : 2;
-    constexpr unsigned kMaxIterations = kParkedRows / kRows;
+        kSegments == 1 ? 8
+                       : (kSegments == 2 ? 4
+                                         : (kX == 4 ? 2 : RTHIP_GEMV1_WIDE_ROWS));
+    constexpr int kLook = kSegments == 1 ? (kX == 4 ? 2 : RTHIP_GEMV1_LOOK) : 2;
+    constexpr unsigned kMaxIterations = kParkedRows / (kRows * kX);
     const LinearProblem& first = problems[0];
     OneRowRest<kMembers> rest{};
     OneRowSource sources[kMembers];
@@ -542,21 +576,21 @@ void launch_instance(const LinearProblem* problems, std::size_t count,
         constexpr bool kWhole = decltype(whole_groups)::value;
         if (request.name != nullptr) {
             std::snprintf(request.name, request.capacity,
-                          "gemv1_forward_kernel<%d, %d, %d, %d, %s, %s, %d>",
-                          kSegments, kRows, kDepth, kLook,
+                          "gemv1_forward_kernel<%d, %d, %d, %d, %d, %s, %s, %d>",
+                          kX, kSegments, kRows, kDepth, kLook,
                           kDoubleQuantized ? "true" : "false",
                           kWhole ? "true" : "false", kMembers);
             return;
         }
-        gemv1_forward_kernel<kSegments, kRows, kDepth, kLook, kDoubleQuantized,
-                             kWhole, kMembers>
+        gemv1_forward_kernel<kX, kSegments, kRows, kDepth, kLook,
+                             kDoubleQuantized, kWhole, kMembers>
             <<<blocks, kThreads, 0, request.stream>>>(
                 first.activations, head.codes, head.primary_scales,
                 static_cast<unsigned>(first.input_width), head.code_bytes,
                 head.primary_bytes, iterations, head.secondary_scales,
                 head.secondary_bytes, head.offset,
-                first.weight.second_level_shift, batch_count, rest,
-                first.lora);
+                first.weight.second_level_shift, batch_count,
+                static_cast<unsigned>(first.rows), rest, first.lora);
     };
     if constexpr (kDoubleQuantized) {
         const std::size_t batch_blocks =
@@ -570,18 +604,40 @@ void launch_instance(const LinearProblem* problems, std::size_t count,
     launch(std::false_type{});
 }
 
-template <bool kDoubleQuantized, int kMembers>
+template <int kX, bool kDoubleQuantized, int kMembers>
 void launch_segments(const LinearProblem* problems, std::size_t count,
-                     const Request& stream) {
+                     const Request& request) {
     switch (segments_per_thread(problems[0])) {
     case 1:
-        launch_instance<1, kDoubleQuantized, kMembers>(problems, count, stream);
+        launch_instance<kX, 1, kDoubleQuantized, kMembers>(problems, count,
+                                                           request);
         break;
     case 2:
-        launch_instance<2, kDoubleQuantized, kMembers>(problems, count, stream);
+        launch_instance<kX, 2, kDoubleQuantized, kMembers>(problems, count,
+                                                           request);
         break;
     default:
-        launch_instance<3, kDoubleQuantized, kMembers>(problems, count, stream);
+        launch_instance<kX, 3, kDoubleQuantized, kMembers>(problems, count,
+                                                           request);
+        break;
+    }
+}
+
+template <bool kDoubleQuantized, int kMembers>
+void launch_rows(const LinearProblem* problems, std::size_t count,
+                 const Request& request) {
+    switch (problems[0].rows) {
+    case 1:
+        launch_segments<1, kDoubleQuantized, kMembers>(problems, count,
+                                                       request);
+        break;
+    case 2:
+        launch_segments<2, kDoubleQuantized, kMembers>(problems, count,
+                                                       request);
+        break;
+    default:
+        launch_segments<4, kDoubleQuantized, kMembers>(problems, count,
+                                                       request);
         break;
     }
 }
@@ -590,9 +646,9 @@ template <int kMembers>
 void launch_encoding(const LinearProblem* problems, std::size_t count,
                      const Request& stream) {
     if (problems[0].weight.encoding == 0) {
-        launch_segments<false, kMembers>(problems, count, stream);
+        launch_rows<false, kMembers>(problems, count, stream);
     } else {
-        launch_segments<true, kMembers>(problems, count, stream);
+        launch_rows<true, kMembers>(problems, count, stream);
     }
 }
 
@@ -604,10 +660,12 @@ bool gemv1_forward_supports(const LinearProblem& p) {
     // Offsets are 32-bit and run up to a few batches past an array's end.
     constexpr std::size_t kMaxBytes = std::size_t{1} << 31;
     const std::size_t weights = p.output_width * p.input_width;
-    return p.rows == 1 && p.block_shift == kBlockShift &&
+    return p.rows >= 1 && p.rows <= kGemvMaxRows &&
+           p.block_shift == kBlockShift &&
            p.output_width % kMaxRows == 0 &&
            p.input_width % (std::size_t{1} << kBlockShift) == 0 &&
            p.input_width <= kMaxWidth && weights / 2 < kMaxBytes &&
+           p.rows * p.output_width < (1ULL << 32) &&
            reinterpret_cast<std::uintptr_t>(p.weight.codes) % 4 == 0 &&
            reinterpret_cast<std::uintptr_t>(p.activations) % 16 == 0;
 }

@@ -261,3 +261,27 @@ class _Fake:
 
     def data_ptr(self):
         return self._address
+
+
+def test_kernel_name_follows_the_launch(package, library):
+    """rthip_nf4_forward_kernel_name: the instance per shape, as a profiler
+    prints it (bench.py matches stored counter summaries against it)."""
+    name = lambda *a, **k: library.forward_kernel_name(*a, **k)  # noqa: E731
+    fp32 = package.SCALE_FLOAT32
+    nested = package.SCALE_DOUBLE_QUANTIZED_UINT8
+    assert name(1, 4096, [4096], 64, fp32) == \
+        "gemv1_forward_kernel<1, 1, 8, 2, 4, false, false, 1>"
+    assert name(1, 4096, [4096] * 3, 64, fp32) == \
+        "gemv1_forward_kernel<1, 1, 8, 2, 4, false, false, 4>"
+    assert name(1, 4096, [11008, 11008], 64, nested, 256) == \
+        "gemv1_forward_kernel<1, 1, 8, 2, 4, true, true, 4>"
+    assert name(1, 11008, [4096], 64, nested, 256) == \
+        "gemv1_forward_kernel<1, 3, 4, 2, 2, true, false, 1>"
+    assert name(4, 11008, [4096], 64, fp32) == \
+        "gemv1_forward_kernel<4, 3, 2, 2, 2, false, false, 1>"
+    assert name(3, 8192, [4096], 64, fp32) == \
+        "gemv1_forward_kernel<4, 2, 4, 2, 2, false, false, 1>"
+    assert name(5, 4096, [4096], 64, fp32) == ""
+    assert name(1, 4096, [4100], 64, fp32) == ""
+    with pytest.raises(package.InvalidArgument):
+        name(1, 4096, [], 64, fp32)
