@@ -4,7 +4,14 @@ reference (Hip = 4, the registry case, the validated-once dispatcher), links
 it with this repository's adapter and builds the reference's
 tests/core/backend/test_quantized_linear_backend.cpp (ExecutionBackend::Hip in
 its accelerator loop, :382-453,502-513) and test_backend.cpp (identity,
-diagnostics, thread-local selection: :172-240,278-395).
+diagnostics, thread-local selection: :172-240,278-395).  The same script
+sends `Linear::forward` of a packed layer with a low-rank adapter through one
+fused graph node on hip, adds RT_BACKEND_HIP to the C ABI bridge, and builds
+the reference's tests/nn/test_quantized_linear.cpp and
+tests/core/test_quantization.cpp with hip in the place of their optional
+accelerator (and the former's CPU-only tests repeated on hip), plus two
+programs of this repository: the fused layer against the reference's
+composition on the CPU backend, and the bridge's identity checks.
 
 Without a GPU they run against the host-only test runtime
 (tests/fakes/fake_rthip.cpp), the role tests/fakes/fake_pjrt_tpu.cpp plays for
@@ -77,18 +84,70 @@ def test_identity_diagnostics_and_thread_local_selection(programs, library):
     assert "backend tests passed" in done.stdout
 
 
+def test_nn_tests_run_on_hip(programs):
+    """tests/nn/test_quantized_linear.cpp: the graph of 2 nodes / 20 elements
+    and the VJP (:140-183), the packed bytes across an Adam step and the
+    merged export (:185-267) repeated on hip, and Module::to to hip and back
+    (:269-318); the program prints a line when the hip copies ran."""
+    done = run("quantized_linear_tests", FAKE)
+    assert done.returncode == 0, done.stderr
+    assert "quantized Linear tests ran on hip" in done.stdout
+    assert "quantized Linear tests passed" in done.stdout
+    without = run("quantized_linear_tests", "/nonexistent/librthip.so")
+    assert without.returncode == 0, without.stderr
+    assert "ran on hip" not in without.stdout
+
+
+def test_quantization_transfer_keeps_bytes_on_hip(programs):
+    # tests/core/test_quantization.cpp:400-435 with hip as the accelerator
+    done = run("quantization_tests", FAKE)
+    assert done.returncode == 0, done.stderr
+    assert "NF4 quantization tests passed" in done.stdout
+
+
+def test_fused_linear_equals_the_reference_composition(programs):
+    done = run("fused_linear_tests", FAKE,
+               RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1")
+    assert done.returncode == 0, done.stderr
+    assert "fused Linear tests passed" in done.stdout
+    skipped = run("fused_linear_tests", "/nonexistent/librthip.so")
+    assert skipped.returncode == 0 and "skipped" in skipped.stdout
+    gate = run("fused_linear_tests", "/nonexistent/librthip.so",
+               RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1")
+    assert gate.returncode == 1
+
+
+def test_c_abi_backend_identity(programs):
+    done = run("c_api_identity_tests", FAKE,
+               RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1")
+    assert done.returncode == 0, done.stderr
+    assert "hip backend selected through the C ABI" in done.stdout
+    refused = run("c_api_identity_tests", "/nonexistent/librthip.so")
+    assert refused.returncode == 0, refused.stderr
+    assert "hip backend refused through the C ABI" in refused.stdout
+    gate = run("c_api_identity_tests", "/nonexistent/librthip.so",
+               RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1")
+    assert gate.returncode == 1
+
+
 @pytest.mark.gpu
 def test_reference_tests_on_the_device():
     """The programs built in the build container, against the real library
     on an MI355X: the reference's accelerator test with hip required (its
-    resident == logical assertion holds because HBM is host-visible), and its
-    backend test."""
+    resident == logical assertion holds because HBM is host-visible), its
+    backend, nn and quantization tests, the fused layer and the C ABI
+    bridge."""
     required = os.path.join(BUILD,
                             "quantized_linear_backend_tests_hip_required")
     if not os.path.exists(required):
         pytest.skip("tests/in_tree/build was not built (no reference tree)")
     for program in ("quantized_linear_backend_tests_hip_required",
-                    "backend_tests"):
-        done = run(program, REAL, RIFTCO_TRANSFORMER_HIP_REJECT_TEST_PLUGIN="1")
-        assert done.returncode == 0, done.stdout + done.stderr
+                    "backend_tests", "quantized_linear_tests",
+                    "quantization_tests", "fused_linear_tests",
+                    "c_api_identity_tests"):
+        done = run(program, REAL, RIFTCO_TRANSFORMER_HIP_REJECT_TEST_PLUGIN="1",
+                   RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1")
+        assert done.returncode == 0, program + done.stdout + done.stderr
         assert "tests passed" in done.stdout
+        if program == "quantized_linear_tests":
+            assert "quantized Linear tests ran on hip" in done.stdout
