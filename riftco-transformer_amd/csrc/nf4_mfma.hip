@@ -13,8 +13,9 @@
 // the matrix cores read.
 //
 // Tiling.  A workgroup of four wavefronts computes a 128 x 128 output tile in
-// steps of 32 along the contraction; each wavefront owns a 64 x 64 quadrant as
-// 2 x 2 blocks of v_mfma_f32_32x32x2_f32.  Both LDS tiles are laid out
+// steps of 32 along the contraction (or eight wavefronts a 256 x 128 tile,
+// see Tile); each wavefront owns a 64 x 64 part as 2 x 2 blocks of
+// v_mfma_f32_32x32x2_f32.  Both LDS tiles are laid out
 // [row-or-column][contraction] with a padded stride of 36 floats, so that one
 // ds_read_b128 per lane fetches four consecutive contraction values; lanes
 // 0-31 take offsets 0..3 and lanes 32-63 offsets 4..7 of each group of eight,
@@ -52,16 +53,32 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int kThreads = 256;
-constexpr int kTileM = 128;       // output rows per workgroup
 constexpr int kTileN = 128;       // output columns per workgroup
 constexpr int kTileK = 32;        // contraction per step
 constexpr int kStride = 36;       // padded LDS row stride in floats
-constexpr int kChunk = 16;        // weights decoded per thread per step
 constexpr unsigned kFlushSteps = 8;  // steps per first-level accumulation
-// LDS of a workgroup: two buffers x (activation tile + weight tile)
-constexpr std::size_t kTileBytes =
-    std::size_t{2} * (kTileM + kTileN) * kStride * sizeof(float);
+
+// The two tile shapes.  Tall: 256 output rows per workgroup of eight
+// wavefronts, one workgroup per compute unit -- a weight tile is decoded once
+// per 256 rows of x.  Otherwise 128 rows per workgroup of four wavefronts, two
+// workgroups per compute unit.  A wavefront owns 64 x 64 in both.
+template <bool kTall>
+struct Tile {
+    static constexpr int kThreads = kTall ? 512 : 256;
+    static constexpr int kTileM = kTall ? 256 : 128;  // output rows
+    // weights decoded per thread per step (the 128 x 32 weight tile over the
+    // workgroup's threads), and the 32-bit words of codes they come in
+    static constexpr int kChunk = kTileN * kTileK / kThreads;
+    static constexpr int kWords = kChunk / 8;
+    static constexpr int kWorkgroupsPerUnit = kTall ? 1 : 2;
+    // workgroups the device holds at once
+    static constexpr unsigned kPlaces = kTall ? 256 : 512;
+    static constexpr unsigned kActivationFloats = kTileM * kStride;
+    static constexpr unsigned kBufferFloats = (kTileM + kTileN) * kStride;
+    // LDS of a workgroup: two buffers x (activation tile + weight tile)
+    static constexpr std::size_t kTileBytes =
+        std::size_t{2} * kBufferFloats * sizeof(float);
+};
 
 struct GemmShape {
     unsigned rows;         // M
@@ -72,21 +89,24 @@ struct GemmShape {
 
 
 // Registers holding one step's global loads of a thread.
+template <bool kTall>
 struct Staged {
     float4 a[4];
-    uint2 codes;
+    unsigned codes[Tile<kTall>::kWords];
     float scale;
 };
 
+template <bool kTall>
 __device__ __forceinline__ void load_activation_tile(
-    Staged& staged, const float* __restrict__ activations,
+    Staged<kTall>& staged, const float* __restrict__ activations,
     const GemmShape& shape, unsigned row0, unsigned k0
 ) {
     const unsigned thread = threadIdx.x;
     const unsigned column = (thread % 8) * 4;
 #pragma unroll
     for (int pass = 0; pass < 4; ++pass) {
-        const unsigned row = row0 + thread / 8 + 32 * pass;
+        const unsigned row =
+            row0 + thread / 8 + (Tile<kTall>::kThreads / 8) * pass;
         staged.a[pass] = row < shape.rows
             ? *reinterpret_cast<const float4*>(
                   activations +
@@ -96,95 +116,115 @@ __device__ __forceinline__ void load_activation_tile(
     }
 }
 
+template <bool kTall>
 __device__ __forceinline__ void store_activation_tile(
-    const Staged& staged, float* __restrict__ tile
+    const Staged<kTall>& staged, float* __restrict__ tile
 ) {
     const unsigned thread = threadIdx.x;
     const unsigned column = (thread % 8) * 4;
 #pragma unroll
     for (int pass = 0; pass < 4; ++pass) {
-        const unsigned row = thread / 8 + 32 * pass;
+        const unsigned row = thread / 8 + (Tile<kTall>::kThreads / 8) * pass;
         *reinterpret_cast<float4*>(tile + row * kStride + column) =
             staged.a[pass];
     }
 }
 
-// Forward weight tile: output columns n0..n0+127 are weight rows; the step's
-// 32 contraction values are 16 contiguous code bytes of each row.  Thread t
-// decodes 16 weights of row t / 2.
-template <bool kDoubleQuantized>
-__device__ __forceinline__ void load_weight_tile_forward(
-    Staged& staged, const Nf4WeightView& weight, const GemmShape& shape,
-    unsigned n0, unsigned k0, unsigned block_shift
+// The codes and the block scale of a thread's chunk, which starts at weight
+// `flat` (row-major index); a chunk outside the weight decodes to zeros.
+template <bool kTall, bool kDoubleQuantized>
+__device__ __forceinline__ void load_chunk(
+    Staged<kTall>& staged, const Nf4WeightView& weight, bool inside,
+    std::size_t flat, unsigned block_shift
 ) {
-    const unsigned thread = threadIdx.x;
-    const unsigned n = n0 + thread / 2;
-    if (n < shape.columns) {
-        const std::size_t flat =
-            static_cast<std::size_t>(n) * shape.input_width + k0 +
-            (thread % 2) * kChunk;
-        staged.codes =
-            *reinterpret_cast<const uint2*>(weight.codes + (flat >> 1));
+    if (inside) {
+        const unsigned* const source =
+            reinterpret_cast<const unsigned*>(weight.codes + (flat >> 1));
+        if constexpr (Tile<kTall>::kWords == 2) {
+            const uint2 both = *reinterpret_cast<const uint2*>(source);
+            staged.codes[0] = both.x;
+            staged.codes[1] = both.y;
+        } else {
+            staged.codes[0] = *source;
+        }
         staged.scale =
             load_block_scale<kDoubleQuantized>(weight, flat >> block_shift);
     } else {
-        staged.codes = make_uint2(0x77777777U, 0x77777777U);
+#pragma unroll
+        for (int w = 0; w < Tile<kTall>::kWords; ++w) {
+            staged.codes[w] = 0x77777777U;
+        }
         staged.scale = 0.0F;
     }
+}
+
+// Forward weight tile: output columns n0..n0+127 are weight rows; the step's
+// 32 contraction values are 16 contiguous code bytes of each row, which two
+// (four) threads share in chunks of 16 (8) weights.
+template <bool kTall, bool kDoubleQuantized>
+__device__ __forceinline__ void load_weight_tile_forward(
+    Staged<kTall>& staged, const Nf4WeightView& weight, const GemmShape& shape,
+    unsigned n0, unsigned k0, unsigned block_shift
+) {
+    constexpr unsigned kChunk = Tile<kTall>::kChunk;
+    constexpr unsigned kPerRow = kTileK / kChunk;
+    const unsigned thread = threadIdx.x;
+    const unsigned n = n0 + thread / kPerRow;
+    load_chunk<kTall, kDoubleQuantized>(
+        staged, weight, n < shape.columns,
+        static_cast<std::size_t>(n) * shape.input_width + k0 +
+            (thread % kPerRow) * kChunk,
+        block_shift);
 }
 
 // Backward weight tile: the step's 32 contraction values are weight rows
 // c0..c0+31; output columns k0..k0+127 are contiguous within each row.
-// Thread t decodes 16 weights of row c0 + t % 32.
-template <bool kDoubleQuantized>
+// Thread t decodes a chunk of row c0 + t % 32.
+template <bool kTall, bool kDoubleQuantized>
 __device__ __forceinline__ void load_weight_tile_backward(
-    Staged& staged, const Nf4WeightView& weight, const GemmShape& shape,
+    Staged<kTall>& staged, const Nf4WeightView& weight, const GemmShape& shape,
     unsigned k0, unsigned c0, unsigned block_shift
 ) {
     const unsigned thread = threadIdx.x;
-    const unsigned column = k0 + (thread / 32) * kChunk;
-    if (column < shape.columns) {
-        const std::size_t flat =
-            static_cast<std::size_t>(c0 + thread % 32) * shape.input_width +
-            column;
-        staged.codes =
-            *reinterpret_cast<const uint2*>(weight.codes + (flat >> 1));
-        staged.scale =
-            load_block_scale<kDoubleQuantized>(weight, flat >> block_shift);
-    } else {
-        staged.codes = make_uint2(0x77777777U, 0x77777777U);
-        staged.scale = 0.0F;
-    }
+    const unsigned column = k0 + (thread / 32) * Tile<kTall>::kChunk;
+    load_chunk<kTall, kDoubleQuantized>(
+        staged, weight, column < shape.columns,
+        static_cast<std::size_t>(c0 + thread % 32) * shape.input_width +
+            column,
+        block_shift);
 }
 
+template <bool kTall>
 __device__ __forceinline__ void decode_chunk(
-    const Staged& staged, const float* __restrict__ table, float (&out)[16]
+    const Staged<kTall>& staged, const float* __restrict__ table,
+    float (&out)[Tile<kTall>::kChunk]
 ) {
 #pragma clang fp contract(off)
-    const unsigned words[2] = {staged.codes.x, staged.codes.y};
 #pragma unroll
-    for (int w = 0; w < 2; ++w) {
+    for (int w = 0; w < Tile<kTall>::kWords; ++w) {
 #pragma unroll
         for (int n = 0; n < 8; ++n) {
             out[8 * w + n] =
-                table[(words[w] >> (4 * n)) & 0xFU] * staged.scale;
+                table[(staged.codes[w] >> (4 * n)) & 0xFU] * staged.scale;
         }
     }
 }
 
-template <bool kBackward>
+template <bool kTall, bool kBackward>
 __device__ __forceinline__ void store_weight_tile(
-    const Staged& staged, const float* __restrict__ table,
+    const Staged<kTall>& staged, const float* __restrict__ table,
     float* __restrict__ tile
 ) {
+    constexpr unsigned kChunk = Tile<kTall>::kChunk;
+    constexpr unsigned kPerRow = kTileK / kChunk;
     const unsigned thread = threadIdx.x;
-    float decoded[16];
-    decode_chunk(staged, table, decoded);
+    float decoded[kChunk];
+    decode_chunk<kTall>(staged, table, decoded);
     if constexpr (!kBackward) {
         float* destination =
-            tile + (thread / 2) * kStride + (thread % 2) * kChunk;
+            tile + (thread / kPerRow) * kStride + (thread % kPerRow) * kChunk;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < static_cast<int>(kChunk) / 4; ++q) {
             *reinterpret_cast<float4*>(destination + 4 * q) = make_float4(
                 decoded[4 * q], decoded[4 * q + 1], decoded[4 * q + 2],
                 decoded[4 * q + 3]);
@@ -194,7 +234,7 @@ __device__ __forceinline__ void store_weight_tile(
         float* destination =
             tile + ((thread / 32) * kChunk) * kStride + thread % 32;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < static_cast<int>(kChunk); ++i) {
             destination[i * kStride] = decoded[i];
         }
     }
@@ -202,9 +242,9 @@ __device__ __forceinline__ void store_weight_tile(
 
 // One segment: contraction values [k_begin, k_end) of the output tile at
 // (row0, col0).  `partial` null: the segment is the whole contraction and the
-// tile goes to `result` with bias and adapter term; otherwise the 128 x 128
+// tile goes to `result` with bias and adapter term; otherwise the tile's
 // partial sums go to `partial`.
-template <bool kDoubleQuantized, bool kBackward>
+template <bool kTall, bool kDoubleQuantized, bool kBackward>
 __device__ __forceinline__ void gemm_segment(
     const float* __restrict__ activations, const Nf4WeightView& weight,
     const float* __restrict__ bias, float* __restrict__ result,
@@ -221,8 +261,8 @@ __device__ __forceinline__ void gemm_segment(
     // tiles: [buffer][activations | weights][row or column][k], two buffers.
     // A step computes from one buffer while the next step's tiles are written
     // into the other, so the writes need no barrier of their own.
-    constexpr unsigned kTileFloats = kTileM * kStride;
-    constexpr unsigned kBufferFloats = 2 * kTileFloats;
+    constexpr unsigned kTileFloats = Tile<kTall>::kActivationFloats;
+    constexpr unsigned kBufferFloats = Tile<kTall>::kBufferFloats;
     const unsigned a_offset =
         (wave_m * 64 + lane % 32) * kStride + 4 * (lane / 32);
     const unsigned b_offset = kTileFloats +
@@ -248,21 +288,22 @@ __device__ __forceinline__ void gemm_segment(
     }
     unsigned steps_since_flush = 0;
 
-    Staged staged;
+    Staged<kTall> staged;
     const auto load_step = [&](unsigned k) {
-        load_activation_tile(staged, activations, shape, row0, k);
+        load_activation_tile<kTall>(staged, activations, shape, row0, k);
         if constexpr (!kBackward) {
-            load_weight_tile_forward<kDoubleQuantized>(
+            load_weight_tile_forward<kTall, kDoubleQuantized>(
                 staged, weight, shape, col0, k, block_shift);
         } else {
-            load_weight_tile_backward<kDoubleQuantized>(
+            load_weight_tile_backward<kTall, kDoubleQuantized>(
                 staged, weight, shape, col0, k, block_shift);
         }
     };
     const auto store_step = [&](unsigned buffer) {
         float* const target = tiles + buffer * kBufferFloats;
-        store_activation_tile(staged, target);
-        store_weight_tile<kBackward>(staged, table, target + kTileFloats);
+        store_activation_tile<kTall>(staged, target);
+        store_weight_tile<kTall, kBackward>(staged, table,
+                                            target + kTileFloats);
     };
     // Matrix instructions of contraction values [kk, kk + 8) of the step.
     const auto multiply = [&](const float* a_fragment,
@@ -364,7 +405,7 @@ __device__ __forceinline__ void gemm_segment(
 
     // Accumulator element e of lane l is output row 8*(e/4) + 4*(l/32) + e%4,
     // column l%32 of its 32 x 32 block.
-    if (partial != nullptr) {  // uniform; layout [kTileM][kTileN]
+    if (partial != nullptr) {  // uniform; layout [tile rows][kTileN]
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -433,13 +474,16 @@ __device__ __forceinline__ void gemm_segment(
     }
 }
 
-template <bool kDoubleQuantized, bool kBackward>
-__global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
+template <bool kTall, bool kDoubleQuantized, bool kBackward>
+__global__ __launch_bounds__(Tile<kTall>::kThreads,
+                             Tile<kTall>::kWorkgroupsPerUnit)
+void mfma_gemm_kernel(
     const float* __restrict__ activations, Nf4WeightView weight,
     const float* __restrict__ bias, float* __restrict__ result,
     float* __restrict__ workspace, GemmShape shape, TilePlan plan,
     unsigned block_shift, LoraEpilogue lora
 ) {
+    constexpr unsigned kTileM = Tile<kTall>::kTileM;
     // two buffers of an activation and a weight tile each: more than the 64
     // KB a static array may have, so sized at launch
     extern __shared__ __attribute__((aligned(16))) float tiles[];
@@ -465,7 +509,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
                 : workspace +
                       static_cast<std::size_t>(group * 2 + segment) * kTileM *
                           kTileN;
-        gemm_segment<kDoubleQuantized, kBackward>(
+        gemm_segment<kTall, kDoubleQuantized, kBackward>(
             activations, weight, bias, result, partial, shape, block_shift,
             lora, tiles, table, (tile / plan.tiles_n) * kTileM,
             (tile % plan.tiles_n) * kTileN, first_step * kTileK,
@@ -478,6 +522,7 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_gemm_kernel(
 // on, in ascending workgroup order, plus bias and adapter term.  One thread
 // per output element: blockIdx.x is the tile among the unit-dealt ones,
 // blockIdx.y a run of 256 elements of it.
+template <unsigned kTileM>
 __global__ __launch_bounds__(256) void gemm_parts_kernel(
     const float* __restrict__ workspace, const float* __restrict__ bias,
     float* __restrict__ result, GemmShape shape, TilePlan plan,
@@ -514,10 +559,13 @@ __global__ __launch_bounds__(256) void gemm_parts_kernel(
     result[static_cast<std::size_t>(row) * shape.columns + column] = sum;
 }
 
-template <bool kDoubleQuantized, bool kBackward>
-hipError_t launch_encoding(const LinearProblem& p, const GemmShape& shape,
-                           hipStream_t stream) {
-    const auto kernel = mfma_gemm_kernel<kDoubleQuantized, kBackward>;
+template <bool kTall, bool kDoubleQuantized, bool kBackward>
+hipError_t launch_tiles(const LinearProblem& p, const GemmShape& shape,
+                        hipStream_t stream) {
+    constexpr unsigned kTileM = Tile<kTall>::kTileM;
+    constexpr unsigned kThreads = Tile<kTall>::kThreads;
+    constexpr std::size_t kTileBytes = Tile<kTall>::kTileBytes;
+    const auto kernel = mfma_gemm_kernel<kTall, kDoubleQuantized, kBackward>;
     const unsigned tiles_m = (shape.rows + kTileM - 1) / kTileM;
     const unsigned tiles_n = (shape.columns + kTileN - 1) / kTileN;
     const unsigned tiles = tiles_m * tiles_n;
@@ -526,7 +574,7 @@ hipError_t launch_encoding(const LinearProblem& p, const GemmShape& shape,
     plan.steps = (shape.contraction + kTileK - 1) / kTileK;
     const unsigned groups =
         plan_tiles(plan, tiles, kTileM * kTileN * sizeof(float),
-                   kStreamWorkspaceBytes);
+                   kStreamWorkspaceBytes, Tile<kTall>::kPlaces);
     WorkspaceLease lease;  // held until both launches are enqueued
     if (groups != 0) {
         if (const hipError_t status = lease_stream_workspace(stream, &lease);
@@ -546,10 +594,38 @@ hipError_t launch_encoding(const LinearProblem& p, const GemmShape& shape,
         p.block_shift, p.lora);
     if (groups != 0) {
         const dim3 grid(tiles - plan.whole_tiles, kTileM * kTileN / 256);
-        gemm_parts_kernel<<<grid, 256, 0, stream>>>(
+        gemm_parts_kernel<kTileM><<<grid, 256, 0, stream>>>(
             workspace, p.bias, p.result, shape, plan, p.lora);
     }
     return hipSuccess;
+}
+
+// The tall tile halves the decode work per product but leaves a compute unit
+// one workgroup, whose barriers nothing covers.  Measured at 2048 rows: the
+// forward wins where its tiles fill the device in whole rounds (4096 x 4096:
+// 123-124 -> 127-128 TFLOP/s) and is level where leftover tiles are dealt in
+// runs (11008 x 4096); the input backward, whose weight tile is written
+// transposed word by word, loses (W 11008 x 4096: 119 -> 116).  So: forward,
+// whole rounds.
+bool tall_tiles_pay(const GemmShape& shape) {
+    const unsigned tall_rows = Tile<true>::kTileM;
+    const unsigned tiles_m = (shape.rows + tall_rows - 1) / tall_rows;
+    const unsigned tiles_n = (shape.columns + kTileN - 1) / kTileN;
+    const unsigned last_row_fill = shape.rows - (tiles_m - 1) * tall_rows;
+    return shape.rows >= tall_rows && last_row_fill > tall_rows / 2 &&
+           (tiles_m * tiles_n) % Tile<true>::kPlaces == 0;
+}
+
+template <bool kDoubleQuantized, bool kBackward>
+hipError_t launch_encoding(const LinearProblem& p, const GemmShape& shape,
+                           hipStream_t stream) {
+    if constexpr (!kBackward) {
+        if (tall_tiles_pay(shape)) {
+            return launch_tiles<true, kDoubleQuantized, false>(p, shape,
+                                                               stream);
+        }
+    }
+    return launch_tiles<false, kDoubleQuantized, kBackward>(p, shape, stream);
 }
 
 template <bool kBackward>
@@ -574,7 +650,7 @@ bool common_supports(const LinearProblem& p) {
     return p.rows >= 1 && p.rows < kLimit && p.input_width < kLimit &&
            p.output_width < kLimit &&
            // tile and (tile, step) unit counts stay 32-bit
-           ((p.rows + kTileM - 1) / kTileM) *
+           ((p.rows + Tile<false>::kTileM - 1) / Tile<false>::kTileM) *
                    ((std::max(p.input_width, p.output_width) + kTileN - 1) /
                     kTileN) <
                (1ULL << 24) &&
@@ -599,7 +675,7 @@ bool mfma_input_backward_supports(const LinearProblem& p) {
     // Contraction over weight rows in steps of 32; output columns in chunks
     // of 16 within a row.
     return common_supports(p) && p.output_width % kTileK == 0 &&
-           p.input_width % kChunk == 0;
+           p.input_width % Tile<false>::kChunk == 0;
 }
 
 hipError_t launch_mfma_input_backward(const LinearProblem& p,

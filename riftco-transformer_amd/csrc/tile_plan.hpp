@@ -43,7 +43,8 @@ struct TilePlan {
     }
 };
 
-// Workgroups of 256 threads the device holds at once: two per compute unit.
+// Workgroups of 256 threads the device holds at once: two per compute unit
+// (`places` of plan_tiles unless the caller's workgroups are another size).
 constexpr unsigned kPlanPlaces = 512;
 // A run is at least this many steps, and unit dealing is not worth a second
 // kernel when the leftover tiles nearly fill the device anyway.
@@ -55,21 +56,22 @@ constexpr unsigned kPlanMinimumRunSteps = 8;
 // workspace_bytes: room for the partial tiles.
 inline unsigned plan_tiles(TilePlan& plan, unsigned tiles,
                            std::size_t slot_bytes,
-                           std::size_t workspace_bytes) {
+                           std::size_t workspace_bytes,
+                           unsigned places = kPlanPlaces) {
     plan.whole_tiles = tiles;
     plan.quotient = 0;
     plan.remainder = 0;
-    const unsigned leftover = tiles % kPlanPlaces;
-    if (leftover == 0 || leftover * 10 >= kPlanPlaces * 9 ||
+    const unsigned leftover = tiles % places;
+    if (leftover == 0 || leftover * 10 >= places * 9 ||
         plan.steps < 2 * kPlanMinimumRunSteps ||
-        static_cast<std::size_t>(kPlanPlaces) * 2 * slot_bytes >
+        static_cast<std::size_t>(places) * 2 * slot_bytes >
             workspace_bytes) {
         return 0;
     }
     const unsigned units = leftover * plan.steps;
     unsigned groups = units / kPlanMinimumRunSteps;
-    if (groups > kPlanPlaces) {
-        groups = kPlanPlaces;
+    if (groups > places) {
+        groups = places;
     }
     if (groups <= leftover) {
         return 0;  // runs of a whole tile: nothing to deal

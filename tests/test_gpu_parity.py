@@ -679,6 +679,9 @@ def test_two_host_threads_launch_on_one_stream(gpu, package, library, oracle):
     (1280, 2560, 4096, True),   # 200 tiles dealt to 512 workgroups
     (2200, 3700, 512, False),   # 522 tiles: 512 whole, 10 cut into runs
     (200, 384, 256, False),     # too few steps: whole tiles only
+    # forward in 256-row tiles (their count fills the device in whole rounds)
+    (448, 16384, 96, True),     # the second tile row three quarters full
+    (256, 32768, 64, False),    # one tile row, two steps
 ])
 def test_gemm_leftover_tiles_are_dealt_in_units(gpu, package, library, oracle,
                                                 rows, out_w, in_w,
