@@ -49,6 +49,7 @@ weights are close to uniform by construction) and block scales drawn around
 the absmax of 64 samples of N(0, 0.02), generated on the device.
 """
 import argparse
+import ctypes
 import importlib
 import json
 import os
@@ -534,13 +535,46 @@ def bench_large_launches(package, device, torch, steps):
     return results
 
 
+class Probes:
+    """librthip_probe.so: a plain streaming read and an empty launch."""
+
+    def __init__(self, path):
+        self._lib = ctypes.CDLL(path)
+        self._lib.rthip_probe_streaming_read.restype = ctypes.c_int
+        self._lib.rthip_probe_streaming_read.argtypes = [
+            ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
+        self._lib.rthip_probe_empty_launch.restype = ctypes.c_int
+        self._lib.rthip_probe_empty_launch.argtypes = [ctypes.c_void_p]
+
+    def probe_streaming_read(self, data_ptr, size, stream):
+        status = self._lib.rthip_probe_streaming_read(data_ptr, size, stream)
+        if status != 0:
+            raise RuntimeError("streaming-read probe: status %d" % status)
+
+    def probe_empty_launch(self, stream):
+        status = self._lib.rthip_probe_empty_launch(stream)
+        if status != 0:
+            raise RuntimeError("empty-launch probe: status %d" % status)
+
+
+def load_probes(package):
+    path = os.path.join(os.path.dirname(os.path.abspath(package.__file__)),
+                        "lib", "librthip_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError(
+            "%s is missing: run `make -C riftco-transformer_amd`" % path)
+    return Probes(path)
+
+
 def bench_practical_roof(package, torch, steps):
     """What the device gives a kernel that only reads: one launch of a plain
-    streaming read (rthip_probe_streaming_read) per buffer, buffers rotating
-    through more than the last-level cache, replayed as a graph exactly like
-    the decode step; and an empty launch of the same grid.  The sizes are the
-    packed payloads of the decode shapes and of the large launches."""
-    library = package.load_library()
+    streaming read (rthip_probe_streaming_read of librthip_probe.so, a
+    library of two measurement launches beside the product's) per buffer,
+    buffers rotating through more than the last-level cache, replayed as a
+    graph exactly like the decode step; and an empty launch of the same grid.
+    The sizes are the packed payloads of the decode shapes and of the large
+    launches."""
+    library = load_probes(package)
     stream = lambda: torch.cuda.current_stream().cuda_stream
     results = {"streaming_read": []}
 

@@ -41,7 +41,7 @@ extern "C" {
 #endif
 
 #define RTHIP_ABI_VERSION_MAJOR 1u
-#define RTHIP_ABI_VERSION_MINOR 8u
+#define RTHIP_ABI_VERSION_MINOR 9u
 
 typedef int32_t rthip_status;
 
@@ -427,18 +427,6 @@ rthip_status rthip_nf4_check_payload(
     const float* secondary_scales, int32_t encoding,
     uint64_t second_level_block, float offset, uint64_t element_count,
     uint64_t block_size, void* stream);
-
-/*
- * Measurement aids, no counterpart in the reference.  The first reads `bytes`
- * (a positive multiple of 16, 16-byte aligned) of device memory once with a
- * plain streaming kernel and does nothing with them: the rate the memory
- * system delivers per launch of that size, which is the practical roof of any
- * kernel that has to read the same bytes.  The second is a launch of the same
- * grid that does nothing: the fixed cost of a launch.  Both only enqueue.
- */
-rthip_status rthip_probe_streaming_read(const void* data, uint64_t bytes,
-                                        void* stream);
-rthip_status rthip_probe_empty_launch(void* stream);
 
 /*
  * Frees the scratch buffers the library keeps per (device, stream) for

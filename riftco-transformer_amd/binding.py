@@ -111,8 +111,6 @@ _PROTOTYPES = {
     "rthip_nf4_linear_input_backward_no_alloc": (
         _i32, [_ptr] + _WEIGHT + [_ptr, _u64, _u64, _u64, _u64, _ptr]),
     "rthip_release_workspaces": (_i32, [_ptr, _i32]),
-    "rthip_probe_streaming_read": (_i32, [_ptr, _u64, _ptr]),
-    "rthip_probe_empty_launch": (_i32, [_ptr]),
     "rthip_nf4_linear_forward_with": (
         _i32,
         [_i32, _ptr] + _WEIGHT + [_ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
@@ -426,14 +424,6 @@ class Library:
             dy_ptr, *weight.abi_arguments(), dx_ptr, rows,
             weight.input_width, weight.output_width, weight.block_size,
             stream))
-
-    def probe_streaming_read(self, data_ptr: int, size: int,
-                             stream: int = 0) -> None:
-        self._check(self._lib.rthip_probe_streaming_read(data_ptr, size,
-                                                         stream))
-
-    def probe_empty_launch(self, stream: int = 0) -> None:
-        self._check(self._lib.rthip_probe_empty_launch(stream))
 
     def release_workspaces(self, stream: int = 0,
                            every_stream: bool = True) -> None:

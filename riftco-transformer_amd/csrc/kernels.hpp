@@ -205,12 +205,6 @@ void launch_check_payload(const Nf4WeightView& weight,
                           unsigned long long* words, hipStream_t stream);
 PayloadViolation classify_payload(const unsigned long long words[3]);
 
-// probe.hip -- measurement aids: a plain streaming read of `bytes` (a multiple
-// of 16, 16-byte aligned) and an empty launch.
-void launch_streaming_read(const void* data, std::size_t bytes,
-                           hipStream_t stream);
-void launch_empty(hipStream_t stream);
-
 // nf4_mfma.hip
 bool mfma_forward_supports(const LinearProblem& problem);
 hipError_t launch_mfma_forward(const LinearProblem& problem,

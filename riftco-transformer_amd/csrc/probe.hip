@@ -1,12 +1,25 @@
-// Measurement aids: the two launches a roofline argument needs beside the
-// kernels themselves -- a plain streaming read of a buffer (what the memory
-// system delivers to a kernel that does nothing else, per launch size) and an
-// empty launch (what a launch costs before it reads anything).  Neither is
-// part of the packed linear path.
+// Measurement aids, built into a library of their own (librthip_probe.so) that
+// only the benchmark loads: the two launches a roofline argument needs beside
+// the kernels themselves -- a plain streaming read of a buffer (what the
+// memory system delivers to a kernel that does nothing else, per launch size)
+// and an empty launch (what a launch costs before it reads anything).  Neither
+// is part of the packed linear path or of its C ABI.
+//
+//   int rthip_probe_streaming_read(const void* data, uint64_t bytes,
+//                                  void* stream);
+//       reads `bytes` (a positive multiple of 16, 16-byte aligned) of device
+//       memory once and does nothing with them
+//   int rthip_probe_empty_launch(void* stream);
+//       a launch of the same grid that does nothing
+//
+// Both only enqueue and return the hipError_t of the launch (0: enqueued; -1:
+// bad argument).
 
-#include "kernels.hpp"
+#include <hip/hip_runtime.h>
 
-namespace rthip {
+#include <cstddef>
+#include <cstdint>
+
 namespace {
 
 constexpr int kThreads = 512;
@@ -49,14 +62,20 @@ __global__ void empty_kernel(unsigned* sink) {
 
 }  // namespace
 
-void launch_streaming_read(const void* data, std::size_t bytes,
-                           hipStream_t stream) {
-    streaming_read_kernel<<<256, kThreads, 0, stream>>>(
+extern "C" int rthip_probe_streaming_read(const void* data,
+                                          std::uint64_t bytes, void* stream) {
+    if (data == nullptr || bytes == 0 || bytes % 16 != 0 ||
+        reinterpret_cast<std::uintptr_t>(data) % 16 != 0) {
+        return -1;
+    }
+    streaming_read_kernel<<<256, kThreads, 0,
+                            static_cast<hipStream_t>(stream)>>>(
         static_cast<const uint4*>(data), bytes / sizeof(uint4), nullptr);
+    return static_cast<int>(hipGetLastError());
 }
 
-void launch_empty(hipStream_t stream) {
-    empty_kernel<<<256, kThreads, 0, stream>>>(nullptr);
+extern "C" int rthip_probe_empty_launch(void* stream) {
+    empty_kernel<<<256, kThreads, 0, static_cast<hipStream_t>(stream)>>>(
+        nullptr);
+    return static_cast<int>(hipGetLastError());
 }
-
-}  // namespace rthip

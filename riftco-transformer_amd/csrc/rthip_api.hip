@@ -1509,30 +1509,6 @@ rthip_status rthip_nf4_forward_kernel_name(
     return RTHIP_OK;
 }
 
-rthip_status rthip_probe_streaming_read(const void* data, uint64_t bytes,
-                                        void* stream) {
-    if (data == nullptr || bytes == 0 || bytes % 16 != 0 ||
-        reinterpret_cast<std::uintptr_t>(data) % 16 != 0) {
-        return fail(RTHIP_INVALID_ARGUMENT,
-                    "the streaming-read probe needs a 16-byte aligned "
-                    "buffer whose size is a positive multiple of 16");
-    }
-    if (const rthip_status status = require_device(); status != RTHIP_OK) {
-        return status;
-    }
-    rthip::launch_streaming_read(data, bytes,
-                                 static_cast<hipStream_t>(stream));
-    return finish_launch("streaming-read probe launch");
-}
-
-rthip_status rthip_probe_empty_launch(void* stream) {
-    if (const rthip_status status = require_device(); status != RTHIP_OK) {
-        return status;
-    }
-    rthip::launch_empty(static_cast<hipStream_t>(stream));
-    return finish_launch("empty probe launch");
-}
-
 rthip_status rthip_release_workspaces(void* stream, int32_t every_stream) {
     if (const rthip_status status = require_device(); status != RTHIP_OK) {
         return status;

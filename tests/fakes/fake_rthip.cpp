@@ -259,16 +259,6 @@ rthip_status rthip_nf4_linear_input_backward_no_alloc(
 
 rthip_status rthip_release_workspaces(void*, int32_t) { return RTHIP_OK; }
 
-rthip_status rthip_probe_streaming_read(const void* data, uint64_t bytes,
-                                        void*) {
-    if (data == nullptr || bytes == 0 || bytes % 16 != 0) {
-        return fail(RTHIP_INVALID_ARGUMENT, "bad probe buffer");
-    }
-    return RTHIP_OK;
-}
-
-rthip_status rthip_probe_empty_launch(void*) { return RTHIP_OK; }
-
 rthip_status rthip_nf4_linear_forward_with(
     int32_t, const float* x, const uint8_t* codes, const void* primary_scales,
     const float* secondary_scales, int32_t encoding,
