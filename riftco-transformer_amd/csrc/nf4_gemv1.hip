@@ -1,8 +1,9 @@
-// Decode GEMV for ONE row of x:
-//     y[o] = sum_i x[i] * codebook[code(o, i)] * scale(o, i / B)
+// Decode GEMV for one to four rows of x:
+//     y[m][o] = sum_i x[m][i] * codebook[code(o, i)] * scale(o, i / B)
 // restating reference_quantized_linear_forward
 // (src/core/backend/nn/quantized_linear/reference/operations.cpp:49-81) for
-// the case the decode step of a model is made of.  A launch of 9 to 50 MB
+// the case the decode step of a model is made of (one row; two to four rows
+// reuse every load and lookup and add multiply-adds).  A launch of 9 to 50 MB
 // lasts three to ten microseconds, and what bounds it besides the bytes is
 // the compute unit's vector-memory pipeline: it takes one load instruction of
 // a wavefront every ~6 clocks when a lane loads 4 bytes, but only every ~28
@@ -45,7 +46,8 @@
 // exact only along straight-line code.
 //
 // Decode is the (low nibble, high nibble) pair table in LDS of nf4_gemv.hip
-// (which serves two to four rows of x and block sizes other than 64).  Row
+// (which serves block sizes other than 64, output widths that are no multiple
+// of eight and rows wider than 12288 weights).  Row
 // sums: transposed butterfly inside each 16-lane DPP row, across the
 // wavefront's four rows with v_permlane swaps, the eight wavefront partials
 // parked in LDS and added in wavefront order after ONE barrier at the end.  A
