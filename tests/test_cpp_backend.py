@@ -185,6 +185,20 @@ def test_work_split_of_the_small_batch_input_backward():
     assert "backward split tests passed" in result.stdout
 
 
+def test_shape_predicates_of_the_kernels():
+    """What a launch may assume is decided on the host: the decode kernel's
+    shapes, the tiled kernel's, and the bound that keeps the adapter term's
+    partial sums inside the workspace (tests/cpp/test_kernel_predicates.hip,
+    linked against librthip.so; nothing is launched)."""
+    binary = os.path.join(BUILD, "test_kernel_predicates")
+    assert os.path.exists(binary), \
+        "tests/cpp/build/test_kernel_predicates is not built (make -C tests/cpp)"
+    result = subprocess.run([binary], capture_output=True, text=True,
+                            timeout=120)
+    assert result.returncode == 0, result.stdout + result.stderr
+    assert "kernel predicate tests passed" in result.stdout
+
+
 def test_unavailable_when_the_runtime_sees_no_device():
     result = run(["--expect-unavailable"],
                  RIFTCO_TRANSFORMER_HIP_LIBRARY=FAKE, FAKE_RTHIP_NO_DEVICE="1")
