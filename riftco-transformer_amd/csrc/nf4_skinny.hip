@@ -86,8 +86,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_buffer(const void* base,
 }
 
 // kBlocks: 16-row blocks of x (rows <= 16 * kBlocks).  kScales: block scales
-// per 64-weight lane chunk (2 for block size 32, else 1).
-template <int kBlocks, int kScales, bool kDoubleQuantized>
+// per 64-weight lane chunk (2 for block size 32, else 1).  kTwoLevel: the
+// matrix instructions' sums are folded into a second accumulator after every
+// slab (see `total` below).
+template <int kBlocks, int kScales, bool kDoubleQuantized, bool kTwoLevel>
 __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
     const float* __restrict__ x, Nf4WeightView weight,
     const float* __restrict__ bias, float* __restrict__ y,
@@ -239,11 +241,41 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
         }
     };
 
+    // Two-level accumulation: the matrix instructions add into `acc` for one
+    // slab (64 instructions, 256 contraction values), then `acc` is folded
+    // into `total`.  One fp32 chain over 7000 and more contraction values
+    // drifts as far as the CPU's sequential sum (1.0-1.7e-5 of an output's
+    // K-normalised scale measured on 28672 x 8192 and 16384 x 20480); chains
+    // of a slab stay an order of magnitude below that (1.5-1.8e-6).  Without
+    // kTwoLevel `total` is not kept (with four blocks of x its registers do
+    // not fit beside the rest); the launcher asks for that only where a
+    // workgroup's run of slabs is short.
     floatx4 acc[kBlocks];
+    floatx4 total[kTwoLevel ? kBlocks : 1];
     const auto clear_accumulators = [&]() {
 #pragma unroll
         for (int b = 0; b < kBlocks; ++b) {
             acc[b] = floatx4{0.0F, 0.0F, 0.0F, 0.0F};
+            if constexpr (kTwoLevel) {
+                total[b] = floatx4{0.0F, 0.0F, 0.0F, 0.0F};
+            }
+        }
+    };
+    const auto fold_accumulators = [&]() {
+        if constexpr (kTwoLevel) {
+#pragma unroll
+            for (int b = 0; b < kBlocks; ++b) {
+                total[b] += acc[b];
+                acc[b] = floatx4{0.0F, 0.0F, 0.0F, 0.0F};
+            }
+        }
+    };
+    // a run's sums, once its last slab has been folded
+    const auto sums = [&](int b) -> const floatx4& {
+        if constexpr (kTwoLevel) {
+            return total[b];
+        } else {
+            return acc[b];
         }
     };
     clear_accumulators();
@@ -281,7 +313,7 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
                         const unsigned m = 16 * b + 4 * quarter + r;
                         if (m < rows) {
                             y[static_cast<std::size_t>(m) * output_width + n] =
-                                (acc[b][r] + addend) + term[r];
+                                (sums(b)[r] + addend) + term[r];
                         }
                     }
                 }
@@ -295,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const unsigned m = 16 * b + 4 * quarter + r;
-                    target[m * kTileN + lane_row] = acc[b][r];
+                    target[m * kTileN + lane_row] = sums(b)[r];
                 }
             }
         }
@@ -354,6 +386,9 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
         __syncthreads();  // the previous slab's fragment reads are done
         store_x(x_staged);
         __syncthreads();
+        // (the previous slab's matrix instructions finished long ago: the
+        // fold waits for nothing)
+        fold_accumulators();
         load_x(x_staged, x_cursor);
         advance(x_cursor);
 
@@ -415,6 +450,7 @@ __global__ __launch_bounds__(kThreads) void skinny_forward_kernel(
             const unsigned slot =
                 group * kSlotsPerGroup +
                 (compute_cursor.tile == first_tile ? 0U : 1U);
+            fold_accumulators();
             flush(compute_cursor.tile, whole_tile, slot);
             clear_accumulators();
             segment_first_slab = 0;
@@ -485,12 +521,40 @@ constexpr std::size_t kWorkspaceBytes =
     sizeof(float);
 static_assert(kWorkspaceBytes <= kStreamWorkspaceBytes);
 
-template <int kBlocks, int kScales, bool kDoubleQuantized>
+// Slabs a workgroup may chain in ONE accumulator (4096 contraction values:
+// rounding stays near 5e-6 of an output's scale).
+constexpr unsigned kSingleChainSlabs = 16;
+
+// The split of (tile, slab) units over the workgroups.
+struct LaunchSplit {
+    UnitSplit split;
+    unsigned tiles;
+    unsigned groups;
+};
+LaunchSplit split_units(const LinearProblem& p) {
+    LaunchSplit launch;
+    launch.tiles =
+        static_cast<unsigned>((p.output_width + kTileN - 1) / kTileN);
+    launch.split.slabs =
+        static_cast<unsigned>((p.input_width + kSlab - 1) / kSlab);
+    const unsigned units = launch.tiles * launch.split.slabs;
+    // One workgroup per compute unit; with at least that many tiles, one
+    // workgroup per tile (no partial tiles at all).
+    launch.groups =
+        launch.tiles >= kComputeUnits
+            ? launch.tiles
+            : (units < kComputeUnits ? units : kComputeUnits);
+    launch.split.quotient = units / launch.groups;
+    launch.split.remainder = units % launch.groups;
+    return launch;
+}
+
+template <int kBlocks, int kScales, bool kDoubleQuantized, bool kTwoLevel>
 hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     constexpr std::size_t kSharedBytes =
         static_cast<std::size_t>(16 * kBlocks) * kStride * sizeof(float);
     const auto kernel =
-        skinny_forward_kernel<kBlocks, kScales, kDoubleQuantized>;
+        skinny_forward_kernel<kBlocks, kScales, kDoubleQuantized, kTwoLevel>;
     // More than the default 64 KB of LDS.
     static std::atomic<std::uint64_t> served{0};
     if (const hipError_t error = allow_dynamic_lds(
@@ -498,20 +562,10 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
         error != hipSuccess) {
         return error;
     }
-    const unsigned tiles =
-        static_cast<unsigned>((p.output_width + kTileN - 1) / kTileN);
-    UnitSplit split;
-    split.slabs =
-        static_cast<unsigned>((p.input_width + kSlab - 1) / kSlab);
-    const unsigned units = tiles * split.slabs;
-    // One workgroup per compute unit; with at least that many tiles, one
-    // workgroup per tile (no partial tiles at all).
-    const unsigned groups =
-        tiles >= kComputeUnits
-            ? tiles
-            : (units < kComputeUnits ? units : kComputeUnits);
-    split.quotient = units / groups;
-    split.remainder = units % groups;
+    const LaunchSplit launch = split_units(p);
+    const UnitSplit& split = launch.split;
+    const unsigned tiles = launch.tiles;
+    const unsigned groups = launch.groups;
     const bool partial_tiles = groups != tiles;
     WorkspaceLease lease;  // held until both launches are enqueued
     if (partial_tiles) {
@@ -535,15 +589,32 @@ hipError_t launch_instance(const LinearProblem& p, hipStream_t stream) {
     return hipSuccess;
 }
 
-template <int kBlocks>
-hipError_t launch_blocks(const LinearProblem& p, hipStream_t stream) {
+template <int kBlocks, bool kTwoLevel>
+hipError_t launch_encoding(const LinearProblem& p, hipStream_t stream) {
     const bool two_scales = p.block_shift == 5;  // block size 32
     if (p.weight.encoding == 0) {
-        return two_scales ? launch_instance<kBlocks, 2, false>(p, stream)
-                          : launch_instance<kBlocks, 1, false>(p, stream);
+        return two_scales
+                   ? launch_instance<kBlocks, 2, false, kTwoLevel>(p, stream)
+                   : launch_instance<kBlocks, 1, false, kTwoLevel>(p, stream);
     }
-    return two_scales ? launch_instance<kBlocks, 2, true>(p, stream)
-                      : launch_instance<kBlocks, 1, true>(p, stream);
+    return two_scales
+               ? launch_instance<kBlocks, 2, true, kTwoLevel>(p, stream)
+               : launch_instance<kBlocks, 1, true, kTwoLevel>(p, stream);
+}
+
+template <int kBlocks>
+hipError_t launch_blocks(const LinearProblem& p, hipStream_t stream) {
+    if constexpr (kBlocks == 4) {
+        // the second accumulator costs four blocks of x spilled registers
+        // (4096 x 11008 at 64 rows: 64.5 -> 69.4 us): kept for long runs only
+        const LaunchSplit launch = split_units(p);
+        const unsigned longest_run =
+            std::min(launch.split.quotient + 1, launch.split.slabs);
+        if (longest_run <= kSingleChainSlabs) {
+            return launch_encoding<4, false>(p, stream);
+        }
+    }
+    return launch_encoding<kBlocks, true>(p, stream);
 }
 
 }  // namespace

@@ -724,6 +724,40 @@ def test_small_batches_at_the_llama_shapes(gpu, package, library, oracle,
                     oracle_rows=2)
 
 
+def test_long_runs_of_the_small_batch_forward_are_summed_in_two_levels(
+        gpu, package, library, oracle):
+    """A 70B feed-forward weight (8192 x 28672) at 33 and 64 rows: 64 output
+    tiles x 112 slabs over 256 workgroups are runs of 28 slabs, 7168
+    contraction values per accumulator.  One fp32 chain of that length drifts
+    1.0-1.6e-5 of an output's K-normalised scale, beyond the bar; the kernel
+    folds its matrix sums into a second accumulator after every slab."""
+    import torch
+    out_w, in_w = 8192, 28672
+    weight = oracle.quantize(helpers.normal(120, (out_w, in_w), 0.02), 64,
+                             True, 256)
+    device_weight = upload(gpu, weight)
+    deq = gpu.dequantize(device_weight)
+    weight_rms = float(deq.double().pow(2).mean().sqrt())
+    for rows in (33, 64):
+        assert library.select_algorithm(package.FORWARD, rows, in_w, out_w,
+                                        64) == package.ALGORITHM_SKINNY
+        x = helpers.normal(121 + rows, (rows, in_w), 1.0)
+        x_device = to_device(x)
+        y = gpu.linear_forward(x_device, device_weight)
+        exact = x_device.double() @ deq.double().T
+        scale = np.sqrt(in_w) * helpers.rms(x) * weight_rms
+        error = float((y.double() - exact).abs().max()) / scale
+        assert error <= TOLERANCE, f"{rows} rows vs fp64: {error:.3g}"
+        cpu = oracle.forward(x[:2], weight)
+        cpu_error = helpers.normalized_error(
+            cpu, host(exact)[:2], in_w, helpers.rms(x), weight_rms)
+        drift = helpers.normalized_error(host(y)[:2], cpu, in_w,
+                                         helpers.rms(x), weight_rms)
+        assert drift <= TOLERANCE + cpu_error
+        del exact, y
+    torch.cuda.empty_cache()
+
+
 def test_zero_scale_blocks_and_saturated_scales(gpu, package, library,
                                                 oracle):
     dense = helpers.normal(70, (64, 128), 0.02)
