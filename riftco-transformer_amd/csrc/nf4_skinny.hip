@@ -521,9 +521,10 @@ constexpr std::size_t kWorkspaceBytes =
     sizeof(float);
 static_assert(kWorkspaceBytes <= kStreamWorkspaceBytes);
 
-// Slabs a workgroup may chain in ONE accumulator (4096 contraction values:
-// rounding stays near 5e-6 of an output's scale).
-constexpr unsigned kSingleChainSlabs = 16;
+// Slabs a workgroup may chain in ONE accumulator (2048 contraction values:
+// rounding stays near 4e-6 of an output's scale; runs of 13.5 slabs measured
+// 7.6e-6).
+constexpr unsigned kSingleChainSlabs = 8;
 
 // The split of (tile, slab) units over the workgroups.
 struct LaunchSplit {
