@@ -22,16 +22,18 @@ TOLERANCE = 1.0e-5
 
 
 def synthetic_weight(package, torch, out_w, in_w, block, double_quantized,
-                     second_level_block, seed):
+                     second_level_block, seed, code_offset=0):
     """A packed weight made on the device: random codes, block scales in
     [0.035, 0.065] (fp32) or random scale codes over second-level scales in
-    [0.02, 0.03] with offset 0.05 (nested)."""
+    [0.02, 0.03] with offset 0.05 (nested).  code_offset: bytes by which the
+    code array is moved off its 256-byte aligned allocation."""
     generator = torch.Generator(device="cuda")
     generator.manual_seed(seed)
     count = out_w * in_w
     blocks = count // block
-    codes = torch.randint(0, 256, (count // 2,), dtype=torch.uint8,
-                          device="cuda", generator=generator)
+    codes = torch.randint(0, 256, (count // 2 + code_offset,),
+                          dtype=torch.uint8, device="cuda",
+                          generator=generator)[code_offset:]
     if not double_quantized:
         scales = torch.rand(blocks, device="cuda",
                             generator=generator) * 0.03 + 0.035
@@ -85,16 +87,25 @@ def test_random_shapes_through_the_automatic_selection(gpu, package, library,
         second_level_block = rng.choice([32, 256])
         with_bias = rng.random() < 0.5
         rank = rng.choice([1, 4, 16, 33])
+        # one case in six hands over arrays that are off the alignment the
+        # fast kernels need (codes by 1-7 bytes, activations by 4-12): the
+        # selection has to notice and fall back
+        code_offset = rng.choice([1, 2, 4, 7]) if rng.random() < 0.17 else 0
+        shift = rng.choice([1, 2, 3]) if rng.random() < 0.17 else 0
         label = (f"seed {seed} case {done}: block {block}, W {out_w}x{in_w}, "
                  f"{rows} rows, nested {double_quantized}/"
-                 f"{second_level_block}, bias {with_bias}, rank {rank}")
+                 f"{second_level_block}, bias {with_bias}, rank {rank}, "
+                 f"codes +{code_offset} B, activations +{4 * shift} B")
         weight = synthetic_weight(package, torch, out_w, in_w, block,
                                   double_quantized, second_level_block,
-                                  1000 * seed + done)
+                                  1000 * seed + done, code_offset)
         deq = gpu.dequantize(weight).double()
         weight_rms = float(deq.pow(2).mean().sqrt())
-        x = torch.randn(rows, in_w, device="cuda")
-        dy = torch.randn(rows, out_w, device="cuda") * 0.01
+        x = torch.randn(rows * in_w + shift,
+                        device="cuda")[shift:].view(rows, in_w)
+        dy = (torch.randn(rows * out_w + shift, device="cuda") *
+              0.01)[shift:].view(rows, out_w)
+        assert x.data_ptr() % 16 == 4 * shift
         bias = torch.randn(out_w, device="cuda") * 0.01 if with_bias else None
         forward_scale = (np.sqrt(max(in_w, 64)) *
                          float(x.pow(2).mean().sqrt()) * weight_rms)
