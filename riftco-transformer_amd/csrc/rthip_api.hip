@@ -1076,8 +1076,15 @@ rthip_status rthip_nf4_linear_forward_group(
                   : rthip::kResidentGroupMax;
         const auto resident_run = [&](uint64_t length) {
             for (uint64_t m = 0; m < length; ++m) {
-                if (select_forward(problems[next + m]) !=
-                    RTHIP_NF4_ALGORITHM_RESIDENT) {
+                // ... as ONE launch: a row count that a call of its own
+                // serves in two parts (65...80 rows: 64 and the rest) is
+                // launched member by member, or a member's rows past the
+                // first part would come from another kernel than in a call
+                // of its own
+                RowSplit split;
+                if (forward_row_split(problems[next + m], &split) ||
+                    select_forward(problems[next + m]) !=
+                        RTHIP_NF4_ALGORITHM_RESIDENT) {
                     return false;
                 }
             }
