@@ -182,6 +182,14 @@ class Oracle:
         values = _f32(values)
         if values.ndim == 1:
             values = values.reshape(1, -1)
+        # QuantizedWeight::quantize_nf4[_double_quantized] check both block
+        # sizes before anything is packed
+        # (src/core/quantization/quantized_weight.cpp:48-53,308,320-321)
+        for size in ((block_size, second_level_block) if double_quantized
+                     else (block_size,)):
+            if not self.block_size_supported(size):
+                raise ValueError("NF4 block size must be one of "
+                                 "32, 64, 128, 256, 512, 1024, 2048, or 4096")
         out_w, in_w = values.shape
         count = values.size
         blocks = -(-count // block_size)

@@ -157,6 +157,15 @@ def test_block_sizes_and_nonfinite_sources(oracle):
     values[0] = np.nan
     with pytest.raises(ValueError):
         oracle.quantize(values, 32)
+    # "double quantization should reject an unsupported scale block size"
+    # (test_quantization.cpp:349-355) and an unsupported first-level one
+    zeros = np.zeros(32, dtype=np.float32)
+    for block, second in ((32, 16), (48, 256), (32, 8192)):
+        with pytest.raises(ValueError, match="NF4 block size must be one of"):
+            oracle.quantize(zeros, block, True, second)
+    with pytest.raises(ValueError, match="NF4 block size must be one of"):
+        oracle.quantize(zeros, 16)
+    oracle.quantize(zeros, 32, True, 32)
 
 
 def test_lora_composes_its_scaled_low_rank_delta(oracle):
