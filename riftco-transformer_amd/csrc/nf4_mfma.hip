@@ -93,7 +93,10 @@ template <bool kTall>
 struct Staged {
     float4 a[4];
     unsigned codes[Tile<kTall>::kWords];
+    // fp32 scales: the block scale; nested: the second-level scale, with the
+    // block's scale code beside it (decoded when the tile is written)
     float scale;
+    unsigned scale_code;
 };
 
 template <bool kTall>
@@ -147,14 +150,25 @@ __device__ __forceinline__ void load_chunk(
         } else {
             staged.codes[0] = *source;
         }
-        staged.scale =
-            load_block_scale<kDoubleQuantized>(weight, flat >> block_shift);
+        const std::size_t block = flat >> block_shift;
+        if constexpr (kDoubleQuantized) {
+            staged.scale_code =
+                static_cast<const std::uint8_t*>(weight.primary_scales)[block];
+            staged.scale =
+                weight.secondary_scales[block >> weight.second_level_shift];
+        } else {
+            staged.scale = static_cast<const float*>(
+                weight.primary_scales)[block];
+        }
     } else {
 #pragma unroll
         for (int w = 0; w < Tile<kTall>::kWords; ++w) {
             staged.codes[w] = 0x77777777U;
         }
         staged.scale = 0.0F;
+        // (nested: factor 0 and second level 0 decode to the offset, which
+        // multiplies level 0)
+        staged.scale_code = 128;
     }
 }
 
@@ -196,7 +210,7 @@ __device__ __forceinline__ void load_weight_tile_backward(
 
 template <bool kTall>
 __device__ __forceinline__ void decode_chunk(
-    const Staged<kTall>& staged, const float* __restrict__ table,
+    const Staged<kTall>& staged, const float* __restrict__ table, float scale,
     float (&out)[Tile<kTall>::kChunk]
 ) {
 #pragma clang fp contract(off)
@@ -205,21 +219,28 @@ __device__ __forceinline__ void decode_chunk(
 #pragma unroll
         for (int n = 0; n < 8; ++n) {
             out[8 * w + n] =
-                table[(staged.codes[w] >> (4 * n)) & 0xFU] * staged.scale;
+                table[(staged.codes[w] >> (4 * n)) & 0xFU] * scale;
         }
     }
 }
 
-template <bool kTall, bool kBackward>
+// table: the sixteen levels, followed for nested scales by the 256 factors
+// (code - 128) / 127.
+template <bool kTall, bool kDoubleQuantized, bool kBackward>
 __device__ __forceinline__ void store_weight_tile(
-    const Staged<kTall>& staged, const float* __restrict__ table,
+    const Staged<kTall>& staged, const float* __restrict__ table, float offset,
     float* __restrict__ tile
 ) {
     constexpr unsigned kChunk = Tile<kTall>::kChunk;
     constexpr unsigned kPerRow = kTileK / kChunk;
     const unsigned thread = threadIdx.x;
     float decoded[kChunk];
-    decode_chunk<kTall>(staged, table, decoded);
+    float scale = staged.scale;
+    if constexpr (kDoubleQuantized) {
+        scale = double_quantized_scale_from_factor(
+            table[16 + staged.scale_code], staged.scale, offset);
+    }
+    decode_chunk<kTall>(staged, table, scale, decoded);
     if constexpr (!kBackward) {
         float* destination =
             tile + (thread / kPerRow) * kStride + (thread % kPerRow) * kChunk;
@@ -302,8 +323,8 @@ __device__ __forceinline__ void gemm_segment(
     const auto store_step = [&](unsigned buffer) {
         float* const target = tiles + buffer * kBufferFloats;
         store_activation_tile<kTall>(staged, target);
-        store_weight_tile<kTall, kBackward>(staged, table,
-                                            target + kTileFloats);
+        store_weight_tile<kTall, kDoubleQuantized, kBackward>(
+            staged, table, weight.offset, target + kTileFloats);
     };
     // Matrix instructions of contraction values [kk, kk + 8) of the step.
     const auto multiply = [&](const float* a_fragment,
@@ -487,8 +508,16 @@ void mfma_gemm_kernel(
     // two buffers of an activation and a weight tile each: more than the 64
     // KB a static array may have, so sized at launch
     extern __shared__ __attribute__((aligned(16))) float tiles[];
-    __shared__ float table[16];
+    __shared__ float table[kDoubleQuantized ? 16 + 256 : 16];
     load_codebook_to_lds(table);
+    if constexpr (kDoubleQuantized) {
+        if (threadIdx.x < 256) {
+            // the division of decode_double_quantized_scale, once per code
+            table[16 + threadIdx.x] =
+                static_cast<float>(static_cast<int>(threadIdx.x) - 128) /
+                127.0F;
+        }
+    }
 
     // A whole tile, or a run of (tile, step) units: one or two segments,
     // each inside one tile.
