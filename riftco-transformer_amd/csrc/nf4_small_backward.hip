@@ -202,6 +202,16 @@ __global__ __launch_bounds__(kThreads) void small_backward_kernel(
     }
 
     build_pair_table<kThreads>(table);
+    // (code - 128) / 127 of a nested scale, once per code: the division of
+    // decode_double_quantized_scale leaves the loop
+    __shared__ float factor[kDoubleQuantized ? 256 : 1];
+    if constexpr (kDoubleQuantized) {
+        if (threadIdx.x < 256) {
+            factor[threadIdx.x] =
+                static_cast<float>(static_cast<int>(threadIdx.x) - 128) /
+                127.0F;
+        }
+    }
     const unsigned lane_bits = pair_table_lane_bits(lane);
     __syncthreads();
 
@@ -238,8 +248,8 @@ __global__ __launch_bounds__(kThreads) void small_backward_kernel(
 #pragma clang fp contract(off)
                 float scale = staged.scales[j];
                 if constexpr (kDoubleQuantized) {
-                    scale = decode_double_quantized_scale(
-                        static_cast<std::uint8_t>(staged.scale_codes[j]),
+                    scale = double_quantized_scale_from_factor(
+                        factor[staged.scale_codes[j] & 0xFFU],
                         staged.scales[j], weight.offset);
                 }
 #pragma unroll

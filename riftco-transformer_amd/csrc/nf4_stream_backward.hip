@@ -179,6 +179,16 @@ __global__ __launch_bounds__(kThreads) void stream_backward_kernel(
     }
 
     build_pair_table<kThreads>(table);
+    // (code - 128) / 127 of a nested scale, once per code: the division of
+    // decode_double_quantized_scale leaves the loop
+    __shared__ float factor[kDoubleQuantized ? 256 : 1];
+    if constexpr (kDoubleQuantized) {
+        if (threadIdx.x < 256) {
+            factor[threadIdx.x] =
+                static_cast<float>(static_cast<int>(threadIdx.x) - 128) /
+                127.0F;
+        }
+    }
     __syncthreads();
     const unsigned lane_bits = pair_table_lane_bits(lane);
 
@@ -221,8 +231,8 @@ __global__ __launch_bounds__(kThreads) void stream_backward_kernel(
                 __builtin_amdgcn_sched_barrier(0);
                 float scale;
                 if constexpr (kDoubleQuantized) {
-                    scale = decode_double_quantized_scale(
-                        static_cast<std::uint8_t>(current.scale_code[r]),
+                    scale = double_quantized_scale_from_factor(
+                        factor[current.scale_code[r] & 0xFFU],
                         current.scale[r], weight.offset);
                 } else {
                     scale = current.scale[r];
