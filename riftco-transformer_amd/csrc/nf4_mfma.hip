@@ -8,7 +8,8 @@
 // restating reference_quantized_linear_forward / _input_backward
 // (src/core/backend/nn/quantized_linear/reference/operations.cpp:49-115).
 // The fp32 weight never exists in HBM: packed nibbles and block scales are
-// read straight from global memory, decoded in registers
+// read straight from global memory (buffer loads: a lane's offset is fixed for
+// a whole tile, the step is a scalar offset), decoded in registers
 // (codebook[code] * scale, one rounded multiply) and written to the LDS tile
 // the matrix cores read.
 //
@@ -41,6 +42,7 @@
 // reads 128 weight rows x 32 contiguous columns, backward reads 32 weight rows
 // (the contraction) x 128 contiguous columns and transposes while writing LDS.
 
+#include "gemv_shared.hpp"
 #include "kernels.hpp"
 #include "launch_config.hpp"
 #include "nf4_decode.hpp"
@@ -52,6 +54,8 @@ namespace rthip {
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
 
 constexpr int kTileN = 128;       // output columns per workgroup
 constexpr int kTileK = 32;        // contraction per step
@@ -100,26 +104,6 @@ struct Staged {
 };
 
 template <bool kTall>
-__device__ __forceinline__ void load_activation_tile(
-    Staged<kTall>& staged, const float* __restrict__ activations,
-    const GemmShape& shape, unsigned row0, unsigned k0
-) {
-    const unsigned thread = threadIdx.x;
-    const unsigned column = (thread % 8) * 4;
-#pragma unroll
-    for (int pass = 0; pass < 4; ++pass) {
-        const unsigned row =
-            row0 + thread / 8 + (Tile<kTall>::kThreads / 8) * pass;
-        staged.a[pass] = row < shape.rows
-            ? *reinterpret_cast<const float4*>(
-                  activations +
-                  static_cast<std::size_t>(row) * shape.contraction + k0 +
-                  column)
-            : make_float4(0.0F, 0.0F, 0.0F, 0.0F);
-    }
-}
-
-template <bool kTall>
 __device__ __forceinline__ void store_activation_tile(
     const Staged<kTall>& staged, float* __restrict__ tile
 ) {
@@ -131,81 +115,6 @@ __device__ __forceinline__ void store_activation_tile(
         *reinterpret_cast<float4*>(tile + row * kStride + column) =
             staged.a[pass];
     }
-}
-
-// The codes and the block scale of a thread's chunk, which starts at weight
-// `flat` (row-major index); a chunk outside the weight decodes to zeros.
-template <bool kTall, bool kDoubleQuantized>
-__device__ __forceinline__ void load_chunk(
-    Staged<kTall>& staged, const Nf4WeightView& weight, bool inside,
-    std::size_t flat, unsigned block_shift
-) {
-    if (inside) {
-        const unsigned* const source =
-            reinterpret_cast<const unsigned*>(weight.codes + (flat >> 1));
-        if constexpr (Tile<kTall>::kWords == 2) {
-            const uint2 both = *reinterpret_cast<const uint2*>(source);
-            staged.codes[0] = both.x;
-            staged.codes[1] = both.y;
-        } else {
-            staged.codes[0] = *source;
-        }
-        const std::size_t block = flat >> block_shift;
-        if constexpr (kDoubleQuantized) {
-            staged.scale_code =
-                static_cast<const std::uint8_t*>(weight.primary_scales)[block];
-            staged.scale =
-                weight.secondary_scales[block >> weight.second_level_shift];
-        } else {
-            staged.scale = static_cast<const float*>(
-                weight.primary_scales)[block];
-        }
-    } else {
-#pragma unroll
-        for (int w = 0; w < Tile<kTall>::kWords; ++w) {
-            staged.codes[w] = 0x77777777U;
-        }
-        staged.scale = 0.0F;
-        // (nested: factor 0 and second level 0 decode to the offset, which
-        // multiplies level 0)
-        staged.scale_code = 128;
-    }
-}
-
-// Forward weight tile: output columns n0..n0+127 are weight rows; the step's
-// 32 contraction values are 16 contiguous code bytes of each row, which two
-// (four) threads share in chunks of 16 (8) weights.
-template <bool kTall, bool kDoubleQuantized>
-__device__ __forceinline__ void load_weight_tile_forward(
-    Staged<kTall>& staged, const Nf4WeightView& weight, const GemmShape& shape,
-    unsigned n0, unsigned k0, unsigned block_shift
-) {
-    constexpr unsigned kChunk = Tile<kTall>::kChunk;
-    constexpr unsigned kPerRow = kTileK / kChunk;
-    const unsigned thread = threadIdx.x;
-    const unsigned n = n0 + thread / kPerRow;
-    load_chunk<kTall, kDoubleQuantized>(
-        staged, weight, n < shape.columns,
-        static_cast<std::size_t>(n) * shape.input_width + k0 +
-            (thread % kPerRow) * kChunk,
-        block_shift);
-}
-
-// Backward weight tile: the step's 32 contraction values are weight rows
-// c0..c0+31; output columns k0..k0+127 are contiguous within each row.
-// Thread t decodes a chunk of row c0 + t % 32.
-template <bool kTall, bool kDoubleQuantized>
-__device__ __forceinline__ void load_weight_tile_backward(
-    Staged<kTall>& staged, const Nf4WeightView& weight, const GemmShape& shape,
-    unsigned k0, unsigned c0, unsigned block_shift
-) {
-    const unsigned thread = threadIdx.x;
-    const unsigned column = k0 + (thread / 32) * Tile<kTall>::kChunk;
-    load_chunk<kTall, kDoubleQuantized>(
-        staged, weight, column < shape.columns,
-        static_cast<std::size_t>(c0 + thread % 32) * shape.input_width +
-            column,
-        block_shift);
 }
 
 template <bool kTall>
@@ -309,15 +218,94 @@ __device__ __forceinline__ void gemm_segment(
     }
     unsigned steps_since_flush = 0;
 
+    // Every load of a step is a buffer load whose per-lane offset is fixed for
+    // the whole segment and whose scalar offset advances with the step: no
+    // vector address arithmetic in the loop, and what lies outside -- rows of
+    // the activations past the last one, weight rows or columns past the
+    // weight -- is past a descriptor's extent (or carries an offset that is),
+    // where the hardware returns zeros: nothing branches on bounds.  (Garbage
+    // in columns past the output width is never stored.)
+    constexpr unsigned kTileRows = Tile<kTall>::kTileM;
+    constexpr unsigned kChunk = Tile<kTall>::kChunk;
+    constexpr unsigned kOutside = 0xFFFFFFFFU;
+    const unsigned tile_rows = min(shape.rows - row0, kTileRows);
+    const __amdgpu_buffer_rsrc_t a_buffer = make_buffer(
+        activations + static_cast<std::size_t>(row0) * shape.contraction,
+        static_cast<std::size_t>(tile_rows) * shape.contraction *
+            sizeof(float));
+    unsigned a_lane[4];
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const unsigned row = thread / 8 + (Tile<kTall>::kThreads / 8) * pass;
+        a_lane[pass] = static_cast<unsigned>(
+            (row * shape.contraction + (thread % 8) * 4) * sizeof(float));
+    }
+    const unsigned weights = shape.input_width *
+        (kBackward ? shape.contraction : shape.columns);
+    const unsigned block_count = ((weights - 1U) >> block_shift) + 1U;
+    const __amdgpu_buffer_rsrc_t code_buffer =
+        make_buffer(weight.codes, weights / 2);
+    const __amdgpu_buffer_rsrc_t primary_buffer = make_buffer(
+        weight.primary_scales,
+        kDoubleQuantized ? block_count : block_count * sizeof(float));
+    const __amdgpu_buffer_rsrc_t secondary_buffer = make_buffer(
+        weight.secondary_scales,
+        kDoubleQuantized
+            ? (((block_count - 1U) >> weight.second_level_shift) + 1U) *
+                  sizeof(float)
+            : 0);
+    // the thread's chunk at step 0 of the weight: its flat index, or nothing
+    unsigned chunk_flat;
+    bool chunk_inside;
+    if constexpr (!kBackward) {
+        constexpr unsigned kPerRow = kTileK / kChunk;
+        const unsigned n = col0 + thread / kPerRow;
+        chunk_inside = n < shape.columns;
+        chunk_flat = n * shape.input_width + (thread % kPerRow) * kChunk;
+    } else {
+        const unsigned column = col0 + (thread / 32) * kChunk;
+        chunk_inside = column < shape.columns;
+        chunk_flat = (thread % 32) * shape.input_width + column;
+    }
+    const unsigned code_lane = chunk_inside ? chunk_flat / 2 : kOutside;
+
     Staged<kTall> staged;
     const auto load_step = [&](unsigned k) {
-        load_activation_tile<kTall>(staged, activations, shape, row0, k);
-        if constexpr (!kBackward) {
-            load_weight_tile_forward<kTall, kDoubleQuantized>(
-                staged, weight, shape, col0, k, block_shift);
+        // scalar: where the step starts in x (bytes) and in the weight (flat)
+        const unsigned a_step = k * static_cast<unsigned>(sizeof(float));
+        const unsigned weight_step = kBackward ? k * shape.input_width : k;
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            const floatx4 loaded = __builtin_bit_cast(
+                floatx4, __builtin_amdgcn_raw_buffer_load_b128(
+                             a_buffer, a_lane[pass], a_step, 0));
+            staged.a[pass] =
+                make_float4(loaded.x, loaded.y, loaded.z, loaded.w);
+        }
+        if constexpr (Tile<kTall>::kWords == 2) {
+            const uintx2 both = __builtin_bit_cast(
+                uintx2, __builtin_amdgcn_raw_buffer_load_b64(
+                            code_buffer, code_lane, weight_step / 2, 0));
+            staged.codes[0] = both.x;
+            staged.codes[1] = both.y;
         } else {
-            load_weight_tile_backward<kTall, kDoubleQuantized>(
-                staged, weight, shape, col0, k, block_shift);
+            staged.codes[0] = __builtin_amdgcn_raw_buffer_load_b32(
+                code_buffer, code_lane, weight_step / 2, 0);
+        }
+        const unsigned block = chunk_inside
+            ? (chunk_flat + weight_step) >> block_shift
+            : kOutside / 4;
+        if constexpr (kDoubleQuantized) {
+            staged.scale_code = __builtin_amdgcn_raw_buffer_load_b8(
+                primary_buffer, block, 0, 0);
+            staged.scale = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(
+                           secondary_buffer,
+                           (block >> weight.second_level_shift) * 4, 0, 0));
+        } else {
+            staged.scale = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(
+                           primary_buffer, block * 4, 0, 0));
         }
     };
     const auto store_step = [&](unsigned buffer) {
@@ -683,6 +671,10 @@ bool common_supports(const LinearProblem& p) {
                    ((std::max(p.input_width, p.output_width) + kTileN - 1) /
                     kTileN) <
                (1ULL << 24) &&
+           // 32-bit flat weight indices and byte offsets inside a tile's rows
+           // of the activations (buffer loads)
+           p.output_width * p.input_width < (1ULL << 32) &&
+           std::max(p.input_width, p.output_width) < (1ULL << 22) &&
            reinterpret_cast<std::uintptr_t>(p.weight.codes) % 8 == 0 &&
            reinterpret_cast<std::uintptr_t>(p.activations) % 16 == 0;
 }

@@ -123,6 +123,14 @@ void test_tiled_kernel_shapes() {
            "prefill backward");
     expect(!rthip::mfma_input_backward_supports(problem(2048, 4096, 11000)),
            "backward contraction not a multiple of 32");
+    // buffer loads: 32-bit flat weight indices, a tile's rows of the
+    // activations within 32-bit byte offsets
+    expect(rthip::mfma_forward_supports(problem(128, 32768, 65536)),
+           "2^31 weights");
+    expect(!rthip::mfma_forward_supports(problem(128, 65536, 65536)),
+           "2^32 weights");
+    expect(!rthip::mfma_forward_supports(problem(128, 1U << 22, 32)),
+           "a row of 2^22 activations");
 }
 
 }  // namespace
