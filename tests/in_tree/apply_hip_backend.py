@@ -5,8 +5,8 @@ reference's own registry, with the reference's own tests.
 
 What it does, in a scratch directory outside this repository:
 
-1. copies the reference's `include/`, `src/core/` and two of its tests
-   (tests/core/backend/test_quantized_linear_backend.cpp, test_backend.cpp)
+1. copies the reference's `include/`, `src/core/`, `src/nn/`, `src/optim/`,
+   `src/model/`, `src/c_api/` and five of its tests
    from /root/reference -- nothing of the reference enters this repository;
 2. applies the edits a maintainer would make to add the backend, each written
    here as "find this short anchor, put that text beside it":
@@ -44,16 +44,23 @@ What it does, in a scratch directory outside this repository:
        CPU-only tests of the former (autograd graph of 2 nodes / 20 elements
        and VJP, :140-183; packed bytes unchanged across an Adam step and the
        merged export, :185-267) are duplicated with `Cpu` replaced by `Hip`
-       and run when the backend is available;
+       and run when the backend is available,
+     * the same for the model: in the scratch copy of
+       tests/model/test_qlora_model.cpp the polymorphic transfer of the
+       decoder-only model (:276-323) names hip, and the training test
+       (:136-274: quantize, attach adapters, one step of cross entropy,
+       backward and paged Adam, merged export) is duplicated with the
+       quantized model moved to hip before its adapters go to the optimizer;
 3. compiles the edited files and this repository's adapter sources
    (hip_adapter.cpp with -DRIFTCO_TRANSFORMER_IN_TREE, hip_runtime.cpp,
    packed_state.cpp) with g++ and links them with the objects of the
    unedited reference sources that oracle/Makefile already built
    (oracle/_ref/obj: tensor, quantization, backend, autograd and the few
-   nn/ files of a Linear);
+   nn/ files of a Linear) and with the reference's optimizer, remaining nn/
+   files and decoder-only model, compiled here as they are;
 4. leaves the test programs (the accelerator test twice: as it is, and with
-   the RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP gate on; the nn and quantization
-   tests; tests/in_tree/test_c_api_identity.cpp, this repository's own few
+   the RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP gate on; the nn, quantization
+   and model tests; tests/in_tree/test_c_api_identity.cpp, this repository's own few
    lines over the edited bridge) in tests/in_tree/build/ (git-ignored; they
    travel to the GPU box, where tests/test_in_tree.py runs them against the
    real librthip.so).
@@ -84,9 +91,19 @@ EDITED_SOURCES = [
     "src/nn/linear.cpp",
 ]
 # ... reference sources that are compiled as they are, beyond the objects
-# oracle/Makefile built (the nn tests need the optimizer) ...
+# oracle/Makefile built (the nn tests need the optimizer, the model test the
+# decoder-only model and the layers under it) ...
 EXTRA_SOURCES = [
     "src/optim/adam.cpp",
+    "src/nn/activations.cpp",
+    "src/nn/embedding.cpp",
+    "src/nn/layer_norm.cpp",
+    "src/nn/loss.cpp",
+    "src/nn/rms_norm.cpp",
+    "src/model/causal_self_attention.cpp",
+    "src/model/decoder_only_transformer.cpp",
+    "src/model/feed_forward.cpp",
+    "src/model/transformer_block.cpp",
 ]
 # ... and the file the Linear edit adds
 ADDED_SOURCES = {"src/nn/hip_fused_linear.cpp": None}  # text: FUSED_LINEAR
@@ -101,6 +118,7 @@ TESTS = {
     "backend_tests": ("tests/core/backend/test_backend.cpp", []),
     "quantized_linear_tests": ("tests/nn/test_quantized_linear.cpp", []),
     "quantization_tests": ("tests/core/test_quantization.cpp", []),
+    "qlora_model_tests": ("tests/model/test_qlora_model.cpp", []),
 }
 # this repository's own programs over the edited tree: the C ABI bridge, and
 # the fused Linear against the reference's composition on the CPU backend
@@ -359,7 +377,7 @@ EDITS = [
 def copy_reference(tree):
     for part in ("include", os.path.join("src", "core"),
                  os.path.join("src", "nn"), os.path.join("src", "optim"),
-                 os.path.join("src", "c_api")):
+                 os.path.join("src", "model"), os.path.join("src", "c_api")):
         shutil.copytree(os.path.join(REFERENCE, part),
                         os.path.join(tree, part))
     for source, _ in TESTS.values():
@@ -441,6 +459,53 @@ QUANTIZATION_TEST = "tests/core/test_quantization.cpp"
 
 def quantization_test_on_hip(source):
     return accelerator_becomes_hip(source, QUANTIZATION_TEST, 6)
+
+
+MODEL_TEST = "tests/model/test_qlora_model.cpp"
+
+
+# the training test of the reference runs on the CPU backend: repeated with
+# the quantized model moved to hip before its adapters are handed to Adam
+MODEL_TRAINING_TEST = "test_model_qlora_training_and_fp32_export"
+MODEL_TRANSFER_TEST = "test_polymorphic_model_transfer_if_metal_available"
+
+
+def model_test_on_hip(source):
+    source = accelerator_becomes_hip(source, MODEL_TEST, 4)
+    transfer = function_text(source, MODEL_TRANSFER_TEST, MODEL_TEST)
+    source = source.replace(
+        transfer,
+        transfer[:-3] +
+        "\n    std::cout << \"QLoRA model moved to hip and back\\n\";\n}\n")
+    training = function_text(source, MODEL_TRAINING_TEST, MODEL_TEST)
+    attached = "    });\n    ParameterList adapters = model.lora_parameters();\n"
+    if training.count(attached) != 1:
+        raise SystemExit(f"{MODEL_TEST}: {MODEL_TRAINING_TEST} has changed")
+    on_hip = training.replace(
+        f"void {MODEL_TRAINING_TEST}()", f"void {MODEL_TRAINING_TEST}_on_hip()"
+    ).replace(
+        attached,
+        "    });\n"
+        "    static_cast<riftco_transformer::Module&>(model).to(\n"
+        "        riftco_transformer::ExecutionBackend::Hip);\n"
+        "    require(\n"
+        "        model.backend() == riftco_transformer::ExecutionBackend::Hip,\n"
+        "        \"the quantized model trains on hip\"\n"
+        "    );\n"
+        "    ParameterList adapters = model.lora_parameters();\n")
+    close = "}  // namespace\n\nint main() {\n"
+    first_call = f"        {MODEL_TRAINING_TEST}();\n"
+    if source.count(close) != 1 or source.count(first_call) != 1:
+        raise SystemExit(f"{MODEL_TEST}: main() has changed")
+    source = source.replace(close, on_hip + "\n" + close)
+    return source.replace(
+        first_call,
+        first_call +
+        "        if (riftco_transformer::execution_backend_available(\n"
+        "                riftco_transformer::ExecutionBackend::Hip)) {\n"
+        f"            {MODEL_TRAINING_TEST}_on_hip();\n"
+        "            std::cout << \"QLoRA model trained on hip\\n\";\n"
+        "        }\n")
 
 
 def compile_one(job):
@@ -527,6 +592,7 @@ def main():
             edit.apply(tree)
         rewrite(tree, NN_TEST, nn_test_on_hip)
         rewrite(tree, QUANTIZATION_TEST, quantization_test_on_hip)
+        rewrite(tree, MODEL_TEST, model_test_on_hip)
         build(tree)
     finally:
         if arguments.keep:

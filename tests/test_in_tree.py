@@ -9,7 +9,9 @@ sends `Linear::forward` of a packed layer with a low-rank adapter through one
 fused graph node on hip, adds RT_BACKEND_HIP to the C ABI bridge, and builds
 the reference's tests/nn/test_quantized_linear.cpp and
 tests/core/test_quantization.cpp with hip in the place of their optional
-accelerator (and the former's CPU-only tests repeated on hip), plus two
+accelerator (and the former's CPU-only tests repeated on hip), its
+tests/model/test_qlora_model.cpp (the decoder-only model moved to hip and
+back, and one QLoRA training step of the whole model on hip), plus two
 programs of this repository: the fused layer against the reference's
 composition on the CPU backend, and the bridge's identity checks.
 
@@ -105,6 +107,22 @@ def test_quantization_transfer_keeps_bytes_on_hip(programs):
     assert "NF4 quantization tests passed" in done.stdout
 
 
+def test_qlora_model_trains_on_hip(programs):
+    """tests/model/test_qlora_model.cpp: the decoder-only model is quantized,
+    given adapters, and -- in the copy the script adds -- moved to hip before
+    one step of cross entropy, backward and paged Adam (:136-274: packed byte
+    counts unchanged by the step, merged export equal to the adapted output);
+    Module::to to hip and back keeps the packed payload (:276-323)."""
+    done = run("qlora_model_tests", FAKE)
+    assert done.returncode == 0, done.stderr
+    assert "QLoRA model trained on hip" in done.stdout
+    assert "QLoRA model moved to hip and back" in done.stdout
+    assert "QLoRA model tests passed" in done.stdout
+    without = run("qlora_model_tests", "/nonexistent/librthip.so")
+    assert without.returncode == 0, without.stderr
+    assert "on hip" not in without.stdout and "to hip" not in without.stdout
+
+
 def test_fused_linear_equals_the_reference_composition(programs):
     done = run("fused_linear_tests", FAKE,
                RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1")
@@ -143,11 +161,14 @@ def test_reference_tests_on_the_device():
         pytest.skip("tests/in_tree/build was not built (no reference tree)")
     for program in ("quantized_linear_backend_tests_hip_required",
                     "backend_tests", "quantized_linear_tests",
-                    "quantization_tests", "fused_linear_tests",
-                    "c_api_identity_tests"):
+                    "quantization_tests", "qlora_model_tests",
+                    "fused_linear_tests", "c_api_identity_tests"):
         done = run(program, REAL, RIFTCO_TRANSFORMER_HIP_REJECT_TEST_PLUGIN="1",
                    RIFTCO_TRANSFORMER_TEST_REQUIRE_HIP="1")
         assert done.returncode == 0, program + done.stdout + done.stderr
         assert "tests passed" in done.stdout
         if program == "quantized_linear_tests":
             assert "quantized Linear tests ran on hip" in done.stdout
+        if program == "qlora_model_tests":
+            assert "QLoRA model trained on hip" in done.stdout
+            assert "QLoRA model moved to hip and back" in done.stdout
