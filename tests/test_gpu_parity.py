@@ -268,7 +268,7 @@ def test_ragged_shapes_and_block_sizes(gpu, package, library, oracle, out_w,
 @pytest.mark.parametrize("out_w,in_w,block,double_quantized", [
     (33000, 64, 32, False),    # >= 256 output tiles: one workgroup per tile
     (300, 1280, 64, True),     # fewer (tile, slab) units than compute units
-    (2000, 1600, 64, False),   # last round and last tile partly empty
+    (2000, 1600, 64, False),   # last pass over the compute units and last tile partly empty
     (5000, 2048, 64, True),    # runs of one and two units, tiles shared
     (1000, 16384, 128, False),  # many workgroups per output tile
     (30000, 512, 32, True),    # runs that cross from one tile into the next
