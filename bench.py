@@ -312,7 +312,7 @@ def bench_gemm(package, device, torch, steps):
             target = torch.empty(rows, in_w, device="cuda")
             body = lambda: device.linear_input_backward(source, weight,
                                                         out=target)
-        for _ in range(5):   # the first launches after idle run at low clocks
+        for _ in range(20):  # the first launches after idle run at low clocks
             body()
         milliseconds = time_region(torch, body, steps) / steps
         flops = 2.0 * rows * out_w * in_w
