@@ -209,6 +209,10 @@ PayloadViolation classify_payload(const unsigned long long words[3]);
 bool mfma_forward_supports(const LinearProblem& problem);
 hipError_t launch_mfma_forward(const LinearProblem& problem,
                                hipStream_t stream);
+// Leading 128-wide tile columns of a forward's output that go out as 256-row
+// tiles in a launch of their own (0: none; all of them: one launch).
+unsigned mfma_forward_tall_tile_columns(std::size_t rows,
+                                        std::size_t output_width);
 bool mfma_input_backward_supports(const LinearProblem& problem);
 hipError_t launch_mfma_input_backward(const LinearProblem& problem,
                                       hipStream_t stream);

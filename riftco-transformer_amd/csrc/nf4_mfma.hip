@@ -528,8 +528,8 @@ void mfma_gemm_kernel(
                           kTileN;
         gemm_segment<kTall, kDoubleQuantized, kBackward>(
             activations, weight, bias, result, partial, shape, block_shift,
-            lora, tiles, table, (tile / plan.tiles_n) * kTileM,
-            (tile % plan.tiles_n) * kTileN, first_step * kTileK,
+            lora, tiles, table, plan.tile_row(tile) * kTileM,
+            plan.tile_column(tile) * kTileN, first_step * kTileK,
             (first_step + segment_steps) * kTileK);
         unit += segment_steps;
     }
@@ -556,8 +556,8 @@ __global__ __launch_bounds__(256) void gemm_parts_kernel(
     const unsigned index = blockIdx.y * blockDim.x + threadIdx.x;
     const unsigned m = index / kTileN;
     const unsigned c = index % kTileN;
-    const unsigned row = (tile / plan.tiles_n) * kTileM + m;
-    const unsigned column = (tile % plan.tiles_n) * kTileN + c;
+    const unsigned row = plan.tile_row(tile) * kTileM + m;
+    const unsigned column = plan.tile_column(tile) * kTileN + c;
     if (row >= shape.rows || column >= shape.columns) {
         return;
     }
@@ -576,18 +576,20 @@ __global__ __launch_bounds__(256) void gemm_parts_kernel(
     result[static_cast<std::size_t>(row) * shape.columns + column] = sum;
 }
 
+// Tile columns [first_tile_n, first_tile_n + tiles_n) of the output.
 template <bool kTall, bool kDoubleQuantized, bool kBackward>
 hipError_t launch_tiles(const LinearProblem& p, const GemmShape& shape,
+                        unsigned first_tile_n, unsigned tiles_n,
                         hipStream_t stream) {
     constexpr unsigned kTileM = Tile<kTall>::kTileM;
     constexpr unsigned kThreads = Tile<kTall>::kThreads;
     constexpr std::size_t kTileBytes = Tile<kTall>::kTileBytes;
     const auto kernel = mfma_gemm_kernel<kTall, kDoubleQuantized, kBackward>;
     const unsigned tiles_m = (shape.rows + kTileM - 1) / kTileM;
-    const unsigned tiles_n = (shape.columns + kTileN - 1) / kTileN;
     const unsigned tiles = tiles_m * tiles_n;
     TilePlan plan;
     plan.tiles_n = tiles_n;
+    plan.first_tile_n = first_tile_n;
     plan.steps = (shape.contraction + kTileK - 1) / kTileK;
     const unsigned groups =
         plan_tiles(plan, tiles, kTileM * kTileN * sizeof(float),
@@ -621,28 +623,58 @@ hipError_t launch_tiles(const LinearProblem& p, const GemmShape& shape,
 // one workgroup, whose barriers nothing covers.  Measured at 2048 rows: the
 // forward wins where its tiles fill the device in whole rounds (4096 x 4096:
 // 123-124 -> 127-128 TFLOP/s) and is level where leftover tiles are dealt in
-// runs (11008 x 4096); the input backward, whose weight tile is written
-// transposed word by word, loses (W 11008 x 4096: 119 -> 116).  So: forward,
-// whole rounds.
-bool tall_tiles_pay(const GemmShape& shape) {
-    const unsigned tall_rows = Tile<true>::kTileM;
-    const unsigned tiles_m = (shape.rows + tall_rows - 1) / tall_rows;
+// runs (all of 11008 x 4096 in tall tiles); the input backward, whose weight
+// tile is written transposed word by word, loses (W 11008 x 4096: 119 ->
+// 116).  So: forward, whole rounds -- and an output whose tile columns do not
+// come out in whole rounds is cut in two launches: as many tile columns as
+// fill whole rounds in tall tiles, the rest in square ones.
+//
+// Returns the number of leading tile columns that tall tiles take.
+unsigned tall_tile_columns(const GemmShape& shape) {
+    constexpr unsigned kTallRows = Tile<true>::kTileM;
+    constexpr unsigned kPlaces = Tile<true>::kPlaces;
+    if (shape.rows < kTallRows) {
+        return 0;
+    }
+    const unsigned tiles_m = (shape.rows + kTallRows - 1) / kTallRows;
+    const unsigned last_row_fill = shape.rows - (tiles_m - 1) * kTallRows;
+    if (last_row_fill <= kTallRows / 2) {
+        return 0;
+    }
+    // tile columns per whole round: the least n with tiles_m * n a multiple
+    // of the places
+    unsigned common = tiles_m;
+    for (unsigned other = kPlaces; other != 0;) {
+        const unsigned rest = common % other;
+        common = other;
+        other = rest;
+    }
+    const unsigned period = kPlaces / common;
     const unsigned tiles_n = (shape.columns + kTileN - 1) / kTileN;
-    const unsigned last_row_fill = shape.rows - (tiles_m - 1) * tall_rows;
-    return shape.rows >= tall_rows && last_row_fill > tall_rows / 2 &&
-           (tiles_m * tiles_n) % Tile<true>::kPlaces == 0;
+    const unsigned tall = tiles_n / period * period;
+    // a second launch is worth it when tall tiles take at least half
+    return tall * 2 >= tiles_n ? tall : 0;
 }
 
 template <bool kDoubleQuantized, bool kBackward>
 hipError_t launch_encoding(const LinearProblem& p, const GemmShape& shape,
                            hipStream_t stream) {
+    const unsigned tiles_n = (shape.columns + kTileN - 1) / kTileN;
     if constexpr (!kBackward) {
-        if (tall_tiles_pay(shape)) {
-            return launch_tiles<true, kDoubleQuantized, false>(p, shape,
-                                                               stream);
+        const unsigned tall = tall_tile_columns(shape);
+        if (tall != 0) {
+            if (const hipError_t status =
+                    launch_tiles<true, kDoubleQuantized, false>(p, shape, 0,
+                                                                tall, stream);
+                status != hipSuccess || tall == tiles_n) {
+                return status;
+            }
+            return launch_tiles<false, kDoubleQuantized, false>(
+                p, shape, tall, tiles_n - tall, stream);
         }
     }
-    return launch_tiles<false, kDoubleQuantized, kBackward>(p, shape, stream);
+    return launch_tiles<false, kDoubleQuantized, kBackward>(p, shape, 0,
+                                                            tiles_n, stream);
 }
 
 template <bool kBackward>
@@ -680,6 +712,14 @@ bool common_supports(const LinearProblem& p) {
 }
 
 }  // namespace
+
+unsigned mfma_forward_tall_tile_columns(std::size_t rows,
+                                        std::size_t output_width) {
+    GemmShape shape{};
+    shape.rows = static_cast<unsigned>(rows);
+    shape.columns = static_cast<unsigned>(output_width);
+    return tall_tile_columns(shape);
+}
 
 bool mfma_forward_supports(const LinearProblem& p) {
     // Contraction over the row width in steps of 32; a 16-weight chunk must

@@ -22,11 +22,21 @@
 namespace rthip {
 
 struct TilePlan {
-    unsigned tiles_n;      // output tiles per tile row
+    unsigned tiles_n;      // output tiles per tile row (of this launch)
     unsigned whole_tiles;  // tiles computed by one workgroup each
     unsigned steps;        // contraction steps per tile
     unsigned quotient;
     unsigned remainder;
+    // A launch may cover only the tile columns [first_tile_n, first_tile_n +
+    // tiles_n) of the output.
+    unsigned first_tile_n = 0;
+
+    __host__ __device__ unsigned tile_row(unsigned tile) const {
+        return tile / tiles_n;
+    }
+    __host__ __device__ unsigned tile_column(unsigned tile) const {
+        return first_tile_n + tile % tiles_n;
+    }
 
     __host__ __device__ unsigned begin(unsigned group) const {
         return group * quotient + (group < remainder ? group : remainder);

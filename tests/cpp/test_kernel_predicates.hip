@@ -131,6 +131,21 @@ void test_tiled_kernel_shapes() {
            "2^32 weights");
     expect(!rthip::mfma_forward_supports(problem(128, 1U << 22, 32)),
            "a row of 2^22 activations");
+    // 256-row tiles take the tile columns that fill the 256 compute units in
+    // whole rounds (a multiple of 256 / gcd(256, tile rows)), if that is at
+    // least half of them and the last tile row is more than half full
+    const auto tall = rthip::mfma_forward_tall_tile_columns;
+    expect(tall(2048, 4096) == 32, "8 x 32 tall tiles: one launch");
+    expect(tall(2048, 11008) == 64, "8 x 64 of 86 tile columns");
+    expect(tall(4096, 11008) == 80, "16 x 80 of 86");
+    expect(tall(1024, 11008) == 64, "4 x 64 of 86");
+    expect(tall(512, 11008) == 0, "2 tile rows: 128 columns per round");
+    expect(tall(2048, 4224) == 32, "32 of 33");
+    expect(tall(2048, 2048) == 0, "16 tile columns: no whole round");
+    expect(tall(2048, 12288 + 64) == 96, "a ragged last column stays square");
+    expect(tall(255, 4096) == 0, "fewer rows than a tall tile");
+    expect(tall(2048 + 100, 4096) == 0, "last tile row under half full");
+    expect(tall(2048 + 129, 11008 * 4) == 256, "9 tile rows: 256 per round");
 }
 
 }  // namespace
