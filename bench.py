@@ -119,6 +119,16 @@ def time_region(torch, body, repeats):
     return start.elapsed_time(stop)
 
 
+def warm(torch, body, seconds=0.03):
+    """Runs body() for a while: the first milliseconds out of idle run at a
+    lower clock, which a sub-millisecond warm-up does not get past."""
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    while time.perf_counter() - start < seconds:
+        body()
+        torch.cuda.synchronize()
+
+
 # Projections of a layer that read the same activations (one launch each when
 # the step is run through rthip_nf4_linear_forward_group).
 SHARED_INPUT_GROUPS = [("q_proj", "k_proj", "v_proj"), ("o_proj",),
@@ -380,7 +390,7 @@ def bench_mid_batch(package, device, torch, steps):
             body()
             torch.cuda.synchronize()
             body = capture(torch, body)
-            body()
+            warm(torch, body)
             milliseconds = time_region(torch, body, steps) / (
                 steps * len(weights))
             tflops = 2.0 * rows * out_w * in_w / milliseconds / 1e9
@@ -712,7 +722,7 @@ def bench_lora(package, device, torch, steps):
                 body()
                 torch.cuda.synchronize()
                 body = capture(torch, body)
-                body()
+                warm(torch, body)
                 timings[label] = time_region(torch, body, steps) / (
                     steps * len(used)) * 1e3
             results.append({
@@ -735,8 +745,7 @@ def bench_matmul(package, device, torch, steps):
         right = torch.randn(shared, columns, device="cuda") * 0.02
         out = torch.empty(rows, columns, device="cuda")
         body = lambda: device.matmul(left, right, out=out)
-        body()
-        body()
+        warm(torch, body)
         milliseconds = time_region(torch, body, steps) / steps
         tflops = 2.0 * rows * shared * columns / (milliseconds / 1e3) / 1e12
         results.append({
