@@ -412,6 +412,85 @@ __device__ __forceinline__ void gemm_segment(
         }
     }
 
+    // The adapter term is a few more, short, steps on the matrix cores: the
+    // tile's rows of `reduced` take the place of the activation tile, the
+    // tile's columns of the second factor that of the weight tile, 32 of the
+    // rank at a time (contraction values past the rank are zeros); the
+    // products land in `acc`, which the fold above has left free, and are
+    // folded into `total` times the adapter's scale.  The segment that starts
+    // the contraction carries the term, so a tile whose steps are shared
+    // between workgroups gets it exactly once.
+    if (lora.reduced != nullptr && k_begin == 0) {  // uniform
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    acc[i][j][e] = 0.0F;
+                }
+            }
+        }
+        float* const reduced_tile = tiles;
+        float* const factor_tile = tiles + kTileFloats;
+        for (unsigned first = 0; first < lora.rank;
+             first += static_cast<unsigned>(kTileK)) {
+            const unsigned count =
+                min(lora.rank - first, static_cast<unsigned>(kTileK));
+            const unsigned padded = (count + 7U) & ~7U;
+            if (first != 0) {
+                __syncthreads();  // the tiles of the 32 before have been read
+            }
+            // (every wavefront is past the last step's barrier: buffer 0 is
+            // free)
+            for (unsigned index = thread; index < kTileRows * padded;
+                 index += Tile<kTall>::kThreads) {
+                const unsigned r = index / padded;
+                const unsigned j = index % padded;
+                float value = 0.0F;
+                if (row0 + r < shape.rows && j < count) {
+                    value = lora.reduced[static_cast<std::size_t>(row0 + r) *
+                                             lora.rank +
+                                         first + j];
+                }
+                reduced_tile[r * kStride + j] = value;
+            }
+            for (unsigned index = thread; index < kTileN * padded;
+                 index += Tile<kTall>::kThreads) {
+                const unsigned c = index / padded;
+                const unsigned j = index % padded;
+                float value = 0.0F;
+                if (col0 + c < shape.columns && j < count) {
+                    value =
+                        lora.b[static_cast<std::size_t>(col0 + c) *
+                                   lora.row_stride +
+                               static_cast<std::size_t>(first + j) *
+                                   lora.rank_stride];
+                }
+                factor_tile[c * kStride + j] = value;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int kk = 0; kk < static_cast<int>(kTileK); kk += 8) {
+                if (static_cast<unsigned>(kk) < padded) {  // uniform
+                    multiply(tiles + a_offset, tiles + b_offset, kk);
+                }
+            }
+        }
+        // (a following segment of this workgroup meets a barrier before it
+        // writes the tiles)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    total[i][j][e] += lora.scale * acc[i][j][e];
+                }
+            }
+        }
+    }
+
     // Accumulator element e of lane l is output row 8*(e/4) + 4*(l/32) + e%4,
     // column l%32 of its 32 x 32 block.
     if (partial != nullptr) {  // uniform; layout [tile rows][kTileN]
@@ -444,39 +523,13 @@ __device__ __forceinline__ void gemm_segment(
                     addend = bias[column];
                 }
             }
-            float term[16];
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                term[e] = 0.0F;
-            }
-            {
-                if (lora.reduced != nullptr) {  // uniform
-                    const float* reduced_rows[16];
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        const unsigned row =
-                            min(row0 + wave_m * 64 + i * 32 + 8 * (e / 4) +
-                                    4 * (lane / 32) + e % 4,
-                                shape.rows - 1);
-                        reduced_rows[e] =
-                            lora.reduced +
-                            static_cast<std::size_t>(row) * lora.rank;
-                    }
-                    lora_terms<16>(
-                        term,
-                        lora.b + static_cast<std::size_t>(column) *
-                                     lora.row_stride,
-                        reduced_rows, lora.rank, lora.scale,
-                        lora.rank_stride);
-                }
-            }
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const unsigned row = row0 + wave_m * 64 + i * 32 +
                                      8 * (e / 4) + 4 * (lane / 32) + e % 4;
                 if (row < shape.rows) {
                     result[static_cast<std::size_t>(row) * shape.columns +
-                           column] = (total[i][j][e] + addend) + term[e];
+                           column] = total[i][j][e] + addend;
                 }
             }
         }
@@ -536,14 +589,14 @@ void mfma_gemm_kernel(
 }
 
 // Adds the parts of every unit-dealt tile that more than one workgroup worked
-// on, in ascending workgroup order, plus bias and adapter term.  One thread
+// on, in ascending workgroup order, plus bias (the adapter term is in the
+// part that starts the contraction).  One thread
 // per output element: blockIdx.x is the tile among the unit-dealt ones,
 // blockIdx.y a run of 256 elements of it.
 template <unsigned kTileM>
 __global__ __launch_bounds__(256) void gemm_parts_kernel(
     const float* __restrict__ workspace, const float* __restrict__ bias,
-    float* __restrict__ result, GemmShape shape, TilePlan plan,
-    LoraEpilogue lora
+    float* __restrict__ result, GemmShape shape, TilePlan plan
 ) {
     const unsigned dealt_tile = blockIdx.x;
     const unsigned first_unit = dealt_tile * plan.steps;
@@ -569,9 +622,6 @@ __global__ __launch_bounds__(256) void gemm_parts_kernel(
     }
     if (bias != nullptr) {
         sum += bias[column];
-    }
-    if (lora.reduced != nullptr) {
-        sum += lora_term(lora, row, column);
     }
     result[static_cast<std::size_t>(row) * shape.columns + column] = sum;
 }
@@ -614,7 +664,7 @@ hipError_t launch_tiles(const LinearProblem& p, const GemmShape& shape,
     if (groups != 0) {
         const dim3 grid(tiles - plan.whole_tiles, kTileM * kTileN / 256);
         gemm_parts_kernel<kTileM><<<grid, 256, 0, stream>>>(
-            workspace, p.bias, p.result, shape, plan, p.lora);
+            workspace, p.bias, p.result, shape, plan);
     }
     return hipSuccess;
 }
