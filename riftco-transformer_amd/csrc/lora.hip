@@ -38,14 +38,16 @@ template <int kBlocks>
 __global__ __launch_bounds__(kThreads) void lora_reduce_kernel(
     const float* __restrict__ x, const float* __restrict__ a,
     float* __restrict__ reduced, unsigned rows, unsigned input_width,
-    unsigned rank
+    unsigned rank, unsigned rows_per_group
 ) {
     __shared__ float partial[kWaves][kBlocks][4][64];
 
     const unsigned lane = threadIdx.x % 64;
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const unsigned quarter = lane / 16;
-    const unsigned row = blockIdx.x * 16 + lane % 16;         // of x
+    // (a workgroup takes 16 rows of x, or 8 or 4 when that leaves compute
+    // units without one: the other rows of its tile are then zeros)
+    const unsigned row = blockIdx.x * rows_per_group + lane % 16;  // of x
     const unsigned first_adapter_row = blockIdx.y * 16 * kBlocks;
 
     const __amdgpu_buffer_rsrc_t x_buffer = raw_buffer(
@@ -58,7 +60,7 @@ __global__ __launch_bounds__(kThreads) void lora_reduce_kernel(
     const unsigned span_begin = wave * span;
     const unsigned span_end = min(span_begin + span, input_width);
 
-    const bool row_valid = row < rows;
+    const bool row_valid = lane % 16 < rows_per_group && row < rows;
     const unsigned x_row_bytes = row * input_width * 4U;
     bool adapter_valid[kBlocks];
     unsigned a_row_bytes[kBlocks];
@@ -136,9 +138,10 @@ __global__ __launch_bounds__(kThreads) void lora_reduce_kernel(
         for (int w = 0; w < kWaves; ++w) {
             sum += partial[w][b][r][l];
         }
-        const unsigned m = blockIdx.x * 16 + 4 * (l / 16) + r;
+        const unsigned row_in_group = 4 * (l / 16) + r;
+        const unsigned m = blockIdx.x * rows_per_group + row_in_group;
         const unsigned j = first_adapter_row + 16 * b + l % 16;
-        if (m < rows && j < rank) {
+        if (row_in_group < rows_per_group && m < rows && j < rank) {
             reduced[static_cast<std::size_t>(m) * rank + j] = sum;
         }
     }
@@ -237,7 +240,7 @@ void launch_lora_reduce(const float* x, const float* a, float* reduced,
         input_width % 4 == 0 &&
         rows * input_width * sizeof(float) < kRejectedOffset &&
         rank * input_width * sizeof(float) < kRejectedOffset &&
-        (rows + 15) / 16 < (1ULL << 31) && (rank + 63) / 64 <= 65535 &&
+        (rows + 3) / 4 < (1ULL << 31) && (rank + 63) / 64 <= 65535 &&
         reinterpret_cast<std::uintptr_t>(x) % 16 == 0 &&
         reinterpret_cast<std::uintptr_t>(a) % 16 == 0;
     if (!tiled) {
@@ -255,20 +258,29 @@ void launch_lora_reduce(const float* x, const float* a, float* reduced,
             static_cast<unsigned>(rank));
         return;
     }
-    const unsigned row_tiles = static_cast<unsigned>((rows + 15) / 16);
     const auto r = static_cast<unsigned>(rows);
     const auto i = static_cast<unsigned>(input_width);
     const auto k = static_cast<unsigned>(rank);
+    const unsigned chunks =
+        rank <= 32 ? 1U : static_cast<unsigned>((rank + 63) / 64);
+    // x comes in through the compute units that hold a workgroup: fewer rows
+    // per workgroup while the grid is smaller than the device
+    unsigned rows_per_group = 16;
+    while (rows_per_group > 4 &&
+           (rows + rows_per_group - 1) / rows_per_group * chunks < 256) {
+        rows_per_group /= 2;
+    }
+    const unsigned row_tiles = static_cast<unsigned>(
+        (rows + rows_per_group - 1) / rows_per_group);
     if (rank <= 16) {
         lora_reduce_kernel<1><<<dim3(row_tiles, 1), kThreads, 0, stream>>>(
-            x, a, reduced, r, i, k);
+            x, a, reduced, r, i, k, rows_per_group);
     } else if (rank <= 32) {
         lora_reduce_kernel<2><<<dim3(row_tiles, 1), kThreads, 0, stream>>>(
-            x, a, reduced, r, i, k);
+            x, a, reduced, r, i, k, rows_per_group);
     } else {
-        const unsigned chunks = static_cast<unsigned>((rank + 63) / 64);
         lora_reduce_kernel<4><<<dim3(row_tiles, chunks), kThreads, 0, stream>>>(
-            x, a, reduced, r, i, k);
+            x, a, reduced, r, i, k, rows_per_group);
     }
 }
 
