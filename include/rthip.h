@@ -41,7 +41,7 @@ extern "C" {
 #endif
 
 #define RTHIP_ABI_VERSION_MAJOR 1u
-#define RTHIP_ABI_VERSION_MINOR 9u
+#define RTHIP_ABI_VERSION_MINOR 10u
 
 typedef int32_t rthip_status;
 
@@ -203,6 +203,33 @@ rthip_status rthip_nf4_linear_forward_group(
     const float* x, const rthip_nf4_member* members, uint64_t member_count,
     int32_t encoding, uint64_t second_level_block, uint64_t rows,
     uint64_t input_width, uint64_t block_size, void* stream);
+
+/*
+ * The same grouped forward for layers that carry low-rank adapters: member m
+ * gets y_m = x.deq(W_m)^T + bias_m + lora_scale_m * (reduced_m . B_m^T), as
+ * rthip_nf4_lora_linear_forward below computes it when its lora_a is NULL --
+ * `reduced` [rows, lora_rank] already holds x.A_m^T (one rthip_lora_reduce over
+ * the stacked A matrices of the members serves them all).  A member whose
+ * lora_b and reduced are both NULL has no adapter.  The reference reaches this
+ * through Linear::forward (src/nn/linear.cpp:147-172) once per projection;
+ * q, k and v of a layer with adapters on q and v are one launch here.
+ * Every member's output equals its own rthip_nf4_lora_linear_forward (or
+ * rthip_nf4_linear_forward) bit for bit.  One launch for up to four rows of x
+ * (members the decode kernel takes) and for 5...128 rows of a row width of
+ * 1024...4096; other members are launched one by one.
+ */
+typedef struct rthip_nf4_lora_member {
+    rthip_nf4_member base;
+    const float* reduced;  /* [rows, lora_rank], read only; NULL: no adapter */
+    const float* lora_b;   /* [output_width, lora_rank] */
+    uint64_t lora_rank;
+    float lora_scale;
+} rthip_nf4_lora_member;
+
+rthip_status rthip_nf4_lora_linear_forward_group(
+    const float* x, const rthip_nf4_lora_member* members,
+    uint64_t member_count, int32_t encoding, uint64_t second_level_block,
+    uint64_t rows, uint64_t input_width, uint64_t block_size, void* stream);
 
 /*
  * y = x.deq(W)^T + bias + lora_scale * ((x.A^T).B^T)

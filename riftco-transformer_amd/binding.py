@@ -92,6 +92,13 @@ class Member(ctypes.Structure):
                 ("bias_or_null", _ptr), ("y", _ptr), ("output_width", _u64)]
 
 
+class LoraMember(ctypes.Structure):
+    """rthip_nf4_lora_member: a member with an optional adapter term."""
+
+    _fields_ = [("base", Member), ("reduced", _ptr), ("lora_b", _ptr),
+                ("lora_rank", _u64), ("lora_scale", _f32)]
+
+
 _PROTOTYPES = {
     "rthip_abi_version": (ctypes.c_uint32, []),
     "rthip_last_error": (ctypes.c_char_p, []),
@@ -118,6 +125,9 @@ _PROTOTYPES = {
         _i32, [_i32, _ptr] + _WEIGHT + [_ptr, _u64, _u64, _u64, _u64, _ptr]),
     "rthip_nf4_linear_forward_group": (
         _i32, [_ptr, ctypes.POINTER(Member), _u64, _i32, _u64, _u64, _u64,
+               _u64, _ptr]),
+    "rthip_nf4_lora_linear_forward_group": (
+        _i32, [_ptr, ctypes.POINTER(LoraMember), _u64, _i32, _u64, _u64, _u64,
                _u64, _ptr]),
     "rthip_matmul": (
         _i32, [_ptr, _ptr, _ptr, _u64, _u64, _u64, _u64, _ptr]),
@@ -324,6 +334,37 @@ class Library:
             slot.y = y_ptr
             slot.output_width = weight.output_width
         self._check(self._lib.rthip_nf4_linear_forward_group(
+            x_ptr, array, len(members), first.encoding,
+            first.second_level_block, rows, first.input_width,
+            first.block_size, stream))
+
+    def lora_linear_forward_group(self, x_ptr: int, members, rows: int,
+                                  stream: int = 0) -> None:
+        """members: (weight, bias_ptr or None, y_ptr, adapter) where adapter is
+        None or (reduced_ptr, lora_b_ptr, rank, scale); `reduced` already
+        holds x.A^T."""
+        first = members[0][0]
+        array = (LoraMember * len(members))()
+        for slot, (weight, bias_ptr, y_ptr, adapter) in zip(array, members):
+            if (weight.input_width, weight.block_size, weight.encoding,
+                    weight.second_level_block) != (
+                    first.input_width, first.block_size, first.encoding,
+                    first.second_level_block):
+                raise ValueError("the weights of a group must share input "
+                                 "width, block size and scale encoding")
+            slot.base.codes = weight.codes.data_ptr()
+            slot.base.primary_scales = weight.primary_scales.data_ptr()
+            slot.base.secondary_scales = (
+                None if weight.secondary_scales is None
+                else weight.secondary_scales.data_ptr())
+            slot.base.offset = weight.offset
+            slot.base.bias_or_null = bias_ptr
+            slot.base.y = y_ptr
+            slot.base.output_width = weight.output_width
+            if adapter is not None:
+                (slot.reduced, slot.lora_b, slot.lora_rank,
+                 slot.lora_scale) = adapter
+        self._check(self._lib.rthip_nf4_lora_linear_forward_group(
             x_ptr, array, len(members), first.encoding,
             first.second_level_block, rows, first.input_width,
             first.block_size, stream))

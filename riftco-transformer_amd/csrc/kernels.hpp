@@ -63,6 +63,10 @@ void launch_gemv_group(const LinearProblem* problems, std::size_t count,
 // gemv1_forward_supports accepts.  launch_gemv_forward / launch_gemv_group
 // route here by themselves.
 bool gemv1_forward_supports(const LinearProblem& problem);
+// Up to kGemvGroupMax members, each accepted by gemv1_forward_supports, that
+// share x, row count, row width and scale encoding; every member may carry its
+// own adapter term.
+bool gemv1_group_supports(const LinearProblem* problems, std::size_t count);
 void launch_gemv1_forward(const LinearProblem* problems, std::size_t count,
                           hipStream_t stream);
 // The name of the instance that launch would run, as a profiler prints it

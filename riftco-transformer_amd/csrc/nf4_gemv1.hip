@@ -95,6 +95,7 @@ struct OneRowTarget {
     const float* bias;
     unsigned output_width;
     unsigned first_batch;
+    LoraEpilogue lora;  // the member's adapter term (reduced == null: none)
 };
 // Members 1 ... of a grouped launch (member 0's source is passed as plain
 // kernel arguments, see the kernel), and every member's target.
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
     float offset_of_scales,
     // read from memory
     unsigned second_level_shift, unsigned batch_count, unsigned x_rows,
-    const OneRowRest<kMembers> rest, const LoraEpilogue lora
+    const OneRowRest<kMembers> rest
 ) {
     constexpr bool kGrouped = kMembers > 1;
     constexpr unsigned kMaxIterations = kParkedRows / (kRows * kX);
@@ -483,8 +484,8 @@ __global__ __launch_bounds__(kThreads) void gemv1_forward_kernel(
             if (target.bias != nullptr) {
                 sum += target.bias[o];
             }
-            if (!kGrouped && lora.reduced != nullptr) {
-                sum += lora_term(lora, r, o);
+            if (target.lora.reduced != nullptr) {
+                sum += lora_term(target.lora, r, o);
             }
             target.y[r * target.output_width + o] = sum;
         }
@@ -559,6 +560,7 @@ void launch_instance(const LinearProblem* problems, std::size_t count,
         source.offset = p.weight.offset;
         target.y = p.result;
         target.bias = p.bias;
+        target.lora = p.lora;
         target.output_width = static_cast<unsigned>(p.output_width);
         batch_count += static_cast<unsigned>(p.output_width / kRows);
     }
@@ -592,7 +594,7 @@ void launch_instance(const LinearProblem* problems, std::size_t count,
                 head.primary_bytes, iterations, head.secondary_scales,
                 head.secondary_bytes, head.offset,
                 first.weight.second_level_shift, batch_count,
-                static_cast<unsigned>(first.rows), rest, first.lora);
+                static_cast<unsigned>(first.rows), rest);
     };
     if constexpr (kDoubleQuantized) {
         const std::size_t batch_blocks =
@@ -670,6 +672,25 @@ bool gemv1_forward_supports(const LinearProblem& p) {
            p.rows * p.output_width < (1ULL << 32) &&
            reinterpret_cast<std::uintptr_t>(p.weight.codes) % 4 == 0 &&
            reinterpret_cast<std::uintptr_t>(p.activations) % 16 == 0;
+}
+
+bool gemv1_group_supports(const LinearProblem* problems, std::size_t count) {
+    if (count < 1 || count > kGemvGroupMax) {
+        return false;
+    }
+    const LinearProblem& first = problems[0];
+    std::size_t batches = 0;
+    for (std::size_t m = 0; m < count; ++m) {
+        const LinearProblem& p = problems[m];
+        if (!gemv1_forward_supports(p) || p.activations != first.activations ||
+            p.rows != first.rows || p.input_width != first.input_width ||
+            p.weight.encoding != first.weight.encoding ||
+            p.weight.second_level_shift != first.weight.second_level_shift) {
+            return false;
+        }
+        batches += (p.output_width + 1) / 2;  // at least two rows per batch
+    }
+    return batches < (1ULL << 31);
 }
 
 void launch_gemv1_forward(const LinearProblem* problems, std::size_t count,

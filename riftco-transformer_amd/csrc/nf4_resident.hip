@@ -91,6 +91,7 @@ struct ResidentMember {
     const float* bias;
     float* y;
     unsigned output_width;
+    LoraEpilogue lora;  // the member's adapter term (reduced == null: none)
 };
 struct ResidentGroup {
     ResidentMember member[kResidentGroupMax];
@@ -104,8 +105,7 @@ struct ResidentGroup {
 template <int kGroups, bool kDoubleQuantized, bool kGrouped>
 __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
     const float* __restrict__ x, ResidentGroup group, unsigned rows,
-    unsigned block_shift, unsigned row_groups, unsigned iterations,
-    LoraEpilogue lora
+    unsigned block_shift, unsigned row_groups, unsigned iterations
 ) {
     constexpr unsigned kInputWidth = 1024U * kGroups;
     constexpr int kSubChunks = 2 * kGroups;  // 16 weights each
@@ -389,8 +389,8 @@ __global__ __launch_bounds__(kThreads) void resident_forward_kernel(
             if (member.bias != nullptr) {
                 sum += member.bias[n];
             }
-            if (lora.reduced != nullptr) {
-                sum += lora_term(lora, row_base + m_row, n);
+            if (member.lora.reduced != nullptr) {
+                sum += lora_term(member.lora, row_base + m_row, n);
             }
             member.y[static_cast<std::size_t>(row_base + m_row) *
                          member.output_width +
@@ -432,6 +432,7 @@ hipError_t launch_instance(const LinearProblem* problems, std::size_t count,
             group.member[m].y = member.result;
             group.member[m].output_width =
                 static_cast<unsigned>(member.output_width);
+            group.member[m].lora = member.lora;
             tiles += static_cast<unsigned>(
                 (member.output_width + kTileRows - 1) / kTileRows + 7) / 8 * 8;
         }
@@ -464,7 +465,7 @@ hipError_t launch_instance(const LinearProblem* problems, std::size_t count,
     }
     kernel<<<groups, kThreads, shared_bytes, stream>>>(
         p.activations, group, static_cast<unsigned>(p.rows), p.block_shift,
-        row_groups, iterations, p.lora);
+        row_groups, iterations);
     return hipSuccess;
 }
 
@@ -520,7 +521,7 @@ bool resident_group_supports(const LinearProblem* problems,
     std::size_t tiles = 0;
     for (std::size_t m = 0; m < count; ++m) {
         const LinearProblem& p = problems[m];
-        if (!resident_forward_supports(p) || p.lora.reduced != nullptr ||
+        if (!resident_forward_supports(p) ||
             p.activations != first.activations || p.rows != first.rows ||
             p.input_width != first.input_width ||
             p.block_shift != first.block_shift ||

@@ -671,6 +671,8 @@ rthip_status rthip_nf4_select_algorithm(
 namespace {
 
 // The adapter arguments of the *_lora_* entry points; a == nullptr: none.
+constexpr uint64_t kMaxGroupMembers = 64;
+
 struct LoraArguments {
     const float* a;
     const float* b;
@@ -989,24 +991,30 @@ rthip_status rthip_nf4_linear_forward(
         input_width, output_width, block_size, stream);
 }
 
-rthip_status rthip_nf4_linear_forward_group(
-    const float* x, const rthip_nf4_member* members, uint64_t member_count,
+namespace {
+
+// A member of a grouped forward: the weight, bias and output of
+// rthip_nf4_member and, when `lora.reduced` is set, the adapter term of
+// rthip_nf4_lora_member.
+struct GroupMember {
+    rthip_nf4_member base;
+    LoraArguments lora;
+};
+
+static rthip_status forward_group(
+    const float* x, const GroupMember* members, uint64_t member_count,
     int32_t encoding, uint64_t second_level_block, uint64_t rows,
     uint64_t input_width, uint64_t block_size, void* stream
 ) {
-    constexpr uint64_t kMaxMembers = 64;
-    if (x == nullptr || members == nullptr) {
-        return fail(RTHIP_INVALID_ARGUMENT,
-                    "input and members must not be null");
-    }
-    if (member_count == 0 || member_count > kMaxMembers) {
+    if (member_count == 0 || member_count > kMaxGroupMembers) {
         return fail(RTHIP_INVALID_ARGUMENT,
                     "a group holds between 1 and %llu weights",
-                    static_cast<unsigned long long>(kMaxMembers));
+                    static_cast<unsigned long long>(kMaxGroupMembers));
     }
-    rthip::LinearProblem problems[kMaxMembers];
+    rthip::LinearProblem problems[kMaxGroupMembers];
     for (uint64_t m = 0; m < member_count; ++m) {
-        const rthip_nf4_member& member = members[m];
+        const rthip_nf4_member& member = members[m].base;
+        const LoraArguments& lora = members[m].lora;
         rthip::LinearProblem& problem = problems[m];
         problem = rthip::LinearProblem{};
         if (member.y == nullptr) {
@@ -1018,7 +1026,7 @@ rthip_status rthip_nf4_linear_forward_group(
                         "quantized linear input and output must not alias");
         }
         for (uint64_t other = 0; other < m; ++other) {
-            if (members[other].y == member.y) {
+            if (members[other].base.y == member.y) {
                 return fail(RTHIP_INVALID_ARGUMENT,
                             "two members of a group write the same output");
             }
@@ -1041,26 +1049,56 @@ rthip_status rthip_nf4_linear_forward_group(
         problem.rows = rows;
         problem.input_width = input_width;
         problem.output_width = member.output_width;
+        if (lora.reduced != nullptr) {
+            if (const rthip_status status = check_lora_arguments(
+                    lora, x, member.y, rows, input_width, member.output_width);
+                status != RTHIP_OK) {
+                return status;
+            }
+            problem.lora.reduced = lora.reduced;
+            problem.lora.b = lora.b;
+            problem.lora.rank = static_cast<unsigned>(lora.rank);
+            problem.lora.scale = lora.scale;
+            problem.lora.row_stride = static_cast<unsigned>(lora.rank);
+            problem.lora.rank_stride = 1;
+        }
     }
     if (const rthip_status status = require_device(); status != RTHIP_OK) {
         return status;
     }
     const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+    const auto with_adapter = [&](uint64_t first, uint64_t length) {
+        for (uint64_t m = first; m < first + length; ++m) {
+            if (problems[m].lora.reduced != nullptr) {
+                return true;
+            }
+        }
+        return false;
+    };
     uint64_t next = 0;
     while (next < member_count) {
         // the longest run of members from here that one streaming launch takes
+        // (members with an adapter term: the one-row kernel only, and only
+        // two or more -- one alone goes the way of a call of its own)
         uint64_t run = 0;
         if (rows <= rthip::kGemvMaxRows) {
             run = member_count - next < rthip::kGemvGroupMax
                       ? member_count - next
                       : rthip::kGemvGroupMax;
             while (run > 0 &&
-                   !rthip::gemv_group_supports(problems + next, run)) {
+                   !(with_adapter(next, run)
+                         ? run > 1 && rthip::gemv1_group_supports(
+                                          problems + next, run)
+                         : rthip::gemv_group_supports(problems + next, run))) {
                 --run;
             }
         }
         if (run > 0) {
-            rthip::launch_gemv_group(problems + next, run, hip_stream);
+            if (with_adapter(next, run)) {
+                rthip::launch_gemv1_forward(problems + next, run, hip_stream);
+            } else {
+                rthip::launch_gemv_group(problems + next, run, hip_stream);
+            }
             if (const rthip_status status =
                     finish_launch("NF4 linear forward launch");
                 status != RTHIP_OK) {
@@ -1107,19 +1145,69 @@ rthip_status rthip_nf4_linear_forward_group(
             next += run;
             continue;
         }
-        const rthip_nf4_member& member = members[next];
+        const rthip_nf4_member& member = members[next].base;
         if (const rthip_status status = linear_forward_common(
                 RTHIP_NF4_ALGORITHM_AUTO, x, member.codes,
                 member.primary_scales, member.secondary_scales, encoding,
                 second_level_block, member.offset, member.bias_or_null,
-                LoraArguments{nullptr, nullptr, 0, 0.0F, nullptr}, member.y,
-                rows, input_width, member.output_width, block_size, stream);
+                members[next].lora, member.y, rows, input_width,
+                member.output_width, block_size, stream);
             status != RTHIP_OK) {
             return status;
         }
         ++next;
     }
     return ok();
+}
+
+}  // namespace
+
+rthip_status rthip_nf4_linear_forward_group(
+    const float* x, const rthip_nf4_member* members, uint64_t member_count,
+    int32_t encoding, uint64_t second_level_block, uint64_t rows,
+    uint64_t input_width, uint64_t block_size, void* stream
+) {
+    if (x == nullptr || members == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "input and members must not be null");
+    }
+    GroupMember group[kMaxGroupMembers];
+    for (uint64_t m = 0; m < member_count && m < kMaxGroupMembers; ++m) {
+        group[m].base = members[m];
+        group[m].lora = LoraArguments{nullptr, nullptr, 0, 0.0F, nullptr};
+    }
+    return forward_group(x, group, member_count, encoding, second_level_block,
+                         rows, input_width, block_size, stream);
+}
+
+rthip_status rthip_nf4_lora_linear_forward_group(
+    const float* x, const rthip_nf4_lora_member* members,
+    uint64_t member_count, int32_t encoding, uint64_t second_level_block,
+    uint64_t rows, uint64_t input_width, uint64_t block_size, void* stream
+) {
+    if (x == nullptr || members == nullptr) {
+        return fail(RTHIP_INVALID_ARGUMENT,
+                    "input and members must not be null");
+    }
+    GroupMember group[kMaxGroupMembers];
+    for (uint64_t m = 0; m < member_count && m < kMaxGroupMembers; ++m) {
+        const rthip_nf4_lora_member& member = members[m];
+        group[m].base = member.base;
+        group[m].lora = LoraArguments{nullptr, nullptr, 0, 0.0F, nullptr};
+        if (member.lora_b != nullptr || member.reduced != nullptr) {
+            // (the reduced buffer is only read here)
+            group[m].lora = LoraArguments{
+                nullptr, member.lora_b, member.lora_rank, member.lora_scale,
+                const_cast<float*>(member.reduced)};
+            if (member.reduced == nullptr) {
+                return fail(RTHIP_INVALID_ARGUMENT,
+                            "the adapter's B matrix and the reduced buffer "
+                            "must not be null");
+            }
+        }
+    }
+    return forward_group(x, group, member_count, encoding, second_level_block,
+                         rows, input_width, block_size, stream);
 }
 
 rthip_status rthip_nf4_linear_input_backward_with(

@@ -107,6 +107,44 @@ def linear_forward_group(x: torch.Tensor, weights, biases=None):
     return outs
 
 
+def lora_linear_forward_group(x: torch.Tensor, weights, adapters,
+                              biases=None):
+    """Like linear_forward_group for layers with low-rank adapters:
+    adapters[m] is None or (lora_a, lora_b, lora_scale).  x . A_m^T is taken
+    first (rthip_lora_reduce per adapter), then ONE call of
+    rthip_nf4_lora_linear_forward_group.  Returns (outputs, reduced) where
+    reduced[m] is x . A_m^T or None."""
+    assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous()
+    library = load_library()
+    rows = x.numel() // weights[0].input_width
+    if biases is None:
+        biases = [None] * len(weights)
+    outs = [torch.empty((rows, weight.output_width), dtype=torch.float32,
+                        device=x.device) for weight in weights]
+    reduced = []
+    members = []
+    for weight, bias, out, adapter in zip(weights, biases, outs, adapters):
+        entry = None
+        if adapter is None:
+            reduced.append(None)
+        else:
+            lora_a, lora_b, lora_scale = adapter
+            rank = lora_a.shape[0]
+            assert tuple(lora_a.shape) == (rank, weight.input_width)
+            assert tuple(lora_b.shape) == (weight.output_width, rank)
+            product = torch.empty((rows, rank), dtype=torch.float32,
+                                  device=x.device)
+            library.lora_reduce(x.data_ptr(), lora_a.data_ptr(),
+                                product.data_ptr(), rows, weight.input_width,
+                                rank, _stream())
+            reduced.append(product)
+            entry = (product.data_ptr(), lora_b.data_ptr(), rank, lora_scale)
+        members.append((weight, None if bias is None else bias.data_ptr(),
+                        out.data_ptr(), entry))
+    library.lora_linear_forward_group(x.data_ptr(), members, rows, _stream())
+    return outs, reduced
+
+
 def lora_linear_forward(x: torch.Tensor, weight: DeviceWeight,
                         lora_a: torch.Tensor, lora_b: torch.Tensor,
                         lora_scale: float,

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol(package, library):
 
 
 def test_abi_version(package, library):
-    assert library.abi_version() == (1, 9)
+    assert library.abi_version() == (1, 10)
 
 
 def test_select_algorithm_is_pure_host_logic(package, library):

@@ -179,3 +179,103 @@ def test_adapter_epilogue_of_the_decode_kernel(gpu, package, library, oracle,
     error = helpers.normalized_error(y, exact, in_w, helpers.rms(x),
                                      helpers.rms(dense))
     assert error <= 2 * TOLERANCE, f"{error:.3g}"
+
+
+@pytest.mark.parametrize("double_quantized", [False, True])
+@pytest.mark.parametrize("rows", [1, 2, 4, 5, 16, 64, 130])
+def test_groups_with_adapters_equal_their_members_launched_alone(
+        gpu, package, library, oracle, double_quantized, rows):
+    """rthip_nf4_lora_linear_forward_group: members with and without a
+    low-rank adapter term (ranks 16, 4 and 33), with and without bias, one
+    that the one-row kernel does not take (output width 100), at row counts
+    of the decode kernel (<= 4), of the kernel that keeps x in registers
+    (<= 128) and beyond (one launch per member).  Every output equals the
+    member's own call bit for bit, and the adapted ones are within the bar of
+    fp64 over deq(W)."""
+    import torch
+    in_w = 4096
+    widths = [4096, 1024, 4096, 100]
+    weights = [oracle.quantize(helpers.normal(61 + m, (width, in_w), 0.02), 64,
+                               double_quantized, 256)
+               for m, width in enumerate(widths)]
+    device_weights = [upload(gpu, weight) for weight in weights]
+    x = to_device(helpers.normal(70 + rows, (rows, in_w), 1.0))
+    ranks = [16, None, 4, 33]
+    adapters = []
+    for m, rank in enumerate(ranks):
+        if rank is None:
+            adapters.append(None)
+            continue
+        adapters.append((to_device(helpers.normal(80 + m, (rank, in_w), 0.05)),
+                         to_device(helpers.normal(90 + m, (widths[m], rank),
+                                                  0.05)),
+                         0.25 * (m + 1)))
+    biases = [None, to_device(helpers.normal(95, (widths[1],), 0.01)),
+              to_device(helpers.normal(96, (widths[2],), 0.01)), None]
+    for members in ([0, 1, 2], [0, 2], [1, 0, 3, 2], [3, 0]):
+        together, reduced = gpu.lora_linear_forward_group(
+            x, [device_weights[m] for m in members],
+            [adapters[m] for m in members], [biases[m] for m in members])
+        torch.cuda.synchronize()
+        for m, got, product in zip(members, together, reduced):
+            if adapters[m] is None:
+                want = gpu.linear_forward(x, device_weights[m], biases[m])
+            else:
+                lora_a, lora_b, scale = adapters[m]
+                want, own = gpu.lora_linear_forward(
+                    x, device_weights[m], lora_a, lora_b, scale,
+                    bias=biases[m])
+                helpers.assert_bit_equal(host(product), host(own),
+                                         f"x.A^T of member {m}")
+            helpers.assert_bit_equal(host(got), host(want),
+                                     f"member {m} of group {members}")
+    # the adapted members against fp64
+    together, _ = gpu.lora_linear_forward_group(x, device_weights, adapters,
+                                                biases)
+    x64 = host(x).astype(np.float64)
+    for m, got in enumerate(together):
+        dense = oracle.dequantize(weights[m]).astype(np.float64)
+        exact = x64 @ dense.T
+        if biases[m] is not None:
+            exact = exact + host(biases[m]).astype(np.float64)
+        if adapters[m] is not None:
+            lora_a, lora_b, scale = adapters[m]
+            exact = exact + scale * (
+                x64 @ host(lora_a).astype(np.float64).T) @ \
+                host(lora_b).astype(np.float64).T
+        error = helpers.normalized_error(host(got), exact, in_w,
+                                         helpers.rms(host(x)),
+                                         helpers.rms(dense))
+        assert error <= 2 * TOLERANCE, f"member {m}: {error:.3g}"
+
+
+def test_grouped_adapter_arguments_are_checked(gpu, package, library, oracle):
+    """A member that names an adapter without its reduced buffer, a rank of
+    zero, and two members writing one output are refused before anything is
+    launched."""
+    import torch
+    weight = upload(gpu, oracle.quantize(helpers.normal(7, (64, 256), 0.02),
+                                         64, False, 256))
+    x = torch.zeros(1, 256, device="cuda")
+    y = torch.zeros(1, 64, device="cuda")
+    z = torch.zeros(1, 64, device="cuda")
+    b = torch.zeros(64, 4, device="cuda")
+    reduced = torch.zeros(1, 4, device="cuda")
+    raw = library
+    with pytest.raises(package.RthipError, match="reduced buffer"):
+        raw.lora_linear_forward_group(
+            x.data_ptr(), [(weight, None, y.data_ptr(),
+                            (None, b.data_ptr(), 4, 1.0))], 1)
+    with pytest.raises(package.RthipError, match="rank"):
+        raw.lora_linear_forward_group(
+            x.data_ptr(), [(weight, None, y.data_ptr(),
+                            (reduced.data_ptr(), b.data_ptr(), 0, 1.0))], 1)
+    with pytest.raises(package.RthipError, match="same output"):
+        raw.lora_linear_forward_group(
+            x.data_ptr(), [(weight, None, y.data_ptr(), None),
+                           (weight, None, y.data_ptr(), None)], 1)
+    # and a well-formed single member runs
+    raw.lora_linear_forward_group(
+        x.data_ptr(), [(weight, None, z.data_ptr(),
+                        (reduced.data_ptr(), b.data_ptr(), 4, 1.0))], 1)
+    torch.cuda.synchronize()
