@@ -736,6 +736,104 @@ def bench_lora(package, device, torch, steps):
     return results
 
 
+def bench_decode_with_adapters(package, device, torch, layers, steps,
+                               rank=16):
+    """The decode step of a model whose query and value projections carry
+    unmerged low-rank adapters (QLoRA serving), M = 1, fp32 scales, three
+    ways: one call per projection (q and v through
+    rthip_nf4_lora_linear_forward: x.A^T and the packed product, two launches
+    each), the shared-input groups with one rthip_lora_reduce per adapter and
+    q/k/v through rthip_nf4_lora_linear_forward_group, and the same with ONE
+    rthip_lora_reduce over the stacked A of q and v (rows = 1: the members'
+    reduced vectors lie side by side)."""
+    library = package.load_library()
+    x = {width: torch.randn(1, width, device="cuda")
+         for width in (4096, 11008)}
+    outputs = {}
+    per_layer = []
+    payload = 0
+    for layer in range(layers):
+        weights = {}
+        for index, (name, out_w, in_w) in enumerate(LAYER_SHAPES):
+            weights[name] = synthetic_weight(package, torch, out_w, in_w,
+                                             False, 3000 * (layer + 1) + index)
+            payload += weights[name].payload_bytes
+            outputs.setdefault(name, torch.empty(1, out_w, device="cuda"))
+        stacked_a = torch.randn(2 * rank, 4096, device="cuda") * 0.05
+        factors = {name: torch.randn(4096, rank, device="cuda") * 0.05
+                   for name in ("q_proj", "v_proj")}
+        reduced = torch.zeros(1, 2 * rank, device="cuda")
+        per_layer.append((weights, stacked_a, factors, reduced))
+    scale = 2.0
+
+    def adapter(entry, name):
+        _, stacked_a, factors, reduced = entry
+        slot = 0 if name == "q_proj" else 1
+        return (stacked_a[slot * rank:(slot + 1) * rank],
+                factors[name], reduced[:, slot * rank:(slot + 1) * rank])
+
+    def per_projection():
+        stream = torch.cuda.current_stream().cuda_stream
+        for entry in per_layer:
+            for name, _, in_w in LAYER_SHAPES:
+                weight = entry[0][name]
+                if name in entry[2]:
+                    lora_a, lora_b, product = adapter(entry, name)
+                    library.lora_linear_forward(
+                        x[in_w].data_ptr(), weight, None, lora_a.data_ptr(),
+                        lora_b.data_ptr(), rank, scale, product.data_ptr(),
+                        outputs[name].data_ptr(), 1, stream)
+                else:
+                    library.linear_forward(x[in_w].data_ptr(), weight, None,
+                                           outputs[name].data_ptr(), 1,
+                                           stream)
+
+    def grouped(stacked):
+        stream = torch.cuda.current_stream().cuda_stream
+        for entry in per_layer:
+            weights, stacked_a, _, reduced = entry
+            if stacked:
+                library.lora_reduce(x[4096].data_ptr(), stacked_a.data_ptr(),
+                                    reduced.data_ptr(), 1, 4096, 2 * rank,
+                                    stream)
+            for group in SHARED_INPUT_GROUPS:
+                members = []
+                for name in group:
+                    entry_adapter = None
+                    if name in entry[2]:
+                        lora_a, lora_b, product = adapter(entry, name)
+                        if not stacked:
+                            library.lora_reduce(
+                                x[4096].data_ptr(), lora_a.data_ptr(),
+                                product.data_ptr(), 1, 4096, rank, stream)
+                        entry_adapter = (product.data_ptr(),
+                                         lora_b.data_ptr(), rank, scale)
+                    members.append((weights[name], None,
+                                    outputs[name].data_ptr(), entry_adapter))
+                in_w = members[0][0].input_width
+                if len(members) == 1:
+                    library.linear_forward(x[in_w].data_ptr(), members[0][0],
+                                           None, members[0][2], 1, stream)
+                else:
+                    library.lora_linear_forward_group(x[in_w].data_ptr(),
+                                                      members, 1, stream)
+
+    results = {"rank": rank, "layers": layers, "bytes_per_step": payload,
+               "adapters_on": ["q_proj", "v_proj"]}
+    for label, body in (
+            ("one_call_per_projection", per_projection),
+            ("shared_input_groups", lambda: grouped(False)),
+            ("shared_input_groups_stacked_reduce", lambda: grouped(True))):
+        body()
+        torch.cuda.synchronize()
+        replay = capture(torch, body)
+        warm(torch, replay, 0.02)
+        milliseconds = time_region(torch, replay, steps) / steps
+        results[label] = {"ms_per_step": milliseconds,
+                          "gb_per_s": payload / milliseconds / 1e6}
+    return results
+
+
 def bench_matmul(package, device, torch, steps):
     """Dense fp32 matmul at the layer's shapes and at adapter shapes."""
     results = []
@@ -1059,6 +1157,8 @@ def main():
             line["small_batch_input_backward"] = bench_small_batch_backward(
                 package, device, torch, few)
             line["lora"] = bench_lora(package, device, torch, few)
+            line["decode_with_adapters"] = bench_decode_with_adapters(
+                package, device, torch, arguments.layers, fewer)
             line["matmul"] = bench_matmul(package, device, torch, few)
             line["quantizer"] = bench_quantizer(package, device, torch)
     if not arguments.skip_cpu:

@@ -338,21 +338,33 @@ public:
         return pending;
     }
 
-    void add(const Shape& shape, const rthip_nf4_member& member) {
+    // `before_joining` runs once the list is known to take the member (what
+    // does not fit has been launched) and before the member joins it: the
+    // place for a launch that the member's own launch depends on and that
+    // must not overtake the one that produces its input.
+    template <typename BeforeJoining>
+    void add(const Shape& shape, const rthip_nf4_lora_member& member,
+             BeforeJoining&& before_joining) {
         const std::lock_guard<std::mutex> lock(mutex_);
         ++statistics_.requests;
         bool fits = count_ != 0 && count_ < kCapacity && shape == shape_;
         for (std::size_t m = 0; fits && m < count_; ++m) {
-            fits = members_[m].y != member.y;
+            fits = members_[m].base.y != member.base.y;
         }
         if (!fits) {
             launch_locked();
         }
+        before_joining();
         shape_ = shape;
         members_[count_++] = member;
         if (count_ == kCapacity) {
             launch_locked();
         }
+    }
+    void add(const Shape& shape, const rthip_nf4_member& member) {
+        rthip_nf4_lora_member plain{};
+        plain.base = member;
+        add(shape, plain, [] {});
     }
 
     void launch() {
@@ -373,17 +385,29 @@ private:
         const std::size_t count = std::exchange(count_, 0);
         ++statistics_.launches;
         const HipRuntime& runtime = require_runtime();
+        bool adapters = false;
+        std::array<rthip_nf4_member, kCapacity> plain{};
+        for (std::size_t m = 0; m < count; ++m) {
+            adapters = adapters || members_[m].reduced != nullptr;
+            plain[m] = members_[m].base;
+        }
         check(runtime,
-              runtime.nf4_linear_forward_group(
-                  shape_.input, members_.data(), count, shape_.encoding,
-                  shape_.second_level_block, shape_.rows, shape_.input_width,
-                  shape_.block_size, nullptr),
+              adapters ? runtime.nf4_lora_linear_forward_group(
+                             shape_.input, members_.data(), count,
+                             shape_.encoding, shape_.second_level_block,
+                             shape_.rows, shape_.input_width,
+                             shape_.block_size, nullptr)
+                       : runtime.nf4_linear_forward_group(
+                             shape_.input, plain.data(), count,
+                             shape_.encoding, shape_.second_level_block,
+                             shape_.rows, shape_.input_width,
+                             shape_.block_size, nullptr),
               "quantized-linear forward (merged launch)");
     }
 
     std::mutex mutex_;
     Shape shape_;
-    std::array<rthip_nf4_member, kCapacity> members_{};
+    std::array<rthip_nf4_lora_member, kCapacity> members_{};
     std::size_t count_ = 0;
     HipForwardMergeStatistics statistics_{};
 };
@@ -1095,7 +1119,6 @@ void hip_quantized_linear_adapter_forward(
         require_elements(*request.bias, 1, d.output_width, "bias");
     }
     const HipRuntime& runtime = require_runtime();
-    launch_pending_forwards();
     const auto& input = require_hip_tensor(request.input, operation);
     const auto& weight = require_hip_weight(request.weight, operation);
     const auto& lora_a = require_hip_tensor(request.lora_a, operation);
@@ -1106,6 +1129,42 @@ void hip_quantized_linear_adapter_forward(
     if (request.bias != nullptr) {
         bias = require_hip_tensor(*request.bias, operation).device_for_read();
     }
+    if (merge_requested() && d.rows <= PendingForwards::kMaximumRows) {
+        // The layer joins the forwards that are held back for its input (the
+        // query and value projections of a decoder carry adapters, the key
+        // projection between them does not): x.A^T goes out now, the packed
+        // product with bias and adapter term with the rest of the list.
+        const float* source = input.device_for_read();
+        rthip_nf4_lora_member member{};
+        member.base.codes = static_cast<const std::uint8_t*>(
+            weight.packed_codes_native_handle());
+        member.base.primary_scales = weight.primary_scales_native_handle();
+        member.base.secondary_scales = static_cast<const float*>(
+            weight.secondary_scales_native_handle());
+        member.base.offset = weight.offset();
+        member.base.bias_or_null = bias;
+        member.base.y = output.device_for_overwrite();
+        member.base.output_width = d.output_width;
+        float* const product = reduced.device_for_overwrite();
+        member.reduced = product;
+        member.lora_b = lora_b.device_for_read();
+        member.lora_rank = request.rank;
+        member.lora_scale = request.scale;
+        const float* const factor = lora_a.device_for_read();
+        PendingForwards::instance().add(
+            {source, static_cast<std::int32_t>(weight.encoding()),
+             weight.second_level_block_size(), d.rows, d.input_width,
+             d.block_size},
+            member, [&] {
+                check(runtime,
+                      runtime.lora_reduce(source, factor, product, d.rows,
+                                          d.input_width, request.rank,
+                                          nullptr),
+                      operation);
+            });
+        return;
+    }
+    launch_pending_forwards();
     check(runtime,
           runtime.nf4_lora_linear_forward(
               input.device_for_read(),

@@ -43,6 +43,9 @@ struct HipRuntime {
     decltype(&rthip_matmul) matmul = nullptr;
     decltype(&rthip_nf4_lora_linear_forward) nf4_lora_linear_forward =
         nullptr;
+    decltype(&rthip_nf4_lora_linear_forward_group)
+        nf4_lora_linear_forward_group = nullptr;
+    decltype(&rthip_lora_reduce) lora_reduce = nullptr;
     decltype(&rthip_lora_backward) lora_backward = nullptr;
     decltype(&rthip_nf4_lora_linear_input_backward)
         nf4_lora_linear_input_backward = nullptr;

@@ -622,6 +622,107 @@ void test_adapter_layer() {
     }
 }
 
+void test_merged_adapter_forwards() {
+    // A decoder whose query and value projections carry adapters: q (adapter,
+    // bias), k (plain, through the dispatcher), v (adapter) on one input, then
+    // a dependent layer whose input is q's output.  Unless
+    // RIFTCO_TRANSFORMER_HIP_MERGE=0 the first three are one launch (their
+    // x.A^T products go out at once) and the dependent one is launched only
+    // after them.
+    namespace detail = riftco_transformer::backend_detail;
+    const char* option = std::getenv("RIFTCO_TRANSFORMER_HIP_MERGE");
+    const bool merging = option == nullptr || std::string_view(option) != "0";
+    const std::size_t in_w = 256, out_w = 256, rank = 4;
+    const float scale = 0.5F;
+    for (const bool double_quantized : {false, true}) {
+        std::vector<HostWeight> weights;
+        std::vector<std::unique_ptr<backend::QuantizedWeightStorage>> storages;
+        for (std::size_t m = 0; m < 4; ++m) {
+            weights.push_back(quantize(
+                pseudo_normal(out_w * in_w, 0.02F, 170 + m), out_w, in_w, 64,
+                double_quantized, 32));
+            storages.push_back(to_hip(weights.back()));
+        }
+        const auto a_values = pseudo_normal(rank * in_w, 0.05F, 181);
+        const auto b_values = pseudo_normal(out_w * rank, 0.05F, 182);
+        const auto bias_values = pseudo_normal(out_w, 0.01F, 183);
+        for (const std::size_t rows : {std::size_t{1}, std::size_t{4},
+                                       std::size_t{9}}) {
+            const auto x = pseudo_normal(rows * in_w, 1.0F, 184 + rows);
+            auto input = backend::make_tensor_storage(kHip, x);
+            auto lora_a = backend::make_tensor_storage(kHip, a_values);
+            auto lora_b = backend::make_tensor_storage(kHip, b_values);
+            auto bias = backend::make_tensor_storage(kHip, bias_values);
+            std::vector<std::unique_ptr<backend::TensorStorage>> outputs;
+            std::vector<std::unique_ptr<backend::TensorStorage>> products;
+            for (std::size_t m = 0; m < 4; ++m) {
+                outputs.push_back(
+                    backend::make_tensor_storage(kHip, rows * out_w, 0.0F));
+                products.push_back(
+                    backend::make_tensor_storage(kHip, rows * rank, 0.0F));
+            }
+            const backend::QuantizedLinearDimensions dimensions{rows, in_w,
+                                                                out_w, 64};
+            const auto before = detail::hip_forward_merge_statistics();
+            detail::hip_quantized_linear_adapter_forward(
+                {*input, *storages[0], bias.get(), *lora_a, *lora_b, rank,
+                 scale, *products[0], *outputs[0], dimensions});
+            backend::dispatch_quantized_linear_forward(
+                kHip, {*input, *storages[1], *outputs[1], dimensions});
+            detail::hip_quantized_linear_adapter_forward(
+                {*input, *storages[2], nullptr, *lora_a, *lora_b, rank, scale,
+                 *products[2], *outputs[2], dimensions});
+            // reads q's output: what is held back goes out first
+            detail::hip_quantized_linear_adapter_forward(
+                {*outputs[0], *storages[3], nullptr, *lora_a, *lora_b, rank,
+                 scale, *products[3], *outputs[3], dimensions});
+            const auto after_calls = detail::hip_forward_merge_statistics();
+
+            std::vector<float> want_q(rows * out_w), want_k, want_v(rows * out_w),
+                want_next(rows * out_w);
+            const nf4o_scales scales_q = weights[0].view();
+            nf4o_lora_linear_forward(
+                x.data(), weights[0].codes.data(), &scales_q,
+                bias_values.data(), a_values.data(), b_values.data(), rank,
+                scale, want_q.data(), rows, in_w, out_w, 64);
+            want_k = oracle_forward(x, weights[1]);
+            const nf4o_scales scales_v = weights[2].view();
+            nf4o_lora_linear_forward(
+                x.data(), weights[2].codes.data(), &scales_v, nullptr,
+                a_values.data(), b_values.data(), rank, scale, want_v.data(),
+                rows, in_w, out_w, 64);
+            const nf4o_scales scales_next = weights[3].view();
+            nf4o_lora_linear_forward(
+                want_q.data(), weights[3].codes.data(), &scales_next, nullptr,
+                a_values.data(), b_values.data(), rank, scale,
+                want_next.data(), rows, in_w, out_w, 64);
+            require_close(std::as_const(*outputs[0]).data(), want_q,
+                          "merged adapter forward, first member");
+            require_close(std::as_const(*outputs[1]).data(), want_k,
+                          "merged adapter forward, plain member");
+            require_close(std::as_const(*outputs[2]).data(), want_v,
+                          "merged adapter forward, third member");
+            require_close(std::as_const(*outputs[3]).data(), want_next,
+                          "a layer that reads a held-back output");
+            // x.A^T is the saved activation of the backward
+            std::vector<float> want_product(rows * rank);
+            nf4o_matmul_nt(x.data(), a_values.data(), want_product.data(),
+                           rows, in_w, rank);
+            require_close(std::as_const(*products[2]).data(), want_product,
+                          "the reduced buffer of a merged member");
+            if (merging) {
+                require(after_calls.requests - before.requests == 4 &&
+                            after_calls.launches - before.launches == 1,
+                        "three forwards on one input are held back until the "
+                        "dependent one arrives: one launch so far");
+                const auto after = detail::hip_forward_merge_statistics();
+                require(after.launches - before.launches == 2,
+                        "reading the outputs launches the dependent one");
+            }
+        }
+    }
+}
+
 void test_merged_forwards() {
     // The decoder's pattern, unchanged callers: three projections of one
     // input and then one of another, each through the dispatcher.  Results are
@@ -1197,6 +1298,7 @@ int main(int argc, char** argv) {
         test_forward_group();
         test_adapter_layer();
         test_merged_forwards();
+        test_merged_adapter_forwards();
         test_tensor_storage();
         test_dispatch_validation();
         test_packed_model_state();

@@ -361,6 +361,37 @@ rthip_status rthip_nf4_lora_linear_forward(
     return RTHIP_OK;
 }
 
+rthip_status rthip_nf4_lora_linear_forward_group(
+    const float* x, const rthip_nf4_lora_member* members,
+    uint64_t member_count, int32_t encoding, uint64_t second_level_block,
+    uint64_t rows, uint64_t input_width, uint64_t block_size, void* stream) {
+    if (members == nullptr || member_count == 0) {
+        return fail(RTHIP_INVALID_ARGUMENT, "a group needs members");
+    }
+    for (uint64_t m = 0; m < member_count; ++m) {
+        const rthip_nf4_lora_member& member = members[m];
+        const rthip_nf4_member& base = member.base;
+        const rthip_status status =
+            member.reduced == nullptr && member.lora_b == nullptr
+                ? rthip_nf4_linear_forward(
+                      x, base.codes, base.primary_scales,
+                      base.secondary_scales, encoding, second_level_block,
+                      base.offset, base.bias_or_null, base.y, rows,
+                      input_width, base.output_width, block_size, stream)
+                : rthip_nf4_lora_linear_forward(
+                      x, base.codes, base.primary_scales,
+                      base.secondary_scales, encoding, second_level_block,
+                      base.offset, base.bias_or_null, nullptr, member.lora_b,
+                      member.lora_rank, member.lora_scale,
+                      const_cast<float*>(member.reduced), base.y, rows,
+                      input_width, base.output_width, block_size, stream);
+        if (status != RTHIP_OK) {
+            return status;
+        }
+    }
+    return RTHIP_OK;
+}
+
 rthip_status rthip_nf4_lora_linear_forward_with(
     int32_t, const float* x, const uint8_t* codes, const void* primary_scales,
     const float* secondary_scales, int32_t encoding,
