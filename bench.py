@@ -742,8 +742,9 @@ def bench_decode_with_adapters(package, device, torch, layers, steps,
     unmerged low-rank adapters (QLoRA serving), M = 1, fp32 scales, three
     ways: one call per projection (q and v through
     rthip_nf4_lora_linear_forward: x.A^T and the packed product, two launches
-    each), the shared-input groups with one rthip_lora_reduce per adapter and
-    q/k/v through rthip_nf4_lora_linear_forward_group, and the same with ONE
+    each), the shared-input groups with q/k/v through
+    rthip_nf4_lora_linear_forward_group (which takes both x.A^T in one launch
+    of its own), and the same with the products taken beforehand by ONE
     rthip_lora_reduce over the stacked A of q and v (rows = 1: the members'
     reduced vectors lie side by side)."""
     library = package.load_library()
@@ -802,12 +803,10 @@ def bench_decode_with_adapters(package, device, torch, layers, steps,
                     entry_adapter = None
                     if name in entry[2]:
                         lora_a, lora_b, product = adapter(entry, name)
-                        if not stacked:
-                            library.lora_reduce(
-                                x[4096].data_ptr(), lora_a.data_ptr(),
-                                product.data_ptr(), 1, 4096, rank, stream)
-                        entry_adapter = (product.data_ptr(),
-                                         lora_b.data_ptr(), rank, scale)
+                        entry_adapter = (
+                            None if stacked else lora_a.data_ptr(),
+                            lora_b.data_ptr(), product.data_ptr(), rank,
+                            scale)
                     members.append((weights[name], None,
                                     outputs[name].data_ptr(), entry_adapter))
                 in_w = members[0][0].input_width

@@ -207,10 +207,12 @@ rthip_status rthip_nf4_linear_forward_group(
 /*
  * The same grouped forward for layers that carry low-rank adapters: member m
  * gets y_m = x.deq(W_m)^T + bias_m + lora_scale_m * (reduced_m . B_m^T), as
- * rthip_nf4_lora_linear_forward below computes it when its lora_a is NULL --
- * `reduced` [rows, lora_rank] already holds x.A_m^T (one rthip_lora_reduce over
- * the stacked A matrices of the members serves them all).  A member whose
- * lora_b and reduced are both NULL has no adapter.  The reference reaches this
+ * rthip_nf4_lora_linear_forward below computes it.  With lora_a given,
+ * `reduced` [rows, lora_rank] receives x.A_m^T first (the products of up to
+ * four members in one launch for up to 64 rows); with lora_a NULL it already
+ * holds it (one rthip_lora_reduce over the stacked A matrices of the members
+ * serves them all when rows is 1).  A member whose lora_b and reduced are both
+ * NULL has no adapter.  The reference reaches this
  * through Linear::forward (src/nn/linear.cpp:147-172) once per projection;
  * q, k and v of a layer with adapters on q and v are one launch here.
  * Every member's output equals its own rthip_nf4_lora_linear_forward (or
@@ -220,8 +222,9 @@ rthip_status rthip_nf4_linear_forward_group(
  */
 typedef struct rthip_nf4_lora_member {
     rthip_nf4_member base;
-    const float* reduced;  /* [rows, lora_rank], read only; NULL: no adapter */
+    const float* lora_a;   /* [lora_rank, input_width]; NULL: `reduced` is given */
     const float* lora_b;   /* [output_width, lora_rank] */
+    float* reduced;        /* [rows, lora_rank]; NULL (with lora_b): no adapter */
     uint64_t lora_rank;
     float lora_scale;
 } rthip_nf4_lora_member;

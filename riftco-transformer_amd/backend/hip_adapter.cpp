@@ -338,13 +338,7 @@ public:
         return pending;
     }
 
-    // `before_joining` runs once the list is known to take the member (what
-    // does not fit has been launched) and before the member joins it: the
-    // place for a launch that the member's own launch depends on and that
-    // must not overtake the one that produces its input.
-    template <typename BeforeJoining>
-    void add(const Shape& shape, const rthip_nf4_lora_member& member,
-             BeforeJoining&& before_joining) {
+    void add(const Shape& shape, const rthip_nf4_lora_member& member) {
         const std::lock_guard<std::mutex> lock(mutex_);
         ++statistics_.requests;
         bool fits = count_ != 0 && count_ < kCapacity && shape == shape_;
@@ -354,7 +348,6 @@ public:
         if (!fits) {
             launch_locked();
         }
-        before_joining();
         shape_ = shape;
         members_[count_++] = member;
         if (count_ == kCapacity) {
@@ -364,7 +357,7 @@ public:
     void add(const Shape& shape, const rthip_nf4_member& member) {
         rthip_nf4_lora_member plain{};
         plain.base = member;
-        add(shape, plain, [] {});
+        add(shape, plain);
     }
 
     void launch() {
@@ -1132,8 +1125,9 @@ void hip_quantized_linear_adapter_forward(
     if (merge_requested() && d.rows <= PendingForwards::kMaximumRows) {
         // The layer joins the forwards that are held back for its input (the
         // query and value projections of a decoder carry adapters, the key
-        // projection between them does not): x.A^T goes out now, the packed
-        // product with bias and adapter term with the rest of the list.
+        // projection between them does not): the launch of the list takes
+        // the members' x.A^T together, then the packed products with bias
+        // and adapter terms.
         const float* source = input.device_for_read();
         rthip_nf4_lora_member member{};
         member.base.codes = static_cast<const std::uint8_t*>(
@@ -1145,23 +1139,16 @@ void hip_quantized_linear_adapter_forward(
         member.base.bias_or_null = bias;
         member.base.y = output.device_for_overwrite();
         member.base.output_width = d.output_width;
-        float* const product = reduced.device_for_overwrite();
-        member.reduced = product;
+        member.lora_a = lora_a.device_for_read();
         member.lora_b = lora_b.device_for_read();
+        member.reduced = reduced.device_for_overwrite();
         member.lora_rank = request.rank;
         member.lora_scale = request.scale;
-        const float* const factor = lora_a.device_for_read();
         PendingForwards::instance().add(
             {source, static_cast<std::int32_t>(weight.encoding()),
              weight.second_level_block_size(), d.rows, d.input_width,
              d.block_size},
-            member, [&] {
-                check(runtime,
-                      runtime.lora_reduce(source, factor, product, d.rows,
-                                          d.input_width, request.rank,
-                                          nullptr),
-                      operation);
-            });
+            member);
         return;
     }
     launch_pending_forwards();

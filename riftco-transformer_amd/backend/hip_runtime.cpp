@@ -91,7 +91,6 @@ void load(HipRuntime& runtime) {
               runtime.nf4_lora_linear_forward, reason) ||
         !bind(library, "rthip_nf4_lora_linear_forward_group",
               runtime.nf4_lora_linear_forward_group, reason) ||
-        !bind(library, "rthip_lora_reduce", runtime.lora_reduce, reason) ||
         !bind(library, "rthip_lora_backward", runtime.lora_backward,
               reason) ||
         !bind(library, "rthip_nf4_lora_linear_input_backward",

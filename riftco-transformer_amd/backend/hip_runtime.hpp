@@ -45,7 +45,6 @@ struct HipRuntime {
         nullptr;
     decltype(&rthip_nf4_lora_linear_forward_group)
         nf4_lora_linear_forward_group = nullptr;
-    decltype(&rthip_lora_reduce) lora_reduce = nullptr;
     decltype(&rthip_lora_backward) lora_backward = nullptr;
     decltype(&rthip_nf4_lora_linear_input_backward)
         nf4_lora_linear_input_backward = nullptr;

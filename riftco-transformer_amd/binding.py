@@ -95,8 +95,8 @@ class Member(ctypes.Structure):
 class LoraMember(ctypes.Structure):
     """rthip_nf4_lora_member: a member with an optional adapter term."""
 
-    _fields_ = [("base", Member), ("reduced", _ptr), ("lora_b", _ptr),
-                ("lora_rank", _u64), ("lora_scale", _f32)]
+    _fields_ = [("base", Member), ("lora_a", _ptr), ("lora_b", _ptr),
+                ("reduced", _ptr), ("lora_rank", _u64), ("lora_scale", _f32)]
 
 
 _PROTOTYPES = {
@@ -341,8 +341,8 @@ class Library:
     def lora_linear_forward_group(self, x_ptr: int, members, rows: int,
                                   stream: int = 0) -> None:
         """members: (weight, bias_ptr or None, y_ptr, adapter) where adapter is
-        None or (reduced_ptr, lora_b_ptr, rank, scale); `reduced` already
-        holds x.A^T."""
+        None or (lora_a_ptr or None, lora_b_ptr, reduced_ptr, rank, scale);
+        with lora_a None, `reduced` already holds x.A^T."""
         first = members[0][0]
         array = (LoraMember * len(members))()
         for slot, (weight, bias_ptr, y_ptr, adapter) in zip(array, members):
@@ -362,7 +362,7 @@ class Library:
             slot.base.y = y_ptr
             slot.base.output_width = weight.output_width
             if adapter is not None:
-                (slot.reduced, slot.lora_b, slot.lora_rank,
+                (slot.lora_a, slot.lora_b, slot.reduced, slot.lora_rank,
                  slot.lora_scale) = adapter
         self._check(self._lib.rthip_nf4_lora_linear_forward_group(
             x_ptr, array, len(members), first.encoding,

@@ -166,6 +166,18 @@ hipError_t launch_lora_backward(const LoraBackwardProblem& problem,
 void launch_lora_reduce(const float* x, const float* a, float* reduced,
                         std::size_t rows, std::size_t input_width,
                         std::size_t rank, hipStream_t stream);
+// The same for several adapters on one x: one launch per four of them for up
+// to 64 rows, else one launch each; every product equals launch_lora_reduce's
+// bit for bit.
+constexpr std::size_t kLoraReduceGroupMax = 4;
+struct LoraReduceItem {
+    const float* a;   // [rank, input_width]
+    float* reduced;   // [rows, rank]
+    std::size_t rank;
+};
+void launch_lora_reduce_group(const float* x, const LoraReduceItem* items,
+                              std::size_t count, std::size_t rows,
+                              std::size_t input_width, hipStream_t stream);
 
 // dense_matmul.hip -- out[b] = left[b] [rows, shared] * right[b] [shared,
 // columns], plain fp32.

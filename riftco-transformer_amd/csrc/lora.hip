@@ -153,13 +153,12 @@ __global__ __launch_bounds__(kThreads) void lora_reduce_kernel(
 // DPP-free shuffles inside each wavefront and then in wavefront order.
 constexpr int kDotThreads = 256;
 
-__global__ __launch_bounds__(kDotThreads) void lora_reduce_rows_kernel(
+__device__ __forceinline__ void reduce_one_output(
     const float* __restrict__ x, const float* __restrict__ a,
-    float* __restrict__ reduced, unsigned input_width, unsigned rank
+    float* __restrict__ reduced, unsigned input_width, unsigned rank,
+    unsigned j, unsigned m
 ) {
     __shared__ float wave_sums[kDotThreads / 64];
-    const unsigned j = blockIdx.x;
-    const unsigned m = blockIdx.y;
     const float4* x_row = reinterpret_cast<const float4*>(
         x + static_cast<std::size_t>(m) * input_width);
     const float4* a_row = reinterpret_cast<const float4*>(
@@ -202,6 +201,45 @@ __global__ __launch_bounds__(kDotThreads) void lora_reduce_rows_kernel(
         }
         reduced[static_cast<std::size_t>(m) * rank + j] = total;
     }
+}
+
+__global__ __launch_bounds__(kDotThreads) void lora_reduce_rows_kernel(
+    const float* __restrict__ x, const float* __restrict__ a,
+    float* __restrict__ reduced, unsigned input_width, unsigned rank
+) {
+    reduce_one_output(x, a, reduced, input_width, rank, blockIdx.x,
+                      blockIdx.y);
+}
+
+// The same for up to four adapters on one x in one launch (the query and
+// value projections of a decoder block): blockIdx.z is the adapter.
+struct ReduceItems {
+    const float* a[kLoraReduceGroupMax];
+    float* reduced[kLoraReduceGroupMax];
+    unsigned rank[kLoraReduceGroupMax];
+};
+
+__global__ __launch_bounds__(kDotThreads) void lora_reduce_rows_group_kernel(
+    const float* __restrict__ x, const ReduceItems items, unsigned input_width
+) {
+    const unsigned item = blockIdx.z;
+    const unsigned rank = items.rank[item];
+    if (blockIdx.x >= rank) {  // uniform
+        return;
+    }
+    // (selects over kernel arguments: indexing them by a register would put
+    // the array into scratch memory)
+    const float* a = items.a[0];
+    float* reduced = items.reduced[0];
+#pragma unroll
+    for (unsigned k = 1; k < kLoraReduceGroupMax; ++k) {
+        if (item == k) {
+            a = items.a[k];
+            reduced = items.reduced[k];
+        }
+    }
+    reduce_one_output(x, a, reduced, input_width, rank, blockIdx.x,
+                      blockIdx.y);
 }
 
 // Any shape and alignment: one wavefront per output.
@@ -281,6 +319,48 @@ void launch_lora_reduce(const float* x, const float* a, float* reduced,
     } else {
         lora_reduce_kernel<4><<<dim3(row_tiles, chunks), kThreads, 0, stream>>>(
             x, a, reduced, r, i, k, rows_per_group);
+    }
+}
+
+
+void launch_lora_reduce_group(const float* x, const LoraReduceItem* items,
+                              std::size_t count, std::size_t rows,
+                              std::size_t input_width, hipStream_t stream) {
+    std::size_t next = 0;
+    while (next < count) {
+        const std::size_t run =
+            count - next < kLoraReduceGroupMax ? count - next
+                                               : kLoraReduceGroupMax;
+        bool together = run > 1 && rows <= 64 && input_width % 4 == 0 &&
+                        rows * input_width * sizeof(float) < kRejectedOffset &&
+                        reinterpret_cast<std::uintptr_t>(x) % 16 == 0;
+        unsigned widest = 0;
+        ReduceItems group{};
+        for (std::size_t k = 0; k < run; ++k) {
+            const LoraReduceItem& item = items[next + k];
+            together = together && item.rank <= 65535 &&
+                       item.rank * input_width * sizeof(float) <
+                           kRejectedOffset &&
+                       reinterpret_cast<std::uintptr_t>(item.a) % 16 == 0;
+            group.a[k] = item.a;
+            group.reduced[k] = item.reduced;
+            group.rank[k] = static_cast<unsigned>(item.rank);
+            widest = widest < group.rank[k] ? group.rank[k] : widest;
+        }
+        if (together) {
+            lora_reduce_rows_group_kernel<<<
+                dim3(widest, static_cast<unsigned>(rows),
+                     static_cast<unsigned>(run)),
+                kDotThreads, 0, stream>>>(x, group,
+                                          static_cast<unsigned>(input_width));
+        } else {
+            for (std::size_t k = 0; k < run; ++k) {
+                const LoraReduceItem& item = items[next + k];
+                launch_lora_reduce(x, item.a, item.reduced, rows, input_width,
+                                   item.rank, stream);
+            }
+        }
+        next += run;
     }
 }
 

@@ -1067,6 +1067,28 @@ static rthip_status forward_group(
         return status;
     }
     const hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+    // x.A^T of the members that bring their A along: together where the
+    // kernel takes several adapters, before any of the main launches
+    {
+        rthip::LoraReduceItem items[kMaxGroupMembers];
+        std::size_t count = 0;
+        for (uint64_t m = 0; m < member_count; ++m) {
+            const LoraArguments& lora = members[m].lora;
+            if (lora.reduced != nullptr && lora.a != nullptr) {
+                items[count++] =
+                    rthip::LoraReduceItem{lora.a, lora.reduced, lora.rank};
+            }
+        }
+        if (count != 0) {
+            rthip::launch_lora_reduce_group(x, items, count, rows,
+                                            input_width, hip_stream);
+            if (const rthip_status status =
+                    finish_launch("LoRA reduce launch");
+                status != RTHIP_OK) {
+                return status;
+            }
+        }
+    }
     const auto with_adapter = [&](uint64_t first, uint64_t length) {
         for (uint64_t m = first; m < first + length; ++m) {
             if (problems[m].lora.reduced != nullptr) {
@@ -1150,8 +1172,12 @@ static rthip_status forward_group(
                 RTHIP_NF4_ALGORITHM_AUTO, x, member.codes,
                 member.primary_scales, member.secondary_scales, encoding,
                 second_level_block, member.offset, member.bias_or_null,
-                members[next].lora, member.y, rows, input_width,
-                member.output_width, block_size, stream);
+                LoraArguments{nullptr, members[next].lora.b,
+                              members[next].lora.rank,
+                              members[next].lora.scale,
+                              members[next].lora.reduced},
+                member.y, rows, input_width, member.output_width, block_size,
+                stream);
             status != RTHIP_OK) {
             return status;
         }
@@ -1195,10 +1221,9 @@ rthip_status rthip_nf4_lora_linear_forward_group(
         group[m].base = member.base;
         group[m].lora = LoraArguments{nullptr, nullptr, 0, 0.0F, nullptr};
         if (member.lora_b != nullptr || member.reduced != nullptr) {
-            // (the reduced buffer is only read here)
             group[m].lora = LoraArguments{
-                nullptr, member.lora_b, member.lora_rank, member.lora_scale,
-                const_cast<float*>(member.reduced)};
+                member.lora_a, member.lora_b, member.lora_rank,
+                member.lora_scale, member.reduced};
             if (member.reduced == nullptr) {
                 return fail(RTHIP_INVALID_ARGUMENT,
                             "the adapter's B matrix and the reduced buffer "

@@ -108,11 +108,12 @@ def linear_forward_group(x: torch.Tensor, weights, biases=None):
 
 
 def lora_linear_forward_group(x: torch.Tensor, weights, adapters,
-                              biases=None):
+                              biases=None, reduce_first=False):
     """Like linear_forward_group for layers with low-rank adapters:
-    adapters[m] is None or (lora_a, lora_b, lora_scale).  x . A_m^T is taken
-    first (rthip_lora_reduce per adapter), then ONE call of
-    rthip_nf4_lora_linear_forward_group.  Returns (outputs, reduced) where
+    adapters[m] is None or (lora_a, lora_b, lora_scale); ONE call of
+    rthip_nf4_lora_linear_forward_group, which takes x . A_m^T itself
+    (reduce_first: rthip_lora_reduce per adapter beforehand, and members that
+    say their product is already there).  Returns (outputs, reduced) where
     reduced[m] is x . A_m^T or None."""
     assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous()
     library = load_library()
@@ -134,11 +135,13 @@ def lora_linear_forward_group(x: torch.Tensor, weights, adapters,
             assert tuple(lora_b.shape) == (weight.output_width, rank)
             product = torch.empty((rows, rank), dtype=torch.float32,
                                   device=x.device)
-            library.lora_reduce(x.data_ptr(), lora_a.data_ptr(),
-                                product.data_ptr(), rows, weight.input_width,
-                                rank, _stream())
+            if reduce_first:
+                library.lora_reduce(x.data_ptr(), lora_a.data_ptr(),
+                                    product.data_ptr(), rows,
+                                    weight.input_width, rank, _stream())
             reduced.append(product)
-            entry = (product.data_ptr(), lora_b.data_ptr(), rank, lora_scale)
+            entry = (None if reduce_first else lora_a.data_ptr(),
+                     lora_b.data_ptr(), product.data_ptr(), rank, lora_scale)
         members.append((weight, None if bias is None else bias.data_ptr(),
                         out.data_ptr(), entry))
     library.lora_linear_forward_group(x.data_ptr(), members, rows, _stream())

@@ -381,10 +381,10 @@ rthip_status rthip_nf4_lora_linear_forward_group(
                 : rthip_nf4_lora_linear_forward(
                       x, base.codes, base.primary_scales,
                       base.secondary_scales, encoding, second_level_block,
-                      base.offset, base.bias_or_null, nullptr, member.lora_b,
-                      member.lora_rank, member.lora_scale,
-                      const_cast<float*>(member.reduced), base.y, rows,
-                      input_width, base.output_width, block_size, stream);
+                      base.offset, base.bias_or_null, member.lora_a,
+                      member.lora_b, member.lora_rank, member.lora_scale,
+                      member.reduced, base.y, rows, input_width,
+                      base.output_width, block_size, stream);
         if (status != RTHIP_OK) {
             return status;
         }

@@ -186,7 +186,8 @@ def test_adapter_epilogue_of_the_decode_kernel(gpu, package, library, oracle,
 def test_groups_with_adapters_equal_their_members_launched_alone(
         gpu, package, library, oracle, double_quantized, rows):
     """rthip_nf4_lora_linear_forward_group: members with and without a
-    low-rank adapter term (ranks 16, 4 and 33), with and without bias, one
+    low-rank adapter term (ranks 16, 4 and 33; x.A^T taken by the call, several
+    adapters in one launch, or beforehand), with and without bias, one
     that the one-row kernel does not take (output width 100), at row counts
     of the decode kernel (<= 4), of the kernel that keeps x in registers
     (<= 128) and beyond (one launch per member).  Every output equals the
@@ -212,10 +213,13 @@ def test_groups_with_adapters_equal_their_members_launched_alone(
                          0.25 * (m + 1)))
     biases = [None, to_device(helpers.normal(95, (widths[1],), 0.01)),
               to_device(helpers.normal(96, (widths[2],), 0.01)), None]
-    for members in ([0, 1, 2], [0, 2], [1, 0, 3, 2], [3, 0]):
+    for members, reduce_first in (([0, 1, 2], False), ([0, 2], True),
+                                  ([1, 0, 3, 2], False), ([3, 0], True),
+                                  ([0, 2, 3], False)):
         together, reduced = gpu.lora_linear_forward_group(
             x, [device_weights[m] for m in members],
-            [adapters[m] for m in members], [biases[m] for m in members])
+            [adapters[m] for m in members], [biases[m] for m in members],
+            reduce_first=reduce_first)
         torch.cuda.synchronize()
         for m, got, product in zip(members, together, reduced):
             if adapters[m] is None:
@@ -265,11 +269,12 @@ def test_grouped_adapter_arguments_are_checked(gpu, package, library, oracle):
     with pytest.raises(package.RthipError, match="reduced buffer"):
         raw.lora_linear_forward_group(
             x.data_ptr(), [(weight, None, y.data_ptr(),
-                            (None, b.data_ptr(), 4, 1.0))], 1)
+                            (None, b.data_ptr(), None, 4, 1.0))], 1)
     with pytest.raises(package.RthipError, match="rank"):
         raw.lora_linear_forward_group(
             x.data_ptr(), [(weight, None, y.data_ptr(),
-                            (reduced.data_ptr(), b.data_ptr(), 0, 1.0))], 1)
+                            (None, b.data_ptr(), reduced.data_ptr(), 0,
+                             1.0))], 1)
     with pytest.raises(package.RthipError, match="same output"):
         raw.lora_linear_forward_group(
             x.data_ptr(), [(weight, None, y.data_ptr(), None),
@@ -277,5 +282,5 @@ def test_grouped_adapter_arguments_are_checked(gpu, package, library, oracle):
     # and a well-formed single member runs
     raw.lora_linear_forward_group(
         x.data_ptr(), [(weight, None, z.data_ptr(),
-                        (reduced.data_ptr(), b.data_ptr(), 4, 1.0))], 1)
+                        (None, b.data_ptr(), reduced.data_ptr(), 4, 1.0))], 1)
     torch.cuda.synchronize()
