@@ -142,3 +142,56 @@ def test_random_shapes_through_the_automatic_selection(gpu, package, library,
         del deq, exact, y, dx, with_adapter, term, weight
     # a sweep that no longer reaches the kernel families tests nothing
     assert {"gemv", "mfma", "skinny"} <= families, families
+
+
+@pytest.mark.parametrize("seed", [5, 6])
+def test_random_groups_with_adapters_equal_single_calls(gpu, package, library,
+                                                        seed):
+    """rthip_nf4_lora_linear_forward_group on random groups: two to five
+    members of one x, each with or without bias and with or without an
+    adapter of rank 1...33 (its x.A^T taken by the call or beforehand), row
+    widths and row counts on both sides of what the decode kernel and the
+    kernel that keeps x in registers take.  Every output, and every x.A^T,
+    equals the member's own call bit for bit."""
+    import torch
+    rng = random.Random(seed)
+    generator = torch.Generator(device="cuda")
+    generator.manual_seed(seed)
+    normal = lambda *shape: torch.randn(*shape, device="cuda",  # noqa: E731
+                                        generator=generator)
+    for case in range(40):
+        in_w = rng.choice([256, 1024, 2048, 4096, 5120, 11008, 12352])
+        rows = rng.choice([1, 2, 3, 4, 5, 16, 33, 64, 128, 129])
+        double_quantized = rng.random() < 0.5
+        widths = [rng.choice([64, 72, 100, 512, 1000, 1024, 4096])
+                  for _ in range(rng.choice([2, 3, 4, 5]))]
+        weights = [synthetic_weight(package, torch, width, in_w, 64,
+                                    double_quantized, 256,
+                                    1000 * seed + 10 * case + m)
+                   for m, width in enumerate(widths)]
+        x = normal(rows, in_w)
+        adapters, biases = [], []
+        for width in widths:
+            adapters.append(None)
+            if rng.random() < 0.6:
+                rank = rng.choice([1, 4, 8, 16, 33])
+                adapters[-1] = (normal(rank, in_w) * 0.05,
+                                normal(width, rank) * 0.05,
+                                rng.choice([0.5, 2.0]))
+            biases.append(normal(width) * 0.01 if rng.random() < 0.5
+                          else None)
+        outputs, products = gpu.lora_linear_forward_group(
+            x, weights, adapters, biases, reduce_first=rng.random() < 0.3)
+        torch.cuda.synchronize()
+        label = (f"seed {seed} case {case}: I={in_w} rows={rows} "
+                 f"widths={widths}")
+        for m, weight in enumerate(weights):
+            if adapters[m] is None:
+                want = gpu.linear_forward(x, weight, biases[m])
+            else:
+                lora_a, lora_b, scale = adapters[m]
+                want, own = gpu.lora_linear_forward(x, weight, lora_a, lora_b,
+                                                    scale, bias=biases[m])
+                assert torch.equal(own, products[m]), \
+                    f"{label}: x.A^T of member {m}"
+            assert torch.equal(want, outputs[m]), f"{label}: member {m}"
