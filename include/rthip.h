@@ -209,7 +209,7 @@ rthip_status rthip_nf4_linear_forward_group(
  * gets y_m = x.deq(W_m)^T + bias_m + lora_scale_m * (reduced_m . B_m^T), as
  * rthip_nf4_lora_linear_forward below computes it.  With lora_a given,
  * `reduced` [rows, lora_rank] receives x.A_m^T first (the products of up to
- * four members in one launch for up to 64 rows); with lora_a NULL it already
+ * four members in one launch while they are small); with lora_a NULL it already
  * holds it (one rthip_lora_reduce over the stacked A matrices of the members
  * serves them all when rows is 1).  A member whose lora_b and reduced are both
  * NULL has no adapter.  The reference reaches this

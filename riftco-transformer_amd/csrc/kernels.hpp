@@ -166,8 +166,9 @@ hipError_t launch_lora_backward(const LoraBackwardProblem& problem,
 void launch_lora_reduce(const float* x, const float* a, float* reduced,
                         std::size_t rows, std::size_t input_width,
                         std::size_t rank, hipStream_t stream);
-// The same for several adapters on one x: one launch per four of them for up
-// to 64 rows, else one launch each; every product equals launch_lora_reduce's
+// The same for several adapters on one x: one launch per four of them while
+// the products are few (the one-workgroup-per-output kernel), else one launch
+// each; every product equals launch_lora_reduce's
 // bit for bit.
 constexpr std::size_t kLoraReduceGroupMax = 4;
 struct LoraReduceItem {

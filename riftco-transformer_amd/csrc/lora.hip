@@ -4,8 +4,9 @@
 // [rank, input_width]; the result is tiny ([rows, rank]) and is consumed by
 // the epilogue of the packed-weight kernels (lora_epilogue.hpp).
 //
-// Up to 64 rows: one workgroup per output element (lora_reduce_rows_kernel).
-// Beyond that x is read exactly once: a workgroup of sixteen wavefronts owns
+// Few outputs (up to 64 rows, or up to about 6000 outputs per sixteen adapter
+// rows): one workgroup per output element (lora_reduce_rows_kernel).  Beyond
+// that x is read exactly once: a workgroup of sixteen wavefronts owns
 // 16 rows of x and up to 64 adapter rows; the contraction axis is cut into
 // sixteen spans,
 // one per wavefront, which each run v_mfma_f32_16x16x4_f32 over their span
@@ -271,6 +272,15 @@ __global__ __launch_bounds__(256) void lora_reduce_generic_kernel(
 
 }  // namespace
 
+// One workgroup per output element pays while there are few outputs: about
+// 3 us plus 1.25 us per thousand outputs of 4096 values, against 12 us and
+// more per sixteen adapter rows for the kernel above (measured: rank 16 up to
+// 384 rows, rank 64 likewise, rank 4 far beyond).
+static bool reduce_by_outputs(std::size_t rows, std::size_t rank) {
+    return rows <= 65535 && rank <= 65535 &&
+           (rows <= 64 || rows * rank <= 6144 * ((rank + 15) / 16));
+}
+
 void launch_lora_reduce(const float* x, const float* a, float* reduced,
                         std::size_t rows, std::size_t input_width,
                         std::size_t rank, hipStream_t stream) {
@@ -288,7 +298,7 @@ void launch_lora_reduce(const float* x, const float* a, float* reduced,
             x, a, reduced, rows, input_width, rank);
         return;
     }
-    if (rows <= 64 && rank <= 65535) {
+    if (reduce_by_outputs(rows, rank)) {
         lora_reduce_rows_kernel<<<dim3(static_cast<unsigned>(rank),
                                        static_cast<unsigned>(rows)),
                                   kDotThreads, 0, stream>>>(
@@ -331,14 +341,14 @@ void launch_lora_reduce_group(const float* x, const LoraReduceItem* items,
         const std::size_t run =
             count - next < kLoraReduceGroupMax ? count - next
                                                : kLoraReduceGroupMax;
-        bool together = run > 1 && rows <= 64 && input_width % 4 == 0 &&
+        bool together = run > 1 && input_width % 4 == 0 &&
                         rows * input_width * sizeof(float) < kRejectedOffset &&
                         reinterpret_cast<std::uintptr_t>(x) % 16 == 0;
         unsigned widest = 0;
         ReduceItems group{};
         for (std::size_t k = 0; k < run; ++k) {
             const LoraReduceItem& item = items[next + k];
-            together = together && item.rank <= 65535 &&
+            together = together && reduce_by_outputs(rows, item.rank) &&
                        item.rank * input_width * sizeof(float) <
                            kRejectedOffset &&
                        reinterpret_cast<std::uintptr_t>(item.a) % 16 == 0;
