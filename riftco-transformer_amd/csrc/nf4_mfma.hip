@@ -36,7 +36,11 @@
 // many workgroups as there are places, a workgroup whose run covers a whole
 // tile writes it as usual, the others write partial tiles to the stream's
 // workspace and a second kernel adds the parts of each tile in ascending
-// workgroup order (plus bias and adapter term).  Nothing depends on timing.
+// workgroup order (plus bias).  Nothing depends on timing.
+//
+// A low-rank adapter's term, s * (x A^T) . B^T, is not an epilogue: after a
+// tile's last step its rows of x A^T and its columns of B pass through the
+// same LDS tiles and the same matrix instructions, 32 of the rank at a time.
 //
 // The two directions share everything except the weight-tile loader: forward
 // reads 128 weight rows x 32 contiguous columns, backward reads 32 weight rows
@@ -172,8 +176,8 @@ __device__ __forceinline__ void store_weight_tile(
 
 // One segment: contraction values [k_begin, k_end) of the output tile at
 // (row0, col0).  `partial` null: the segment is the whole contraction and the
-// tile goes to `result` with bias and adapter term; otherwise the tile's
-// partial sums go to `partial`.
+// tile goes to `result` with bias; otherwise the tile's partial sums go to
+// `partial`.  The segment that starts at 0 includes the adapter term.
 template <bool kTall, bool kDoubleQuantized, bool kBackward>
 __device__ __forceinline__ void gemm_segment(
     const float* __restrict__ activations, const Nf4WeightView& weight,
