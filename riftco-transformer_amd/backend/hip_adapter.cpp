@@ -343,7 +343,9 @@ public:
         ++statistics_.requests;
         bool fits = count_ != 0 && count_ < kCapacity && shape == shape_;
         for (std::size_t m = 0; fits && m < count_; ++m) {
-            fits = members_[m].base.y != member.base.y;
+            fits = members_[m].base.y != member.base.y &&
+                   (member.reduced == nullptr ||
+                    members_[m].reduced != member.reduced);
         }
         if (!fits) {
             launch_locked();

@@ -1030,6 +1030,12 @@ static rthip_status forward_group(
                 return fail(RTHIP_INVALID_ARGUMENT,
                             "two members of a group write the same output");
             }
+            if (lora.reduced != nullptr && lora.a != nullptr &&
+                members[other].lora.reduced == lora.reduced) {
+                return fail(RTHIP_INVALID_ARGUMENT,
+                            "two members of a group write the same reduced "
+                            "buffer");
+            }
         }
         if (const rthip_status status = check_dimensions(
                 rows, input_width, member.output_width, block_size,

@@ -279,6 +279,14 @@ def test_grouped_adapter_arguments_are_checked(gpu, package, library, oracle):
         raw.lora_linear_forward_group(
             x.data_ptr(), [(weight, None, y.data_ptr(), None),
                            (weight, None, y.data_ptr(), None)], 1)
+    a = torch.zeros(4, 256, device="cuda")
+    with pytest.raises(package.RthipError, match="same reduced"):
+        raw.lora_linear_forward_group(
+            x.data_ptr(),
+            [(weight, None, y.data_ptr(),
+              (a.data_ptr(), b.data_ptr(), reduced.data_ptr(), 4, 1.0)),
+             (weight, None, z.data_ptr(),
+              (a.data_ptr(), b.data_ptr(), reduced.data_ptr(), 4, 1.0))], 1)
     # and a well-formed single member runs
     raw.lora_linear_forward_group(
         x.data_ptr(), [(weight, None, z.data_ptr(),
