@@ -222,6 +222,57 @@ int main(int argc, char** argv) {
                             static_cast<unsigned long long>(merged.launches));
             }
         }
+        // The same block with unmerged rank-16 adapters on the query and value
+        // projections (what Linear::forward of such a layer calls on hip).
+        namespace detail = riftco_transformer::backend_detail;
+        constexpr std::size_t rank = 16;
+        std::vector<float> a_values(rank * width), b_values(width * rank);
+        for (auto& value : a_values) {
+            value = static_cast<float>(random() % 2001) / 20000.0F - 0.05F;
+        }
+        for (auto& value : b_values) {
+            value = static_cast<float>(random() % 2001) / 20000.0F - 0.05F;
+        }
+        const auto lora_a = backend::make_tensor_storage(kHip, a_values);
+        const auto lora_b = backend::make_tensor_storage(kHip, b_values);
+        for (int phase = 0; phase < 2; ++phase) {  // 0: warm-up
+            const int repeats = phase == 0 ? 20 : calls;
+            const auto before = backend::hip_forward_merge_statistics();
+            const auto begin = std::chrono::steady_clock::now();
+            std::unique_ptr<backend::TensorStorage> outputs[3];
+            std::unique_ptr<backend::TensorStorage> products[3];
+            for (int call = 0; call < repeats; ++call) {
+                for (int m = 0; m < 3; ++m) {
+                    outputs[m] = backend::make_tensor_storage(kHip, width, 0.0F);
+                    products[m] = backend::make_tensor_storage(kHip, rank, 0.0F);
+                }
+                for (int m = 0; m < 3; ++m) {
+                    if (m == 1) {
+                        backend::dispatch_quantized_linear_forward(
+                            kHip,
+                            {*input, *weights[m], *outputs[m], dimensions});
+                    } else {
+                        detail::hip_quantized_linear_adapter_forward(
+                            {*input, *weights[m], nullptr, *lora_a, *lora_b,
+                             rank, 2.0F, *products[m], *outputs[m],
+                             dimensions});
+                    }
+                }
+            }
+            checksum += std::as_const(*outputs[2]).data()[0];
+            if (phase == 1) {
+                const auto merged = backend::hip_forward_merge_statistics();
+                std::printf("q/k/v, adapters on q,v %8.2f us per projection "
+                            "(%d steps, checksum %.6g; %llu requests in %llu "
+                            "launches)\n",
+                            seconds_since(begin) / (3.0 * repeats) * 1e6,
+                            repeats, checksum,
+                            static_cast<unsigned long long>(
+                                merged.requests - before.requests),
+                            static_cast<unsigned long long>(
+                                merged.launches - before.launches));
+            }
+        }
     }
     return 0;
 }
