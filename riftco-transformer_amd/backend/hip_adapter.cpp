@@ -425,16 +425,16 @@ void launch_pending_forwards_or_abort() noexcept {
 
 class HipTensorStorage final : public TensorStorage {
 public:
+    // A tensor of one value.  The value is written where it is first needed:
+    // the outputs the reference allocates before every operation
+    // (src/nn/quantized_linear.cpp:41) are overwritten by the kernel that
+    // follows and never filled.
     HipTensorStorage(std::size_t element_count, float fill_value)
         : count_(element_count),
           device_(checked_bytes(element_count), DeviceBuffer::Kind::Pooled),
-          freshest_(Freshest::Device) {
-        const HipRuntime& runtime = require_runtime();
-        check(runtime,
-              runtime.fill_f32(static_cast<float*>(device_.get()), fill_value,
-                               count_, nullptr),
-              "tensor fill");
-        finish_operation(runtime, "tensor fill synchronisation");
+          fill_value_(fill_value),
+          freshest_(Freshest::Neither) {
+        static_cast<void>(require_runtime());
     }
 
     explicit HipTensorStorage(std::vector<float> values)
@@ -487,6 +487,15 @@ public:
     // HBM pointer with the tensor's current contents.
     [[nodiscard]] const float* device_for_read() const {
         const std::lock_guard<std::mutex> lock(sync_);
+        if (freshest_ == Freshest::Neither) {
+            const HipRuntime& runtime = require_runtime();
+            check(runtime,
+                  runtime.fill_f32(static_cast<float*>(device_.get()),
+                                   fill_value_, count_, nullptr),
+                  "tensor fill");
+            freshest_ = Freshest::Device;
+            finish_operation(runtime, "tensor fill synchronisation");
+        }
         if (freshest_ == Freshest::Host) {
             const HipRuntime& runtime = require_runtime();
             check(runtime,
@@ -506,7 +515,8 @@ public:
     }
 
 private:
-    enum class Freshest { Host, Device, Both };
+    // Neither: no copy has been written yet, every element is fill_value_.
+    enum class Freshest { Host, Device, Both, Neither };
 
     static std::size_t checked_bytes(std::size_t element_count) {
         if (element_count >
@@ -522,6 +532,11 @@ private:
     // (sync_ held; queued forwards have been launched by the caller, outside
     // the lock: launching them reads and writes other tensors' state)
     void refresh_host_locked() const noexcept {
+        if (freshest_ == Freshest::Neither) {
+            host_.assign(count_, fill_value_);
+            freshest_ = Freshest::Host;  // HBM gets it when a kernel reads it
+            return;
+        }
         if (freshest_ != Freshest::Device) {
             return;
         }
@@ -537,6 +552,7 @@ private:
 
     std::size_t count_;
     DeviceBuffer device_;
+    float fill_value_ = 0.0F;
     mutable std::mutex sync_;  // guards host_ and freshest_
     mutable std::vector<float> host_;
     mutable Freshest freshest_;

@@ -622,6 +622,45 @@ void test_adapter_layer() {
     }
 }
 
+void test_one_value_tensors() {
+    // make_tensor_storage(count, value) writes the value where it is first
+    // needed: read by host code, read by a kernel (as the input of a
+    // forward), cloned, or never (an output that a kernel overwrites).
+    const std::size_t in_w = 256, out_w = 64;
+    const HostWeight weight = quantize(
+        pseudo_normal(out_w * in_w, 0.02F, 301), out_w, in_w, 64, false, 256);
+    const auto storage = to_hip(weight);
+    {
+        auto tensor = backend::make_tensor_storage(kHip, 5, 3.5F);
+        const auto values = std::as_const(*tensor).data();
+        require(values.size() == 5 && values[0] == 3.5F && values[4] == 3.5F,
+                "a one-value tensor read by host code");
+        tensor->data()[2] = 1.0F;  // host write, then a device read
+        auto copy = tensor->clone();
+        require(std::as_const(*copy).data()[2] == 1.0F &&
+                    std::as_const(*copy).data()[3] == 3.5F,
+                "a clone of a one-value tensor that host code changed");
+    }
+    {
+        auto input = backend::make_tensor_storage(kHip, in_w, 0.25F);
+        auto output = backend::make_tensor_storage(kHip, out_w, 9.0F);
+        backend::dispatch_quantized_linear_forward(
+            kHip, {*input, *storage, *output, {1, in_w, out_w, 64}});
+        require_close(std::as_const(*output).data(),
+                      oracle_forward(std::vector<float>(in_w, 0.25F), weight),
+                      "a one-value tensor read by a kernel first");
+        // the input still reads as its value on the host
+        require(std::as_const(*input).data()[in_w - 1] == 0.25F,
+                "a one-value tensor read by a kernel, then by host code");
+    }
+    {
+        auto untouched = backend::make_tensor_storage(kHip, 3, -2.0F);
+        auto copy = untouched->clone();
+        require(std::as_const(*copy).data()[1] == -2.0F,
+                "a clone of a one-value tensor nobody has read");
+    }
+}
+
 void test_merged_adapter_forwards() {
     // A decoder whose query and value projections carry adapters: q (adapter,
     // bias), k (plain, through the dispatcher), v (adapter) on one input, then
@@ -1297,6 +1336,7 @@ int main(int argc, char** argv) {
         test_transformer_sized_layer();
         test_forward_group();
         test_adapter_layer();
+        test_one_value_tensors();
         test_merged_forwards();
         test_merged_adapter_forwards();
         test_tensor_storage();
