@@ -521,10 +521,10 @@ constexpr std::size_t kWorkspaceBytes =
     sizeof(float);
 static_assert(kWorkspaceBytes <= kStreamWorkspaceBytes);
 
-// Slabs a workgroup may chain in ONE accumulator (2048 contraction values:
-// rounding stays near 4e-6 of an output's scale; runs of 13.5 slabs measured
-// 7.6e-6).
-constexpr unsigned kSingleChainSlabs = 8;
+// Slabs a workgroup may chain in ONE accumulator (1536 contraction values:
+// rounding stays below 5e-6 of an output's scale; runs of 8 slabs measured
+// 6.0e-6 on 5000 x 12352, runs of 13.5 slabs 7.6e-6).
+constexpr unsigned kSingleChainSlabs = 6;
 
 // The split of (tile, slab) units over the workgroups.
 struct LaunchSplit {
