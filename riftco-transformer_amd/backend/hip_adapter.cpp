@@ -437,12 +437,16 @@ public:
         static_cast<void>(require_runtime());
     }
 
+    // A tensor of host values (the result of an operation that ran on the
+    // host, an input a caller built): they go to HBM when a kernel first
+    // reads the tensor -- never, if only host code does.
     explicit HipTensorStorage(std::vector<float> values)
         : count_(values.size()),
-          device_(values.data(), checked_bytes(values.size()),
-                  DeviceBuffer::Kind::Pooled),
+          device_(checked_bytes(values.size()), DeviceBuffer::Kind::Pooled),
           host_(std::move(values)),
-          freshest_(Freshest::Both) {}
+          freshest_(Freshest::Host) {
+        static_cast<void>(require_runtime());
+    }
 
     [[nodiscard]] ExecutionBackend backend() const noexcept override {
         return kHipBackend;
